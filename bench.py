@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q8_0 decode hot path on one MI355X.
+
+Workload ("llama3_8b_q8_0_decode_projection_set"): one step is one decode
+token's worth of Q8_0 projections of Llama-3-8B at batch 1 — 32 layers x
+{q, k, v, o, gate, up, down} plus lm_head, 225 matvecs over 7.97 GB of
+distinct weights (so every launch streams from HBM, not from cache), f32
+activations ~N(0,1), random weights: quants U{-127..127}, block scales
+|N(0,0.02)|/127 in f16.  Inputs are resident in HBM before timing starts.
+
+Prints ONE JSON line: whole-step GB/s of algorithmic bytes
+(N*K*34/32 + 4K + 4N per matvec), per-shape GB/s, the roofline fraction of the
+matvec kernel against 8 TB/s, and the CPU baseline (the oracle's restatement of
+the reference's dequantise-then-f32-matmul path) timed on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    return ap.parse_args()
+
+
+def make_weight(torch, lib, capi, n, k, gen, dev):
+    """Random Q8_0 weight built on the device as raw GGUF blocks, then repacked
+    by the library (the same path a loader takes)."""
+    nb = n * k // 32
+    qs = torch.randint(-127, 128, (nb, 32), dtype=torch.int8, device=dev, generator=gen)
+    d = (torch.randn((nb, 1), device=dev, generator=gen).abs() * (0.02 / 127.0)).to(torch.float16)
+    raw = torch.empty((nb, 34), dtype=torch.uint8, device=dev)
+    raw[:, :2] = d.view(torch.uint8)
+    raw[:, 2:] = qs.view(torch.uint8)
+    planar = torch.empty(lib.lhip_q8_0_planar_nbytes(n, k), dtype=torch.uint8, device=dev)
+    capi.check(lib.lhip_q8_0_repack(raw.data_ptr(), planar.data_ptr(), n, k,
+                                    torch.cuda.current_stream().cuda_stream), "lhip_q8_0_repack")
+    torch.cuda.synchronize()
+    return planar
+
+
+def cpu_baseline(seconds: float):
+    """Dequantise once (untimed, as the reference's loader does), then time the
+    f32 matvecs of ONE layer's seven projections, single-threaded like the
+    reference's matrixmultiply configuration, for about `seconds`."""
+    import numpy as np
+
+    from luminal_amd import synth
+    from oracle import cpu_oracle
+
+    names = ["q", "k", "v", "o", "gate", "up", "down"]
+    ws, xs, outs, q8_bytes = [], [], [], 0
+    for i, nm in enumerate(names):
+        n, k = synth.LLAMA3_8B_PROJ[nm]
+        qs, d = synth.q8_0_random(n, k, seed=900 + i)
+        w = cpu_oracle.q8_0_dequant(synth.q8_0_raw_blocks(qs, d), n * k).reshape(n, k)
+        ws.append(w)
+        xs.append(synth.activations(1, k, seed=950 + i))
+        outs.append(np.empty((1, n), np.float32))
+        q8_bytes += synth.q8_0_gemv_bytes(n, k)
+
+    def one_pass(threads):
+        for w, x, o in zip(ws, xs, outs):
+            cpu_oracle.matmul_fast_f32(x, w, threads=threads, out=o)
+
+    def timed(threads, budget):
+        one_pass(threads)  # warm
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            one_pass(threads)
+            reps += 1
+            if time.perf_counter() - t0 >= budget:
+                break
+        return (time.perf_counter() - t0) / reps, reps
+
+    t1, reps1 = timed(1, seconds * 0.7)
+    ncpu = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    tn, repsn = timed(ncpu, seconds * 0.3)
+    return {
+        "value": round(q8_bytes / t1 / 1e9, 3),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": (f"one layer's 7 projections (q,k,v,o,gate,up,down; {q8_bytes} Q8_0-equivalent bytes, "
+                   f"f32 weights after load-time dequant), {reps1} passes, {t1 * 1e3:.1f} ms/pass single-threaded"),
+        "all_cores": {"value": round(q8_bytes / tn / 1e9, 3), "cores": ncpu, "passes": repsn,
+                      "ms_per_pass": round(tn * 1e3, 2)},
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU's share of the path (no collectives, no sharding); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from luminal_amd import capi, synth
+
+    lib = capi.load_library()  # no fallback: raises if the HIP library is missing
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    capi.check(lib.lhip_init(0), "lhip_init")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0x5EED)
+
+    layers = args.layers or synth.LLAMA3_8B_LAYERS
+    layer_names = ["q", "k", "v", "o", "gate", "up", "down"]
+    shapes = synth.LLAMA3_8B_PROJ
+
+    weights = {nm: [] for nm in layer_names}
+    for _ in range(layers):
+        for nm in layer_names:
+            n, k = shapes[nm]
+            weights[nm].append(make_weight(torch, lib, capi, n, k, gen, dev))
+    weights["lm_head"] = [make_weight(torch, lib, capi, *shapes["lm_head"], gen, dev)]
+
+    x = {4096: torch.randn(4096, device=dev, generator=gen), 14336: torch.randn(14336, device=dev, generator=gen)}
+    y = {nm: torch.empty(shapes[nm][0], device=dev) for nm in shapes}
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def gemv(nm, wbuf):
+        n, k = shapes[nm]
+        st = lib.lhip_q8_0_matmul_f32(wbuf.data_ptr(), x[k].data_ptr(), y[nm].data_ptr(), 1, n, k, stream)
+        if st:
+            capi.check(st, "lhip_q8_0_matmul_f32")
+
+    def step():
+        for l in range(layers):
+            for nm in layer_names:
+                gemv(nm, weights[nm][l])
+        gemv("lm_head", weights["lm_head"][0])
+
+    launches = layers * len(layer_names) + 1
+    step_bytes = layers * sum(synth.q8_0_gemv_bytes(*shapes[nm]) for nm in layer_names) \
+        + synth.q8_0_gemv_bytes(*shapes["lm_head"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = ev0.elapsed_time(ev1)
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes / (wall / args.steps) / 1e9
+
+    # Per-shape rates: back-to-back launches rotating over that shape's distinct
+    # weight buffers (lm_head alone is 558 MB, larger than the 256 MB last-level
+    # cache), HIP events on the launch stream.
+    per_shape = {}
+    for nm in list(layer_names) + ["lm_head"]:
+        bufs = weights[nm]
+        reps = 20 if nm == "lm_head" else max(1, 128 // len(bufs))
+        for b in bufs[:2]:
+            gemv(nm, b)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for b in bufs:
+                gemv(nm, b)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * len(bufs))
+        nbytes = synth.q8_0_gemv_bytes(*shapes[nm])
+        per_shape[nm] = {"n": shapes[nm][0], "k": shapes[nm][1], "us": round(us, 2),
+                         "gbs": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    achieved = step_bytes / (gpu_ms / args.steps) / 1e6  # GB/s from HIP events over the timed region
+    roofline = {
+        "bound": "hbm",
+        "kernel": "q8_gemv_f32_kernel (all launch shapes of the step)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "launches_per_step": launches,
+        "bytes_per_launch": round(step_bytes / launches),
+        "avg_launch_us": round(gpu_ms * 1e3 / (args.steps * launches), 3),
+    }
+
+    out = {
+        "metric": "Q8_0 GEMV HBM GB/s (% of peak) + Llama-3-8B Q8_0 decode tok/s, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 weights x f32 activations, f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "llama3_8b_q8_0_decode_projection_set" + ("" if layers == 32 else f"_DEBUG_{layers}_layers"),
+            "batch": 1,
+            "launches_per_step": launches,
+            "bytes_per_step": step_bytes,
+            "projection_tokens_per_s": round(args.steps / wall, 1),
+        },
+        "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "per_shape": per_shape,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        del weights
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

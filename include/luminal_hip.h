@@ -1,0 +1,122 @@
+/*
+ * luminal_hip — C ABI of the MI355X (gfx950) quantized-matmul backend.
+ *
+ * This is the surface a `luminal_hip` Rust crate binds with `extern "C"`:
+ * plain pointers and sizes, no C++ or framework types.  Every device pointer
+ * is an ordinary HIP allocation (hipMalloc, or lhip_malloc below); `stream`
+ * is a hipStream_t passed as void* (NULL = the default stream).  All launches
+ * are asynchronous on `stream`; nothing here synchronises except
+ * lhip_stream_sync and the two blocking copies.  The caller owns every buffer
+ * and the library never frees or keeps one.
+ *
+ * Where the reference panics (unwrap/assert!/panic!), these functions return
+ * a status instead; a Rust wrapper turns non-zero into panic! to keep the
+ * reference's behaviour.
+ *
+ * Reference files cited below are relative to the luminal source tree.
+ */
+#ifndef LUMINAL_HIP_H
+#define LUMINAL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t lhip_status;
+enum {
+    LHIP_OK = 0,
+    LHIP_ERR_NULL_PTR = 1,      /* a required pointer argument is NULL */
+    LHIP_ERR_INVALID_SHAPE = 2, /* zero dim, K % 32 != 0, dim too large ... */
+    LHIP_ERR_MISALIGNED = 3,    /* a device pointer misses its required alignment */
+    LHIP_ERR_HIP = 4,           /* a HIP runtime call failed: see lhip_last_hip_error */
+    LHIP_ERR_UNSUPPORTED = 5    /* valid arguments, but no kernel for this case */
+};
+
+/* Human-readable name of a status code (static storage). */
+const char *lhip_status_string(lhip_status s);
+/* hipError_t of the most recent LHIP_ERR_HIP on this thread (0 if none). */
+int lhip_last_hip_error(void);
+/* Library version, "major.minor.patch". */
+const char *lhip_version(void);
+
+/* ---- device plumbing ------------------------------------------------------
+ * Counterparts of what luminal_cuda takes from cudarc: CudaContext::new(0)
+ * (crates/luminal_cuda/src/quantized.rs:247), stream.alloc / memcpy_stod /
+ * memcpy_dtov (quantized.rs:144, examples/llama/src/loader.rs:157,
+ * crates/luminal_cuda/src/prim.rs:60-75). */
+lhip_status lhip_init(int device);
+lhip_status lhip_malloc(void **dptr, size_t nbytes);
+lhip_status lhip_free(void *dptr);
+lhip_status lhip_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, void *stream);
+lhip_status lhip_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, void *stream);
+lhip_status lhip_stream_sync(void *stream);
+
+/* ---- Q8_0 weight storage ---------------------------------------------------
+ * A weight (N, K) arrives as raw GGUF Q8_0 blocks: N*K/32 blocks of 34 bytes
+ * {f16 d; int8 qs[32]}, row-major, N*K + N*K/16 bytes — exactly the bytes the
+ * reference's loader copies to the device
+ * (examples/llama/src/loader.rs:124-130,156-158; block struct
+ * crates/luminal_cuda/src/quantized.rs:30-33).
+ *
+ * The kernels read a "planar" re-arrangement of the same bytes made once at
+ * load: all quants first (int8[N][K], so every 16-byte load is aligned), then
+ * all scales (f16[N][K/32]).  Same byte count apart from padding the quant
+ * plane to 256 B.  K % 32 == 0 is required (as in the reference, which
+ * computes K/32 blocks per row, quantized.rs:58). */
+
+/* Bytes of the raw GGUF form: N*K + N*K/16. */
+size_t lhip_q8_0_raw_nbytes(int64_t n, int64_t k);
+/* Bytes of the planar form (what to allocate for `planar`). */
+size_t lhip_q8_0_planar_nbytes(int64_t n, int64_t k);
+/* Byte offset of the scale plane inside the planar buffer. */
+size_t lhip_q8_0_planar_scale_offset(int64_t n, int64_t k);
+/* raw (device) -> planar (device).  `planar` must be 256-byte aligned, `raw`
+ * 2-byte aligned.  The buffers must not overlap. */
+lhip_status lhip_q8_0_repack(const void *raw_dev, void *planar_dev, int64_t n, int64_t k, void *stream);
+/* planar (device) -> raw (device): inverse of lhip_q8_0_repack. */
+lhip_status lhip_q8_0_unpack(const void *planar_dev, void *raw_dev, int64_t n, int64_t k, void *stream);
+
+/* ---- Q8_0 operators --------------------------------------------------------
+ */
+
+/* Dequantise a planar weight to f32[N][K]: w = (float)q * (float)d, exact.
+ * Restates the reference's CPU loader (examples/llama/src/loader.rs:227-241). */
+lhip_status lhip_q8_0_dequant_f32(const void *planar_dev, float *out_dev, int64_t n, int64_t k, void *stream);
+
+/* y[m][n] = sum_k x[m][k] * W[n][k], f32 activations, f32 accumulate, f32 out.
+ * Replaces QuantizedMatmul<f32>::process + its matvec kernel
+ * (crates/luminal_cuda/src/quantized.rs:42-109,116-168): x is (m, K) row-major
+ * with m = batch*m of the reference's launch (grid z, quantized.rs:159), y is
+ * (m, N).  x and y must be 16-byte aligned. */
+lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
+                                 int64_t k, void *stream);
+
+/* Same operator with the launch shape given by the caller instead of chosen by
+ * the library (for tuning and for tests that cover every shape):
+ * rows_per_wave in {1,2,4,8}, k_unroll in {1,2,4}; LHIP_ERR_UNSUPPORTED for a
+ * combination that is not built. */
+lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
+                                     int64_t k, int rows_per_wave, int k_unroll, void *stream);
+
+/* Row gather: out[t][j] = dequant(W[(int)idx[t]][j]), idx carried as f32 like
+ * the reference's (crates/luminal_cuda/src/quantized.rs:191-198,202-233), but
+ * read from device memory.  An index outside [0, n) yields a row of zeros. */
+lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
+                                 int64_t n, int64_t k, void *stream);
+
+/* ---- calibration kernels ---------------------------------------------------
+ * No counterpart in the reference.  A plain device-to-device copy and a
+ * read-only pass with known byte counts, used to calibrate hardware counters
+ * and to measure the HBM rate a streaming kernel can reach on this part.
+ * src/dst 16-byte aligned, nbytes a multiple of 16. */
+lhip_status lhip_copy_bytes(void *dst_dev, const void *src_dev, size_t nbytes, void *stream);
+/* Reads nbytes and writes one 32-bit XOR checksum to *out_dev (4-byte aligned). */
+lhip_status lhip_read_bytes(const void *src_dev, size_t nbytes, uint32_t *out_dev, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUMINAL_HIP_H */

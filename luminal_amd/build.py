@@ -1,0 +1,59 @@
+"""Build recipe of libluminal_hip.so (hipcc, gfx950 only).
+
+``python -m luminal_amd.build`` compiles every HIP source under ``csrc/`` into
+one shared library beside this file, plus a code object (``.hsaco``) holding
+the same kernels for callers that load them with hipModuleLoad.
+"""
+from __future__ import annotations
+
+import glob
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libluminal_hip.so")
+HSACO = os.path.join(HERE, "luminal_hip_gfx950.hsaco")
+
+ARCH = "gfx950"
+# Packed-FP32 instructions are switched off for all device code.
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", f"--offload-arch={ARCH}"]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
+
+
+def sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # The host pass does not know the device-only feature flag and says so: harmless.
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("build failed: " + " ".join(cmd) + "\n" + out)
+    if out.strip():
+        print(out, file=sys.stderr)
+
+
+def build(verbose: bool = True) -> str:
+    srcs = sources()
+    if not srcs:
+        raise RuntimeError(f"no HIP sources under {CSRC}")
+    cc = hipcc()
+    if verbose:
+        print(f"[luminal_amd.build] {cc} -> {LIB}", file=sys.stderr)
+    _run([cc, *COMMON, *DEVICE_FLAGS, "-shared", "-o", LIB, *srcs])
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

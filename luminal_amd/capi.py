@@ -1,0 +1,81 @@
+"""ctypes binding of the luminal_hip C ABI (include/luminal_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libluminal_hip.so")
+
+LHIP_OK = 0
+LHIP_ERR_NULL_PTR = 1
+LHIP_ERR_INVALID_SHAPE = 2
+LHIP_ERR_MISALIGNED = 3
+LHIP_ERR_HIP = 4
+LHIP_ERR_UNSUPPORTED = 5
+
+_vp, _i64, _sz, _int = C.c_void_p, C.c_int64, C.c_size_t, C.c_int
+
+# name -> (restype, argtypes); one entry per declaration in include/luminal_hip.h
+SIGNATURES = {
+    "lhip_status_string": (C.c_char_p, [C.c_int32]),
+    "lhip_last_hip_error": (_int, []),
+    "lhip_version": (C.c_char_p, []),
+    "lhip_init": (C.c_int32, [_int]),
+    "lhip_malloc": (C.c_int32, [C.POINTER(_vp), _sz]),
+    "lhip_free": (C.c_int32, [_vp]),
+    "lhip_memcpy_h2d": (C.c_int32, [_vp, _vp, _sz, _vp]),
+    "lhip_memcpy_d2h": (C.c_int32, [_vp, _vp, _sz, _vp]),
+    "lhip_stream_sync": (C.c_int32, [_vp]),
+    "lhip_q8_0_raw_nbytes": (_sz, [_i64, _i64]),
+    "lhip_q8_0_planar_nbytes": (_sz, [_i64, _i64]),
+    "lhip_q8_0_planar_scale_offset": (_sz, [_i64, _i64]),
+    "lhip_q8_0_repack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_q8_0_unpack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_q8_0_dequant_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
+    "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
+    "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),
+}
+
+
+class LhipError(RuntimeError):
+    def __init__(self, status: int, where: str, detail: str = ""):
+        self.status = status
+        super().__init__(f"{where}: {detail or status}")
+
+
+_lib = None
+
+
+def load_library(path: str | None = None) -> C.CDLL:
+    """Load libluminal_hip.so; there is no fallback if it has not been built."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise LhipError(-1, "load_library", f"{p} is missing: build it with `python -m luminal_amd.build`")
+    lib = C.CDLL(p)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def status_string(s: int) -> str:
+    return load_library().lhip_status_string(s).decode()
+
+
+def check(status: int, where: str) -> None:
+    if status != LHIP_OK:
+        lib = load_library()
+        detail = lib.lhip_status_string(status).decode()
+        if status == LHIP_ERR_HIP:
+            detail += f" (hipError_t {lib.lhip_last_hip_error()})"
+        raise LhipError(status, where, detail)

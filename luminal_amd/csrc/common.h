@@ -1,0 +1,48 @@
+// Shared internals of the luminal_hip library: status plumbing, argument
+// checks, and the planar Q8_0 layout arithmetic.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/luminal_hip.h"
+
+namespace lhip {
+
+// Records the failing hipError_t for lhip_last_hip_error().
+lhip_status hip_failed(hipError_t e);
+
+#define LHIP_HIP_TRY(expr)                                        \
+    do {                                                          \
+        hipError_t _e = (expr);                                   \
+        if (_e != hipSuccess) return ::lhip::hip_failed(_e);      \
+    } while (0)
+
+// Kernel launches report configuration errors through hipGetLastError.
+#define LHIP_CHECK_LAUNCH() LHIP_HIP_TRY(hipGetLastError())
+
+static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+static inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Largest dimension accepted: keeps every int32 index computed in the kernels
+// (rows, columns, blocks per row) in range.
+constexpr int64_t kMaxDim = (int64_t{1} << 30);
+
+static inline lhip_status check_q8_shape(int64_t n, int64_t k) {
+    if (n <= 0 || k <= 0 || n > kMaxDim || k > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (k % 32 != 0) return LHIP_ERR_INVALID_SHAPE;
+    return LHIP_OK;
+}
+
+// Planar Q8_0: [int8 qs[N][K]] padded to 256 B, then [f16 d[N][K/32]].
+static inline size_t q8_scale_offset(int64_t n, int64_t k) {
+    size_t q = static_cast<size_t>(n) * static_cast<size_t>(k);
+    return (q + 255) & ~size_t{255};
+}
+static inline size_t q8_planar_nbytes(int64_t n, int64_t k) {
+    return q8_scale_offset(n, k) + static_cast<size_t>(n) * static_cast<size_t>(k / 32) * 2;
+}
+
+}  // namespace lhip

@@ -1,0 +1,168 @@
+// Q8_0 storage kernels: raw GGUF blocks <-> planar, dequantise, row gather.
+//
+// Raw block (34 B): little-endian f16 scale, then 32 int8 quants
+// (crates/luminal_cuda/src/quantized.rs:30-33).  Raw rows are only 2-byte
+// aligned, so these kernels move 16-bit units: unit u of the raw stream lies
+// in block u/17; unit u%17 == 0 is the scale, the others are quant pairs.
+// All of this is HBM-bound byte shuffling with both sides fully coalesced.
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace lhip {
+
+constexpr int kThreads = 256;
+
+__global__ __launch_bounds__(kThreads) void q8_repack_kernel(const uint16_t *__restrict__ raw,
+                                                              uint16_t *__restrict__ qs,
+                                                              uint16_t *__restrict__ ds, size_t n_units) {
+    size_t u = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    for (; u < n_units; u += stride) {
+        const size_t blk = u / 17;
+        const unsigned off = static_cast<unsigned>(u - blk * 17);
+        const uint16_t v = raw[u];
+        if (off == 0)
+            ds[blk] = v;
+        else
+            qs[blk * 16 + (off - 1)] = v;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void q8_unpack_kernel(const uint16_t *__restrict__ qs,
+                                                              const uint16_t *__restrict__ ds,
+                                                              uint16_t *__restrict__ raw, size_t n_units) {
+    size_t u = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    for (; u < n_units; u += stride) {
+        const size_t blk = u / 17;
+        const unsigned off = static_cast<unsigned>(u - blk * 17);
+        raw[u] = (off == 0) ? ds[blk] : qs[blk * 16 + (off - 1)];
+    }
+}
+
+// One thread dequantises 4 consecutive quants: w = (float)q * (float)d.  The
+// product of an int8 and a binary16 value is exact in binary32.
+__device__ __forceinline__ float4 dequant4(uint32_t q4, float d) {
+    float4 o;
+    o.x = static_cast<float>(static_cast<int8_t>(q4 & 0xff)) * d;
+    o.y = static_cast<float>(static_cast<int8_t>((q4 >> 8) & 0xff)) * d;
+    o.z = static_cast<float>(static_cast<int8_t>((q4 >> 16) & 0xff)) * d;
+    o.w = static_cast<float>(static_cast<int8_t>(q4 >> 24)) * d;
+    return o;
+}
+
+__global__ __launch_bounds__(kThreads) void q8_dequant_kernel(const uint32_t *__restrict__ qs,
+                                                               const __half *__restrict__ ds,
+                                                               float4 *__restrict__ out, size_t n_quads) {
+    size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    for (; i < n_quads; i += stride) out[i] = dequant4(qs[i], __half2float(ds[i >> 3]));
+}
+
+// grid.x = index row, threads stride over the K/4 quads of that row.
+__global__ __launch_bounds__(kThreads) void q8_gather_kernel(const uint32_t *__restrict__ qs,
+                                                              const __half *__restrict__ ds,
+                                                              const float *__restrict__ idx,
+                                                              float4 *__restrict__ out, int n, int k) {
+    const int t = blockIdx.x;
+    const float fi = idx[t];
+    // `as usize` in the reference's CPU gather truncates toward zero.
+    const long row = (fi >= 0.0f && fi < 2147483648.0f) ? static_cast<long>(fi) : -1;
+    const int quads = k >> 2;
+    float4 *o = out + static_cast<size_t>(t) * quads;
+    if (row < 0 || row >= n) {
+        for (int j = threadIdx.x; j < quads; j += kThreads) o[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        return;
+    }
+    const uint32_t *q = qs + static_cast<size_t>(row) * quads;
+    const __half *d = ds + static_cast<size_t>(row) * (k >> 5);
+    for (int j = threadIdx.x; j < quads; j += kThreads) o[j] = dequant4(q[j], __half2float(d[j >> 3]));
+}
+
+static inline unsigned grid_for(size_t items) {
+    size_t g = (items + kThreads - 1) / kThreads;
+    // Grid-stride loops: cap the grid at a few waves per SIMD of the whole chip.
+    const size_t cap = 256u * 64u;
+    return static_cast<unsigned>(g < cap ? (g ? g : 1) : cap);
+}
+
+}  // namespace lhip
+
+using namespace lhip;
+
+extern "C" {
+
+size_t lhip_q8_0_raw_nbytes(int64_t n, int64_t k) {
+    if (check_q8_shape(n, k) != LHIP_OK) return 0;
+    size_t e = static_cast<size_t>(n) * static_cast<size_t>(k);
+    return e + e / 16;
+}
+
+size_t lhip_q8_0_planar_nbytes(int64_t n, int64_t k) {
+    if (check_q8_shape(n, k) != LHIP_OK) return 0;
+    return q8_planar_nbytes(n, k);
+}
+
+size_t lhip_q8_0_planar_scale_offset(int64_t n, int64_t k) {
+    if (check_q8_shape(n, k) != LHIP_OK) return 0;
+    return q8_scale_offset(n, k);
+}
+
+lhip_status lhip_q8_0_repack(const void *raw_dev, void *planar_dev, int64_t n, int64_t k, void *stream) {
+    if (!raw_dev || !planar_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (!aligned(raw_dev, 2) || !aligned(planar_dev, 256)) return LHIP_ERR_MISALIGNED;
+    const size_t n_units = static_cast<size_t>(n) * (k / 32) * 17;
+    auto *base = static_cast<uint8_t *>(planar_dev);
+    hipLaunchKernelGGL(q8_repack_kernel, dim3(grid_for(n_units)), dim3(kThreads), 0, as_stream(stream),
+                       static_cast<const uint16_t *>(raw_dev), reinterpret_cast<uint16_t *>(base),
+                       reinterpret_cast<uint16_t *>(base + q8_scale_offset(n, k)), n_units);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_q8_0_unpack(const void *planar_dev, void *raw_dev, int64_t n, int64_t k, void *stream) {
+    if (!raw_dev || !planar_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (!aligned(raw_dev, 2) || !aligned(planar_dev, 256)) return LHIP_ERR_MISALIGNED;
+    const size_t n_units = static_cast<size_t>(n) * (k / 32) * 17;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    hipLaunchKernelGGL(q8_unpack_kernel, dim3(grid_for(n_units)), dim3(kThreads), 0, as_stream(stream),
+                       reinterpret_cast<const uint16_t *>(base),
+                       reinterpret_cast<const uint16_t *>(base + q8_scale_offset(n, k)),
+                       static_cast<uint16_t *>(raw_dev), n_units);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_q8_0_dequant_f32(const void *planar_dev, float *out_dev, int64_t n, int64_t k, void *stream) {
+    if (!planar_dev || !out_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (!aligned(planar_dev, 256) || !aligned(out_dev, 16)) return LHIP_ERR_MISALIGNED;
+    const size_t n_quads = static_cast<size_t>(n) * static_cast<size_t>(k) / 4;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    hipLaunchKernelGGL(q8_dequant_kernel, dim3(grid_for(n_quads)), dim3(kThreads), 0, as_stream(stream),
+                       reinterpret_cast<const uint32_t *>(base),
+                       reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)),
+                       reinterpret_cast<float4 *>(out_dev), n_quads);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
+                                 int64_t n, int64_t k, void *stream) {
+    if (!planar_dev || !idx_dev || !out_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (n_idx <= 0 || n_idx > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(planar_dev, 256) || !aligned(out_dev, 16) || !aligned(idx_dev, 4)) return LHIP_ERR_MISALIGNED;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    hipLaunchKernelGGL(q8_gather_kernel, dim3(static_cast<unsigned>(n_idx)), dim3(kThreads), 0, as_stream(stream),
+                       reinterpret_cast<const uint32_t *>(base),
+                       reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), idx_dev,
+                       reinterpret_cast<float4 *>(out_dev), static_cast<int>(n), static_cast<int>(k));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+}  // extern "C"

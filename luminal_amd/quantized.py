@@ -1,0 +1,118 @@
+"""Host-side mirror of the reference's quantized operators over the C ABI.
+
+Names and argument meaning follow crates/luminal_cuda/src/quantized.rs:
+``QuantizedMatmul.process`` takes the activations first and the weight second
+and returns a freshly allocated output; ``QuantizedGather`` carries
+``embed_dim``.  torch is used for device memory and the current stream only:
+all arithmetic happens in libluminal_hip.so, and there is no fallback.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import capi
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor) -> int:
+    return t.data_ptr()
+
+
+class Q8Weight:
+    """A (N, K) Q8_0 weight resident on the device in planar form
+    (the role of ``CudaData<u8>`` in examples/llama/src/loader.rs:156-158)."""
+
+    def __init__(self, planar: torch.Tensor, n: int, k: int):
+        self.planar, self.n, self.k = planar, n, k
+
+    @staticmethod
+    def planar_nbytes(n: int, k: int) -> int:
+        nb = capi.load_library().lhip_q8_0_planar_nbytes(n, k)
+        if nb == 0:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "Q8Weight", f"invalid Q8_0 shape ({n}, {k})")
+        return nb
+
+    @classmethod
+    def from_raw(cls, raw, n: int, k: int, device="cuda:0") -> "Q8Weight":
+        """raw: GGUF Q8_0 block bytes (numpy uint8, or a uint8 torch tensor on host or device)."""
+        lib = capi.load_library()
+        if isinstance(raw, np.ndarray):
+            raw = torch.from_numpy(np.ascontiguousarray(raw, dtype=np.uint8))
+        raw = raw.reshape(-1)
+        expect = lib.lhip_q8_0_raw_nbytes(n, k)
+        if expect == 0 or raw.numel() != expect:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "Q8Weight.from_raw",
+                                 f"expected {expect} bytes for ({n}, {k}), got {raw.numel()}")
+        raw_dev = raw.to(device)
+        planar = torch.empty(cls.planar_nbytes(n, k), dtype=torch.uint8, device=device)
+        with torch.cuda.device(planar.device):
+            capi.check(lib.lhip_q8_0_repack(_ptr(raw_dev), _ptr(planar), n, k, _stream()), "lhip_q8_0_repack")
+            torch.cuda.current_stream().synchronize()  # raw_dev is released on return
+        return cls(planar, n, k)
+
+    def to_raw(self) -> torch.Tensor:
+        lib = capi.load_library()
+        raw = torch.empty(lib.lhip_q8_0_raw_nbytes(self.n, self.k), dtype=torch.uint8, device=self.planar.device)
+        with torch.cuda.device(raw.device):
+            capi.check(lib.lhip_q8_0_unpack(_ptr(self.planar), _ptr(raw), self.n, self.k, _stream()),
+                       "lhip_q8_0_unpack")
+        return raw
+
+    def dequantize(self) -> torch.Tensor:
+        lib = capi.load_library()
+        out = torch.empty((self.n, self.k), dtype=torch.float32, device=self.planar.device)
+        with torch.cuda.device(out.device):
+            capi.check(lib.lhip_q8_0_dequant_f32(_ptr(self.planar), _ptr(out), self.n, self.k, _stream()),
+                       "lhip_q8_0_dequant_f32")
+        return out
+
+
+class QuantizedMatmul:
+    """(.., M, K) x Q8_0 (N, K) -> (.., M, N), f32
+    (QuantizedMatmul<f32>::process, crates/luminal_cuda/src/quantized.rs:116-168)."""
+
+    def __init__(self, rows_per_wave: int | None = None, k_unroll: int | None = None):
+        self.cfg = (rows_per_wave, k_unroll) if rows_per_wave else None
+
+    def process(self, x: torch.Tensor, w: Q8Weight) -> torch.Tensor:
+        lib = capi.load_library()
+        if x.dtype != torch.float32 or not x.is_cuda:
+            raise TypeError("QuantizedMatmul expects f32 activations on the GPU")
+        if x.shape[-1] != w.k:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "QuantizedMatmul",
+                                 f"activation K {x.shape[-1]} != weight K {w.k}")
+        x = x.contiguous()
+        m = x.numel() // w.k
+        out = torch.empty(x.shape[:-1] + (w.n,), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            if self.cfg:
+                st = lib.lhip_q8_0_matmul_f32_cfg(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, self.cfg[0],
+                                                  self.cfg[1], _stream())
+            else:
+                st = lib.lhip_q8_0_matmul_f32(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, _stream())
+        capi.check(st, "lhip_q8_0_matmul_f32")
+        return out
+
+
+class QuantizedGather:
+    """Row gather from a Q8_0 table; indices are f32 as in the reference
+    (QuantizedGather<f32>::process, crates/luminal_cuda/src/quantized.rs:202-233)."""
+
+    def __init__(self, embed_dim: int):
+        self.embed_dim = embed_dim
+
+    def process(self, indexes: torch.Tensor, w: Q8Weight) -> torch.Tensor:
+        lib = capi.load_library()
+        if w.k != self.embed_dim:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "QuantizedGather",
+                                 f"embed_dim {self.embed_dim} != weight K {w.k}")
+        idx = indexes.to(device=w.planar.device, dtype=torch.float32).contiguous().reshape(-1)
+        out = torch.empty((idx.numel(), w.k), dtype=torch.float32, device=idx.device)
+        with torch.cuda.device(idx.device):
+            st = lib.lhip_q8_0_gather_f32(_ptr(w.planar), _ptr(idx), _ptr(out), idx.numel(), w.n, w.k, _stream())
+        capi.check(st, "lhip_q8_0_gather_f32")
+        return out

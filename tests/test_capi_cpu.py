@@ -1,0 +1,98 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every declared symbol, and its size arithmetic and argument validation (which
+run before any HIP call) behave as documented."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from luminal_amd import capi, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "luminal_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lhip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load_library()
+    names = declared_symbols()
+    assert len(names) >= 15
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in luminal_hip.h but not exported"
+    # and the binding covers every declaration
+    assert sorted(capi.SIGNATURES) == names
+
+
+def test_status_strings():
+    lib = capi.load_library()
+    assert lib.lhip_status_string(0) == b"LHIP_OK"
+    assert lib.lhip_status_string(2) == b"LHIP_ERR_INVALID_SHAPE"
+    assert lib.lhip_status_string(99) == b"LHIP_ERR_UNKNOWN"
+    assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.lhip_version())
+
+
+def test_size_laws():
+    lib = capi.load_library()
+    for name, (n, k) in synth.LLAMA3_8B_PROJ.items():
+        raw = lib.lhip_q8_0_raw_nbytes(n, k)
+        assert raw == n * k + n * k // 16, name  # examples/llama/src/loader.rs:128
+        assert lib.lhip_q8_0_planar_nbytes(n, k) == raw  # same bytes, re-arranged
+        assert lib.lhip_q8_0_planar_scale_offset(n, k) == n * k
+    # quant plane padded to 256 B
+    assert lib.lhip_q8_0_planar_scale_offset(3, 32) == 256
+    assert lib.lhip_q8_0_planar_nbytes(3, 32) == 256 + 6
+    # invalid shapes give 0
+    for n, k in [(0, 32), (4, 0), (4, 31), (4, 48), (-1, 32), (1 << 31, 32)]:
+        assert lib.lhip_q8_0_raw_nbytes(n, k) == 0
+        assert lib.lhip_q8_0_planar_nbytes(n, k) == 0
+
+
+def test_argument_validation_before_any_device_work():
+    lib = capi.load_library()
+    ok_ptr = 0x1000  # never dereferenced: validation fails first
+    assert lib.lhip_q8_0_matmul_f32(None, ok_ptr, ok_ptr, 1, 32, 32, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, None, ok_ptr, 1, 32, 32, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, ok_ptr, None, 1, 32, 32, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, ok_ptr, ok_ptr, 1, 32, 33, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, ok_ptr, ok_ptr, 0, 32, 32, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, ok_ptr, ok_ptr, 1, 0, 32, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr + 16, ok_ptr, ok_ptr, 1, 32, 32, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_matmul_f32(ok_ptr, ok_ptr + 4, ok_ptr, 1, 32, 32, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_repack(None, ok_ptr, 1, 32, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_repack(ok_ptr + 1, ok_ptr, 1, 32, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_repack(ok_ptr, ok_ptr + 128, 1, 32, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_unpack(ok_ptr, ok_ptr, 1, 40, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_dequant_f32(ok_ptr, None, 1, 32, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_gather_f32(ok_ptr, ok_ptr, ok_ptr, 0, 4, 32, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_gather_f32(ok_ptr, None, ok_ptr, 1, 4, 32, None) == capi.LHIP_ERR_NULL_PTR
+    out = C.c_void_p()
+    assert lib.lhip_malloc(None, 16) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_malloc(C.byref(out), 0) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_free(None) == capi.LHIP_OK
+    assert lib.lhip_memcpy_h2d(None, ok_ptr, 4, None) == capi.LHIP_ERR_NULL_PTR
+
+
+def test_check_raises_with_status_name():
+    with pytest.raises(capi.LhipError) as e:
+        capi.check(capi.LHIP_ERR_INVALID_SHAPE, "somewhere")
+    assert "LHIP_ERR_INVALID_SHAPE" in str(e.value) and e.value.status == 2
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(capi.LhipError):
+        capi.load_library(str(tmp_path / "nope.so"))
+
+
+def test_gemv_byte_model():
+    # figures the roofline fraction is computed from
+    assert synth.q8_0_gemv_bytes(4096, 4096) == 17858560
+    assert synth.q8_0_gemv_bytes(1024, 4096) == 4476928
+    assert synth.q8_0_gemv_bytes(14336, 4096) == 62464000
+    assert synth.q8_0_gemv_bytes(4096, 14336) == 62464000
+    assert synth.q8_0_gemv_bytes(128256, 4096) == 558699520
