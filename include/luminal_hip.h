@@ -95,11 +95,15 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
                                  int64_t k, void *stream);
 
 /* Same operator with the launch shape given by the caller instead of chosen by
- * the library (for tuning and for tests that cover every shape):
- * rows_per_wave in {1,2,4,8}, k_unroll in {1,2,4}; LHIP_ERR_UNSUPPORTED for a
- * combination that is not built. */
+ * the library (for tuning and for tests that cover every shape).
+ * blocks_per_cu in 1..16 runs the persistent pipelined kernel with that many
+ * resident workgroups per compute unit (rows_per_wave in {1,2,4}, k_unroll =
+ * 1024-quant slices per pipeline step in {1,2,4}, K <= 16384);
+ * blocks_per_cu == 0 runs the one-shot kernel (rows_per_wave in {1,2,4,8},
+ * k_unroll in {1,2,4}, any K).  LHIP_ERR_UNSUPPORTED for a combination that
+ * is not built. */
 lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
-                                     int64_t k, int rows_per_wave, int k_unroll, void *stream);
+                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu, void *stream);
 
 /* Row gather: out[t][j] = dequant(W[(int)idx[t]][j]), idx carried as f32 like
  * the reference's (crates/luminal_cuda/src/quantized.rs:191-198,202-233), but
@@ -113,7 +117,8 @@ lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, f
  * and to measure the HBM rate a streaming kernel can reach on this part.
  * src/dst 16-byte aligned, nbytes a multiple of 16. */
 lhip_status lhip_copy_bytes(void *dst_dev, const void *src_dev, size_t nbytes, void *stream);
-/* Reads nbytes and writes one 32-bit XOR checksum to *out_dev (4-byte aligned). */
+/* Reads nbytes; each wavefront leaves the XOR of what it read in one of the
+ * 1024 words of out_dev (4096 bytes, 4-byte aligned). */
 lhip_status lhip_read_bytes(const void *src_dev, size_t nbytes, uint32_t *out_dev, void *stream);
 
 #ifdef __cplusplus

@@ -6,6 +6,7 @@
 namespace lhip {
 
 typedef uint32_t cu32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned kReadSlots = 1024;  // out_dev of lhip_read_bytes holds this many words
 
 __global__ __launch_bounds__(256) void copy_kernel(cu32x4 *__restrict__ dst, const cu32x4 *__restrict__ src,
                                                    size_t n16) {
@@ -28,8 +29,11 @@ __global__ __launch_bounds__(256) void read_kernel(const cu32x4 *__restrict__ sr
         a ^= v0 ^ v1 ^ v2 ^ v3;
     }
     for (; i < n16; i += stride) a ^= __builtin_nontemporal_load(src + i);
-    const uint32_t x = a.x ^ a.y ^ a.z ^ a.w;
-    if (x != 0) atomicXor(out, x);
+    uint32_t x = a.x ^ a.y ^ a.z ^ a.w;
+    for (int o = 32; o > 0; o >>= 1) x ^= __shfl_xor(x, o);
+    // one plain store per wavefront into a slot of its own (no atomics: they
+    // would serialise on one address and dominate the timing)
+    if ((threadIdx.x & 63) == 0) out[(blockIdx.x * 4 + (threadIdx.x >> 6)) & (kReadSlots - 1)] = x;
 }
 
 }  // namespace lhip

@@ -141,9 +141,166 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__res
     if (lane < R && row0 + lane < n) y[row0 + lane] = out;
 }
 
+// ---------------------------------------------------------------------------
+// Persistent, software-pipelined variant (the one the library normally runs).
+// Requires K to be a multiple of S*1024 and at most 16384.
+//
+// A grid of G workgroups of 4 wavefronts stays resident; wave w walks the row
+// groups w, w + 4G, ...  The activation vector is staged once per workgroup
+// into LDS, so the only HBM traffic in the loop is the weight stream.  Work is
+// cut into steps of R rows x S slices of 1024 quants; the loads of step t+1
+// are issued before the arithmetic of step t starts (two register buffers,
+// scheduling fenced), so each wave always has R*S 16-byte loads per lane in
+// flight.
+//
+// LDS layout of the activations: float4 index  slice*256 + j*64 + lane  holds
+// x[slice*1024 + lane*16 + j*4 .. +3], so the four 16-byte reads a lane makes
+// per slice are contiguous across lanes (no bank conflicts).
+// ---------------------------------------------------------------------------
+
+template <int R, int S>
+struct StepBuf {
+    u32x4 q[S][R];
+    unsigned d[S][R];  // f16 scale code, zero-extended
+};
+
+// Row bases are wave-uniform (scalar registers); the per-lane part of every
+// address is one 32-bit byte offset plus a compile-time slice offset.
+template <int R, int S>
+__device__ __forceinline__ void load_step(StepBuf<R, S> &b, const int8_t *__restrict__ qs,
+                                          const unsigned short *__restrict__ ds, int row0, int n, int k, int slice0,
+                                          unsigned lane, bool live) {
+    // `live` is wave-uniform.  A dead step (one past the wave's last) still
+    // issues its loads, so the count of outstanding loads is the same on every
+    // trip through the pipeline, but aims them all at the first bytes of the
+    // planes: one cached line instead of a stream from HBM.
+    const int nblk = k >> 5;
+    const unsigned kbase = live ? static_cast<unsigned>(slice0) * 1024u : 0u;
+    const unsigned qoff = live ? lane * 16u : 0u;
+    const unsigned doff = live ? (lane >> 1) * 2u : 0u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = live ? min(row0 + r, n - 1) : 0;  // rows past the end re-read the last row
+        const char *qrow = reinterpret_cast<const char *>(qs) + static_cast<size_t>(row) * k + kbase;
+        const char *drow = reinterpret_cast<const char *>(ds) + (static_cast<size_t>(row) * nblk + (kbase >> 5)) * 2;
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            b.q[s][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow + (s * 1024u + qoff)));
+            b.d[s][r] = __builtin_nontemporal_load(reinterpret_cast<const unsigned short *>(drow + (s * 64u + doff)));
+        }
+    }
+}
+
+template <int R, int S>
+__device__ __forceinline__ void compute_step(StepBuf<R, S> &b, const float4 *xs4, int slice0, unsigned lane,
+                                             float (&acc)[R]) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const float4 *xp = xs4 + (slice0 + s) * 256 + lane;
+        float4 xv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[j] = xp[j * 64];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            // Opaque to the optimiser: keeps the int8->f32 conversions of this
+            // buffer here instead of next to its loads, where they would stall
+            // the wave on data it has only just requested.
+            asm volatile("" : "+v"(b.q[s][r]), "+v"(b.d[s][r]));
+            acc[r] = fmaf(dot16(b.q[s][r], xv),
+                          __half2float(__ushort_as_half(static_cast<unsigned short>(b.d[s][r]))), acc[r]);
+        }
+    }
+}
+
+template <int R, int S>
+__global__ __launch_bounds__(256) void q8_gemv_f32_pipe_kernel(const int8_t *__restrict__ qs,
+                                                                const unsigned short *__restrict__ ds,
+                                                                const float *__restrict__ x, float *__restrict__ y,
+                                                                int n, int k) {
+    extern __shared__ float4 xs4[];
+    const unsigned lane = threadIdx.x & 63u;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: stays in a scalar register
+    const int wave_global = blockIdx.x * 4 + wave;
+    const int total_waves = gridDim.x * 4;
+    x += static_cast<size_t>(blockIdx.y) * k;
+    y += static_cast<size_t>(blockIdx.y) * n;
+
+    const int n_groups = (n + R - 1) / R;
+    const int chunks = k / (S * 1024);  // steps per row group
+    const int my_groups = wave_global < n_groups ? (n_groups - wave_global + total_waves - 1) / total_waves : 0;
+    const int T = my_groups * chunks;
+
+    StepBuf<R, S> a, b;
+    // First weight loads go out before the activations are staged, so the
+    // HBM round trip overlaps the staging.
+    load_step(a, qs, ds, wave_global * R, n, k, 0, lane, T > 0);
+
+    {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
+        const int k4 = k >> 2;
+#pragma unroll 4
+        for (int i = threadIdx.x; i < k4; i += 256) {
+            // destination index i = slice*256 + j*64 + l  <-  source slice*256 + l*4 + j
+            const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
+            xs4[i] = x4[src];
+        }
+    }
+    __syncthreads();
+    if (T == 0) return;
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+    int t = 0;            // step being computed
+    int g = wave_global;  // its row group
+    int c = 0;            // its chunk within the row group
+
+    auto next = [&](int &gg, int &cc) {
+        if (++cc == chunks) {
+            cc = 0;
+            gg += total_waves;
+        }
+    };
+    auto finish_group = [&](int gg) {
+        float out = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float s = wave_sum(acc[r]);
+            if (lane == static_cast<unsigned>(r)) out = s;
+            acc[r] = 0.f;
+        }
+        const int row0 = gg * R;
+        if (lane < static_cast<unsigned>(R) && row0 + static_cast<int>(lane) < n) y[row0 + lane] = out;
+    };
+
+    while (true) {
+        int g1 = g, c1 = c;
+        next(g1, c1);
+        load_step(b, qs, ds, g1 * R, n, k, c1 * S, lane, t + 1 < T);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(a, xs4, c * S, lane, acc);
+        if (c == chunks - 1) finish_group(g);
+        if (++t >= T) break;
+        g = g1;
+        c = c1;
+        next(g1, c1);
+        load_step(a, qs, ds, g1 * R, n, k, c1 * S, lane, t + 1 < T);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(b, xs4, c * S, lane, acc);
+        if (c == chunks - 1) finish_group(g);
+        if (++t >= T) break;
+        g = g1;
+        c = c1;
+    }
+}
+
+constexpr int kNumCUs = 256;
+constexpr int kMaxLdsK = 16384;  // 64 KiB of staged activations
+
 template <int R, int W, int U>
-static lhip_status launch(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
-                          hipStream_t s) {
+static lhip_status launch_oneshot(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
+                                  hipStream_t s) {
     const unsigned tiles = static_cast<unsigned>((n + R * W - 1) / (R * W));
     hipLaunchKernelGGL((q8_gemv_f32_kernel<R, W, U>), dim3(tiles, static_cast<unsigned>(m)), dim3(W * 64), 0, s, qs,
                        ds, x, y, n, k);
@@ -151,29 +308,74 @@ static lhip_status launch(const int8_t *qs, const __half *ds, const float *x, fl
     return LHIP_OK;
 }
 
-// Launch-shape table.  rows_per_wave in {1,2,4,8}, k_unroll in {1,2,4}.
-static lhip_status dispatch(int rows_per_wave, int k_unroll, const int8_t *qs, const __half *ds, const float *x,
-                            float *y, int m, int n, int k, hipStream_t s) {
+template <int R, int S>
+static lhip_status launch_pipe(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
+                               int blocks_per_cu, hipStream_t s) {
+    if (k % (S * 1024) != 0 || k > kMaxLdsK) return LHIP_ERR_UNSUPPORTED;
+    const int n_groups = (n + R - 1) / R;
+    int grid = (n_groups + 3) / 4;
+    const int cap = kNumCUs * blocks_per_cu;
+    if (grid > cap) grid = cap;
+    hipLaunchKernelGGL((q8_gemv_f32_pipe_kernel<R, S>), dim3(static_cast<unsigned>(grid), static_cast<unsigned>(m)),
+                       dim3(256), static_cast<size_t>(k) * sizeof(float), s, qs,
+                       reinterpret_cast<const unsigned short *>(ds), x, y, n, k);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+// Launch-shape table.  blocks_per_cu == 0 selects the one-shot kernel
+// (rows_per_wave in {1,2,4,8}, k_unroll in {1,2,4}); otherwise the pipelined
+// kernel (rows_per_wave in {1,2,4}, k_unroll = slices per step in {1,2,4}).
+static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, const int8_t *qs, const __half *ds,
+                            const float *x, float *y, int m, int n, int k, hipStream_t s) {
+    if (blocks_per_cu < 0 || blocks_per_cu > 16) return LHIP_ERR_UNSUPPORTED;
+    if (blocks_per_cu == 0) {
 #define LHIP_CASE(R, U) \
-    if (rows_per_wave == R && k_unroll == U) return launch<R, 4, U>(qs, ds, x, y, m, n, k, s);
+    if (rows_per_wave == R && k_unroll == U) return launch_oneshot<R, 4, U>(qs, ds, x, y, m, n, k, s);
+        LHIP_CASE(1, 1) LHIP_CASE(1, 2) LHIP_CASE(1, 4)
+        LHIP_CASE(2, 1) LHIP_CASE(2, 2) LHIP_CASE(2, 4)
+        LHIP_CASE(4, 1) LHIP_CASE(4, 2) LHIP_CASE(4, 4)
+        LHIP_CASE(8, 1) LHIP_CASE(8, 2)
+#undef LHIP_CASE
+        return LHIP_ERR_UNSUPPORTED;
+    }
+#define LHIP_CASE(R, S) \
+    if (rows_per_wave == R && k_unroll == S) return launch_pipe<R, S>(qs, ds, x, y, m, n, k, blocks_per_cu, s);
     LHIP_CASE(1, 1) LHIP_CASE(1, 2) LHIP_CASE(1, 4)
     LHIP_CASE(2, 1) LHIP_CASE(2, 2) LHIP_CASE(2, 4)
     LHIP_CASE(4, 1) LHIP_CASE(4, 2) LHIP_CASE(4, 4)
-    LHIP_CASE(8, 1) LHIP_CASE(8, 2)
 #undef LHIP_CASE
     return LHIP_ERR_UNSUPPORTED;
 }
 
-// Heuristic: keep at least ~8 waves per CU (256 CUs) when N allows it, and
-// as many 16-byte loads in flight per lane as the registers carry.
-static void choose(int n, int k, int *rows_per_wave, int *k_unroll) {
-    int r = 4;
-    if (n < 8192) r = 2;
-    if (n < 4096) r = 1;
-    int u = (k >= 4096) ? 4 : (k >= 2048 ? 2 : 1);
-    if (r == 4 && u == 4) u = 2;
-    *rows_per_wave = r;
-    *k_unroll = u;
+// Default launch shape per problem size.
+static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_per_cu) {
+    int slices = 0;  // slices per pipeline step that divide K, 0 if none
+    if (k <= kMaxLdsK) {
+        if (k % 4096 == 0) slices = 4;
+        else if (k % 2048 == 0) slices = 2;
+        else if (k % 1024 == 0) slices = 1;
+    }
+    if (slices == 0) {  // ragged or very long K: one-shot kernel
+        *rows_per_wave = n >= 8192 ? 4 : (n >= 4096 ? 2 : 1);
+        *k_unroll = 1;
+        *blocks_per_cu = 0;
+        return;
+    }
+    // Measured on MI355X: very tall matrices run best with one fat wave per
+    // SIMD (2 rows x 4 slices, double-buffered); everything else with one row
+    // x 2 slices per step and as many resident workgroups as the LDS stage of
+    // the activations allows, up to 3 per CU.
+    if (n >= 32768 && slices == 4) {
+        *rows_per_wave = 2;
+        *k_unroll = 4;
+        *blocks_per_cu = 1;
+        return;
+    }
+    *rows_per_wave = 1;
+    *k_unroll = slices >= 2 ? 2 : 1;
+    const int fit = (160 * 1024) / (k * 4);  // workgroups whose staged activations fit the CU's LDS
+    *blocks_per_cu = fit >= 3 ? 3 : (fit >= 2 ? 2 : 1);
 }
 
 static lhip_status check_args(const void *planar, const float *x, float *y, int64_t m, int64_t n, int64_t k) {
@@ -192,10 +394,10 @@ using namespace lhip;
 extern "C" {
 
 lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
-                                     int64_t k, int rows_per_wave, int k_unroll, void *stream) {
+                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
     auto *base = static_cast<const uint8_t *>(planar_dev);
-    return dispatch(rows_per_wave, k_unroll, reinterpret_cast<const int8_t *>(base),
+    return dispatch(rows_per_wave, k_unroll, blocks_per_cu, reinterpret_cast<const int8_t *>(base),
                     reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_dev, y_dev, static_cast<int>(m),
                     static_cast<int>(n), static_cast<int>(k), as_stream(stream));
 }
@@ -203,9 +405,9 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
 lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
                                  int64_t k, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
-    int r, u;
-    choose(static_cast<int>(n), static_cast<int>(k), &r, &u);
-    return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, stream);
+    int r, u, b;
+    choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b);
+    return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, b, stream);
 }
 
 }  // extern "C"

@@ -99,26 +99,36 @@ def test_config0_single_matvec_4096(oracle):
     assert np.max(np.abs(y - seq)) < 1e-3 * max(1.0, float(np.max(np.abs(seq))))
 
 
-CFGS = [(1, 1), (1, 2), (1, 4), (2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4), (8, 1), (8, 2)]
+# (rows_per_wave, k_unroll, blocks_per_cu): blocks_per_cu == 0 is the one-shot kernel
+ONESHOT = [(r, u, 0) for r, u in [(1, 1), (1, 2), (1, 4), (2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4), (8, 1),
+                                  (8, 2)]]
+PIPE = [(r, s, b) for r in (1, 2, 4) for s in (1, 2, 4) for b in (1, 3)]
 
 
 @pytest.mark.parametrize("n,k", [(1, 32), (5, 64), (33, 1024), (37, 1056), (64, 2048), (130, 3104), (257, 4096),
-                                 (96, 14336)])
+                                 (2051, 4096), (96, 14336), (1029, 8192), (70, 16384), (9, 20480)])
 def test_matvec_every_launch_shape_ragged(oracle, n, k):
     qs, d = synth.q8_0_random(n, k, seed=n + k)
     x = synth.activations(1, k, seed=n * k)
     w = upload(qs, d)
     truth = oracle.matmul_f64(x, dequant_truth(oracle, qs, d))
-    for cfg in [None] + CFGS:
+    for cfg in [None] + ONESHOT:
         y = run_matmul(w, x, cfg)
         assert rel_err(y, truth) < TOL, (n, k, cfg)
+    for cfg in PIPE:
+        if k % (cfg[1] * 1024) == 0 and k <= 16384:
+            assert rel_err(run_matmul(w, x, cfg), truth) < TOL, (n, k, cfg)
+        else:  # the pipelined kernel needs K to be a whole number of steps that fits its LDS stage
+            with pytest.raises(capi.LhipError) as e:
+                run_matmul(w, x, cfg)
+            assert e.value.status == capi.LHIP_ERR_UNSUPPORTED
 
 
 def test_unbuilt_launch_shape_is_reported():
     qs, d = synth.q8_0_random(4, 32, seed=1)
     w = upload(qs, d)
     with pytest.raises(capi.LhipError) as e:
-        run_matmul(w, synth.activations(1, 32, 2), cfg=(3, 1))
+        run_matmul(w, synth.activations(1, 32, 2), cfg=(3, 1, 0))
     assert e.value.status == capi.LHIP_ERR_UNSUPPORTED
 
 
@@ -164,7 +174,7 @@ def test_integer_exact_any_order():
     x = rng.integers(-4, 5, (1, k)).astype(np.float32)
     want = (qs.astype(np.float64) * np.repeat(d.astype(np.float64), 32, axis=1)) @ x[0].astype(np.float64)
     w = upload(qs, d)
-    for cfg in [None, (1, 1), (2, 2), (4, 4), (8, 2)]:
+    for cfg in [None, (1, 1, 0), (2, 2, 0), (4, 4, 0), (8, 2, 0), (1, 2, 2), (2, 1, 1), (4, 2, 4)]:
         assert np.array_equal(run_matmul(w, x, cfg)[0].astype(np.float64), want), cfg
 
 
