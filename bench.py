@@ -193,6 +193,28 @@ def main():
         per_shape[nm] = {"n": shapes[nm][0], "k": shapes[nm][1], "us": round(us, 2),
                          "gbs": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
+    # Calibration: plain copy and read-only kernels of known size (1 GiB), for
+    # scaling hardware byte counters and as the streaming rate of this part.
+    cal_n = 1 << 30
+    cal_src = torch.empty(cal_n, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+    cal_dst = torch.empty(cal_n, dtype=torch.uint8, device=dev)
+    cal_out = torch.zeros(1024, dtype=torch.int32, device=dev)
+    calibration = {}
+    for label, fn, moved in (
+            ("copy_1GiB", lambda: lib.lhip_copy_bytes(cal_dst.data_ptr(), cal_src.data_ptr(), cal_n, stream), 2 * cal_n),
+            ("read_1GiB", lambda: lib.lhip_read_bytes(cal_src.data_ptr(), cal_n, cal_out.data_ptr(), stream), cal_n)):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 5
+        calibration[label] = {"us": round(us, 1), "gbs": round(moved / us / 1e3, 1)}
+    del cal_src, cal_dst
+
     achieved = step_bytes / (gpu_ms / args.steps) / 1e6  # GB/s from HIP events over the timed region
     roofline = {
         "bound": "hbm",
@@ -229,6 +251,7 @@ def main():
         },
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "per_shape": per_shape,
+        "calibration": calibration,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:

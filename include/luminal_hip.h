@@ -97,13 +97,15 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
 /* Same operator with the launch shape given by the caller instead of chosen by
  * the library (for tuning and for tests that cover every shape).
  * blocks_per_cu in 1..16 runs the persistent pipelined kernel with that many
- * resident workgroups per compute unit (rows_per_wave in {1,2,4}, k_unroll =
- * 1024-quant slices per pipeline step in {1,2,4}, K <= 16384);
+ * resident workgroups of waves_per_block (4, 8 or 16) wavefronts per compute
+ * unit (rows_per_wave in {1,2,4}, k_unroll = 1024-quant slices per pipeline
+ * step in {1,2,4}, K <= 16384 and a multiple of k_unroll*1024);
  * blocks_per_cu == 0 runs the one-shot kernel (rows_per_wave in {1,2,4,8},
- * k_unroll in {1,2,4}, any K).  LHIP_ERR_UNSUPPORTED for a combination that
- * is not built. */
+ * k_unroll in {1,2,4}, any K; waves_per_block ignored).  LHIP_ERR_UNSUPPORTED
+ * for a combination that is not built. */
 lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
-                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu, void *stream);
+                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu,
+                                     int waves_per_block, void *stream);
 
 /* Row gather: out[t][j] = dequant(W[(int)idx[t]][j]), idx carried as f32 like
  * the reference's (crates/luminal_cuda/src/quantized.rs:191-198,202-233), but

@@ -145,8 +145,8 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__res
 // Persistent, software-pipelined variant (the one the library normally runs).
 // Requires K to be a multiple of S*1024 and at most 16384.
 //
-// A grid of G workgroups of 4 wavefronts stays resident; wave w walks the row
-// groups w, w + 4G, ...  The activation vector is staged once per workgroup
+// A grid of G workgroups of W wavefronts stays resident; wave w walks the row
+// groups w, w + W*G, ...  The activation vector is staged once per workgroup
 // into LDS, so the only HBM traffic in the loop is the weight stream.  Work is
 // cut into steps of R rows x S slices of 1024 quants; the loads of step t+1
 // are issued before the arithmetic of step t starts (two register buffers,
@@ -212,16 +212,16 @@ __device__ __forceinline__ void compute_step(StepBuf<R, S> &b, const float4 *xs4
     }
 }
 
-template <int R, int S>
-__global__ __launch_bounds__(256) void q8_gemv_f32_pipe_kernel(const int8_t *__restrict__ qs,
+template <int R, int S, int W>
+__global__ __launch_bounds__(W * 64) void q8_gemv_f32_pipe_kernel(const int8_t *__restrict__ qs,
                                                                 const unsigned short *__restrict__ ds,
                                                                 const float *__restrict__ x, float *__restrict__ y,
                                                                 int n, int k) {
     extern __shared__ float4 xs4[];
     const unsigned lane = threadIdx.x & 63u;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: stays in a scalar register
-    const int wave_global = blockIdx.x * 4 + wave;
-    const int total_waves = gridDim.x * 4;
+    const int wave_global = blockIdx.x * W + wave;
+    const int total_waves = gridDim.x * W;
     x += static_cast<size_t>(blockIdx.y) * k;
     y += static_cast<size_t>(blockIdx.y) * n;
 
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256) void q8_gemv_f32_pipe_kernel(const int8_t *__r
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         const int k4 = k >> 2;
 #pragma unroll 4
-        for (int i = threadIdx.x; i < k4; i += 256) {
+        for (int i = threadIdx.x; i < k4; i += W * 64) {
             // destination index i = slice*256 + j*64 + l  <-  source slice*256 + l*4 + j
             const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
             xs4[i] = x4[src];
@@ -308,16 +308,16 @@ static lhip_status launch_oneshot(const int8_t *qs, const __half *ds, const floa
     return LHIP_OK;
 }
 
-template <int R, int S>
+template <int R, int S, int W>
 static lhip_status launch_pipe(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
                                int blocks_per_cu, hipStream_t s) {
     if (k % (S * 1024) != 0 || k > kMaxLdsK) return LHIP_ERR_UNSUPPORTED;
     const int n_groups = (n + R - 1) / R;
-    int grid = (n_groups + 3) / 4;
+    int grid = (n_groups + W - 1) / W;
     const int cap = kNumCUs * blocks_per_cu;
     if (grid > cap) grid = cap;
-    hipLaunchKernelGGL((q8_gemv_f32_pipe_kernel<R, S>), dim3(static_cast<unsigned>(grid), static_cast<unsigned>(m)),
-                       dim3(256), static_cast<size_t>(k) * sizeof(float), s, qs,
+    hipLaunchKernelGGL((q8_gemv_f32_pipe_kernel<R, S, W>), dim3(static_cast<unsigned>(grid), static_cast<unsigned>(m)),
+                       dim3(W * 64), static_cast<size_t>(k) * sizeof(float), s, qs,
                        reinterpret_cast<const unsigned short *>(ds), x, y, n, k);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
@@ -325,9 +325,10 @@ static lhip_status launch_pipe(const int8_t *qs, const __half *ds, const float *
 
 // Launch-shape table.  blocks_per_cu == 0 selects the one-shot kernel
 // (rows_per_wave in {1,2,4,8}, k_unroll in {1,2,4}); otherwise the pipelined
-// kernel (rows_per_wave in {1,2,4}, k_unroll = slices per step in {1,2,4}).
-static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, const int8_t *qs, const __half *ds,
-                            const float *x, float *y, int m, int n, int k, hipStream_t s) {
+// kernel (rows_per_wave in {1,2,4}, k_unroll = slices per step in {1,2,4},
+// waves_per_block in {4,8,16}).
+static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, int waves_per_block, const int8_t *qs,
+                            const __half *ds, const float *x, float *y, int m, int n, int k, hipStream_t s) {
     if (blocks_per_cu < 0 || blocks_per_cu > 16) return LHIP_ERR_UNSUPPORTED;
     if (blocks_per_cu == 0) {
 #define LHIP_CASE(R, U) \
@@ -339,8 +340,13 @@ static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, 
 #undef LHIP_CASE
         return LHIP_ERR_UNSUPPORTED;
     }
-#define LHIP_CASE(R, S) \
-    if (rows_per_wave == R && k_unroll == S) return launch_pipe<R, S>(qs, ds, x, y, m, n, k, blocks_per_cu, s);
+#define LHIP_CASE(R, S)                                                                                          \
+    if (rows_per_wave == R && k_unroll == S) {                                                                   \
+        if (waves_per_block == 4) return launch_pipe<R, S, 4>(qs, ds, x, y, m, n, k, blocks_per_cu, s);          \
+        if (waves_per_block == 8) return launch_pipe<R, S, 8>(qs, ds, x, y, m, n, k, blocks_per_cu, s);          \
+        if (waves_per_block == 16 && R * S <= 8) return launch_pipe<R, S, 16>(qs, ds, x, y, m, n, k, blocks_per_cu, s); \
+        return LHIP_ERR_UNSUPPORTED;                                                                             \
+    }
     LHIP_CASE(1, 1) LHIP_CASE(1, 2) LHIP_CASE(1, 4)
     LHIP_CASE(2, 1) LHIP_CASE(2, 2) LHIP_CASE(2, 4)
     LHIP_CASE(4, 1) LHIP_CASE(4, 2) LHIP_CASE(4, 4)
@@ -349,7 +355,8 @@ static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, 
 }
 
 // Default launch shape per problem size.
-static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_per_cu) {
+static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_per_cu, int *waves_per_block) {
+    *waves_per_block = 4;
     int slices = 0;  // slices per pipeline step that divide K, 0 if none
     if (k <= kMaxLdsK) {
         if (k % 4096 == 0) slices = 4;
@@ -375,7 +382,12 @@ static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_
     *rows_per_wave = 1;
     *k_unroll = slices >= 2 ? 2 : 1;
     const int fit = (160 * 1024) / (k * 4);  // workgroups whose staged activations fit the CU's LDS
-    *blocks_per_cu = fit >= 3 ? 3 : (fit >= 2 ? 2 : 1);
+    if (fit >= 3) {
+        *blocks_per_cu = 3;
+    } else {  // long K: one workgroup of 16 waves per CU shares a single staged copy
+        *blocks_per_cu = 1;
+        *waves_per_block = 16;
+    }
 }
 
 static lhip_status check_args(const void *planar, const float *x, float *y, int64_t m, int64_t n, int64_t k) {
@@ -394,10 +406,11 @@ using namespace lhip;
 extern "C" {
 
 lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
-                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu, void *stream) {
+                                     int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu,
+                                     int waves_per_block, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
     auto *base = static_cast<const uint8_t *>(planar_dev);
-    return dispatch(rows_per_wave, k_unroll, blocks_per_cu, reinterpret_cast<const int8_t *>(base),
+    return dispatch(rows_per_wave, k_unroll, blocks_per_cu, waves_per_block, reinterpret_cast<const int8_t *>(base),
                     reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_dev, y_dev, static_cast<int>(m),
                     static_cast<int>(n), static_cast<int>(k), as_stream(stream));
 }
@@ -405,9 +418,9 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
 lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
                                  int64_t k, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
-    int r, u, b;
-    choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b);
-    return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, b, stream);
+    int r, u, b, w;
+    choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
+    return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, b, w, stream);
 }
 
 }  // extern "C"

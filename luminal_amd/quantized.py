@@ -75,8 +75,9 @@ class QuantizedMatmul:
     """(.., M, K) x Q8_0 (N, K) -> (.., M, N), f32
     (QuantizedMatmul<f32>::process, crates/luminal_cuda/src/quantized.rs:116-168)."""
 
-    def __init__(self, rows_per_wave: int | None = None, k_unroll: int | None = None, blocks_per_cu: int = 0):
-        self.cfg = (rows_per_wave, k_unroll, blocks_per_cu) if rows_per_wave else None
+    def __init__(self, rows_per_wave: int | None = None, k_unroll: int | None = None, blocks_per_cu: int = 0,
+                 waves_per_block: int = 4):
+        self.cfg = (rows_per_wave, k_unroll, blocks_per_cu, waves_per_block) if rows_per_wave else None
 
     def process(self, x: torch.Tensor, w: Q8Weight) -> torch.Tensor:
         lib = capi.load_library()
@@ -91,7 +92,7 @@ class QuantizedMatmul:
         with torch.cuda.device(x.device):
             if self.cfg:
                 st = lib.lhip_q8_0_matmul_f32_cfg(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, self.cfg[0],
-                                                  self.cfg[1], self.cfg[2], _stream())
+                                                  self.cfg[1], self.cfg[2], self.cfg[3], _stream())
             else:
                 st = lib.lhip_q8_0_matmul_f32(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, _stream())
         capi.check(st, "lhip_q8_0_matmul_f32")

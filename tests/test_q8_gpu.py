@@ -102,7 +102,8 @@ def test_config0_single_matvec_4096(oracle):
 # (rows_per_wave, k_unroll, blocks_per_cu): blocks_per_cu == 0 is the one-shot kernel
 ONESHOT = [(r, u, 0) for r, u in [(1, 1), (1, 2), (1, 4), (2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4), (8, 1),
                                   (8, 2)]]
-PIPE = [(r, s, b) for r in (1, 2, 4) for s in (1, 2, 4) for b in (1, 3)]
+PIPE = [(r, s, b, w) for r in (1, 2, 4) for s in (1, 2, 4) for b, w in ((1, 4), (3, 4), (2, 8), (1, 16))
+        if not (w == 16 and r * s > 8)]
 
 
 @pytest.mark.parametrize("n,k", [(1, 32), (5, 64), (33, 1024), (37, 1056), (64, 2048), (130, 3104), (257, 4096),
@@ -174,7 +175,8 @@ def test_integer_exact_any_order():
     x = rng.integers(-4, 5, (1, k)).astype(np.float32)
     want = (qs.astype(np.float64) * np.repeat(d.astype(np.float64), 32, axis=1)) @ x[0].astype(np.float64)
     w = upload(qs, d)
-    for cfg in [None, (1, 1, 0), (2, 2, 0), (4, 4, 0), (8, 2, 0), (1, 2, 2), (2, 1, 1), (4, 2, 4)]:
+    for cfg in [None, (1, 1, 0), (2, 2, 0), (4, 4, 0), (8, 2, 0), (1, 2, 2), (2, 1, 1), (4, 2, 4), (2, 2, 1, 8),
+                (1, 2, 2, 16)]:
         assert np.array_equal(run_matmul(w, x, cfg)[0].astype(np.float64), want), cfg
 
 
