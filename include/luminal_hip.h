@@ -107,6 +107,23 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
                                      int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu,
                                      int waves_per_block, void *stream);
 
+/* Prefill GEMM: y[m][n] = sum_k x[m][k] * W[n][k] with bf16 activations
+ * (x (m, K) row-major, 16-byte aligned), f32 accumulation on the matrix cores
+ * and bf16 output (y (m, N) row-major).  The reference has no bf16 type and no
+ * Q8_0 GEMM on CUDA (crates/luminal_cuda/src/quantized.rs:146-164 re-runs the
+ * matvec per row); the counterpart is the Metal GEMM, which also rounds q*d to
+ * the activation type before the matrix unit
+ * (crates/luminal_metal/src/quantized.rs:54-61,63-199,353-376).  Weights are
+ * rounded to bf16 after dequantisation, so results are within 1e-2 of the f32
+ * semantics, not bit-equal.  K must be a multiple of 64 (LHIP_ERR_UNSUPPORTED
+ * otherwise). */
+lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
+                                  int64_t k, void *stream);
+/* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
+ * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each). */
+lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
+                                      int64_t k, int tile, void *stream);
+
 /* Row gather: out[t][j] = dequant(W[(int)idx[t]][j]), idx carried as f32 like
  * the reference's (crates/luminal_cuda/src/quantized.rs:191-198,202-233), but
  * read from device memory.  An index outside [0, n) yields a row of zeros. */

@@ -35,6 +35,8 @@ SIGNATURES = {
     "lhip_q8_0_dequant_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "lhip_q8_0_matmul_bf16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_bf16_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
     "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),

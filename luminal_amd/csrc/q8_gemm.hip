@@ -1,0 +1,240 @@
+// Q8_0 GEMM for prefill:  Y[M][N] = X[M][K] . W[N][K]^T, bf16 activations,
+// f32 accumulation on the matrix cores, bf16 output.
+//
+// The reference has no such kernel on CUDA (its QuantizedMatmul re-runs the
+// matvec once per activation row, crates/luminal_cuda/src/quantized.rs:146-164);
+// the design precedent is the Metal backend's GEMM, which dequantises a weight
+// tile into threadgroup memory (q * d rounded to the activation type) and feeds
+// the matrix unit (crates/luminal_metal/src/quantized.rs:54-61,63-199).  This
+// kernel does the same for gfx950:
+//   * a workgroup owns a BM x BN output tile and walks K in steps of 64 (two
+//     Q8_0 blocks);
+//   * activations go global -> registers -> LDS as bf16; weights go global
+//     (planar int8, 16-byte loads) -> registers -> dequantised q*d, rounded to
+//     bf16 (v_cvt_pk_bf16_f32, round-to-nearest-even) -> LDS;
+//   * LDS is double-buffered: the global loads of tile t+1 are in flight while
+//     the MFMAs of tile t run, and one barrier per tile separates them;
+//   * each wavefront computes a (BM/WM) x (BN/WN) sub-tile with
+//     v_mfma_f32_32x32x16_bf16; LDS rows are padded by 16 bytes so the 16-byte
+//     operand reads of 8 consecutive lanes hit all banks once;
+//   * workgroups that share a weight tile (same N tile, different M tiles) get
+//     consecutive slots on the same XCD (block id modulo 8), so the weight tile
+//     is fetched from HBM once and re-read from that XCD's L2.
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace lhip {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t gu32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBK = 64;             // K per tile: two Q8_0 blocks
+constexpr int kRowBytes = 144;      // 64 bf16 + 16 bytes of padding
+
+__device__ __forceinline__ float sbyte(uint32_t w, int i) {
+    return static_cast<float>(static_cast<int8_t>((w >> (8 * i)) & 0xff));
+}
+
+// 4 packed int8 -> 4 bf16 (q * d, rounded to nearest even), as two dwords.
+__device__ __forceinline__ uint2 dequant4_bf16(uint32_t q4, float d) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 lo = {static_cast<__bf16>(sbyte(q4, 0) * d), static_cast<__bf16>(sbyte(q4, 1) * d)};
+    bf16x2 hi = {static_cast<__bf16>(sbyte(q4, 2) * d), static_cast<__bf16>(sbyte(q4, 3) * d)};
+    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
+                                                                   const __half *__restrict__ ds,
+                                                                   const __bf16 *__restrict__ x,
+                                                                   __bf16 *__restrict__ y, int M, int N, int K,
+                                                                   int m_tiles, int n_tiles) {
+    constexpr int T = WM * WN * 64;
+    constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 MFMA tiles per wave
+    constexpr int A_CHUNKS = BM * 8 / T;       // 16-byte chunks (8 bf16) per thread per tile
+    constexpr int B_CHUNKS = BN * 4 / T;       // 16-byte chunks (16 int8) per thread per tile
+    static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * 8 % T == 0 && BN * 4 % T == 0, "tile/thread mismatch");
+    constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x (A tile, B tile)
+
+    // Block id -> (m tile, n tile): ids that differ by 8 run on the same XCD;
+    // the m tiles of one n tile take consecutive such ids.
+    int mt, nt;
+    {
+        const int id = blockIdx.x;
+        const int xcd = id & 7, slot = id >> 3;
+        const int n_hi = slot / m_tiles;
+        mt = slot - n_hi * m_tiles;
+        nt = n_hi * 8 + xcd;
+        if (nt >= n_tiles) return;  // grid is padded to a multiple of 8 n tiles
+    }
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int nblk = K >> 5;
+
+    // Per-thread global sources (rows past the edge re-read the last row; their results are not stored).
+    const __bf16 *a_src[A_CHUNKS];
+    int a_dst[A_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        const int c = tid + i * T;
+        const int row = c >> 3, col = (c & 7) * 8;
+        a_src[i] = x + static_cast<size_t>(min(m0 + row, M - 1)) * K + col;
+        a_dst[i] = row * kRowBytes + col * 2;
+    }
+    const int8_t *b_src[B_CHUNKS];
+    const __half *d_src[B_CHUNKS];
+    int b_dst[B_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+        const int c = tid + i * T;
+        const int row = c >> 2, q16 = c & 3;
+        const int grow = min(n0 + row, N - 1);
+        b_src[i] = qs + static_cast<size_t>(grow) * K + q16 * 16;
+        d_src[i] = ds + static_cast<size_t>(grow) * nblk + (q16 >> 1);
+        b_dst[i] = row * kRowBytes + q16 * 32;
+    }
+
+    gu32x4 a_reg[A_CHUNKS], b_reg[B_CHUNKS];
+    __half d_reg[B_CHUNKS];
+    auto load_tile = [&](int kt) {
+        const int k0 = kt * kBK;
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) a_reg[i] = *reinterpret_cast<const gu32x4 *>(a_src[i] + k0);
+#pragma unroll
+        for (int i = 0; i < B_CHUNKS; ++i) {
+            b_reg[i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
+            d_reg[i] = d_src[i][k0 >> 5];
+        }
+    };
+    auto store_tile = [&](int buf) {
+        unsigned char *A = lds + buf * (A_BYTES + B_BYTES);
+        unsigned char *B = A + A_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[i];
+#pragma unroll
+        for (int i = 0; i < B_CHUNKS; ++i) {
+            const float d = __half2float(d_reg[i]);
+            const uint2 w0 = dequant4_bf16(b_reg[i].x, d), w1 = dequant4_bf16(b_reg[i].y, d);
+            const uint2 w2 = dequant4_bf16(b_reg[i].z, d), w3 = dequant4_bf16(b_reg[i].w, d);
+            gu32x4 lo = {w0.x, w0.y, w1.x, w1.y}, hi = {w2.x, w2.y, w3.x, w3.y};
+            *reinterpret_cast<gu32x4 *>(B + b_dst[i]) = lo;
+            *reinterpret_cast<gu32x4 *>(B + b_dst[i] + 16) = hi;
+        }
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int KT = K / kBK;
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    // MFMA operand addresses inside a tile: lane l reads 8 consecutive k of row (l % 32), k group (l / 32).
+    const int frag_off = (lane & 31) * kRowBytes + (lane >> 5) * 16;
+    for (int kt = 0; kt < KT; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < KT) load_tile(kt + 1);
+        const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
+        const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+            bf16x8 af[FM], bfr[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8 *>(A + i * 32 * kRowBytes + kk * 32);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) bfr[j] = *reinterpret_cast<const bf16x8 *>(B + j * 32 * kRowBytes + kk * 32);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < KT) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Epilogue: acc element v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile.
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int col = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = static_cast<__bf16>(acc[i][j][v]);
+            }
+        }
+}
+
+template <int BM, int BN, int WM, int WN>
+static lhip_status launch_gemm(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
+                               hipStream_t s) {
+    const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
+    const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
+    const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
+    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN>;
+    if (lds_bytes > 64 * 1024) {
+        // Opting in to more than 64 KiB of dynamic LDS is a per-function attribute.
+        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    }
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad)), dim3(WM * WN * 64), lds_bytes, s, qs,
+                       ds, static_cast<const __bf16 *>(x), static_cast<__bf16 *>(y), m, n, k, m_tiles, n_tiles);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+}  // namespace lhip
+
+using namespace lhip;
+
+extern "C" {
+
+lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
+                                      int64_t k, int tile, void *stream) {
+    if (!planar_dev || !x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (k % kBK != 0) return LHIP_ERR_UNSUPPORTED;
+    if (!aligned(planar_dev, 256) || !aligned(x_dev, 16) || !aligned(y_dev, 2)) return LHIP_ERR_MISALIGNED;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    auto *qs = reinterpret_cast<const int8_t *>(base);
+    auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
+    const int mi = static_cast<int>(m), ni = static_cast<int>(n), ki = static_cast<int>(k);
+    hipStream_t s = as_stream(stream);
+    switch (tile) {
+        case 0: return launch_gemm<256, 128, 4, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        case 1: return launch_gemm<128, 128, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        case 2: return launch_gemm<128, 64, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        case 3: return launch_gemm<64, 64, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        default: return LHIP_ERR_UNSUPPORTED;
+    }
+}
+
+lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
+                                  int64_t k, void *stream) {
+    // Largest tile that still gives every CU (256) at least one workgroup.
+    auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    int tile = 3;
+    if (blocks(256, 128) >= 256) tile = 0;
+    else if (blocks(128, 128) >= 256) tile = 1;
+    else if (blocks(128, 64) >= 256) tile = 2;
+    return lhip_q8_0_matmul_bf16_cfg(planar_dev, x_dev, y_dev, m, n, k, tile, stream);
+}
+
+}  // extern "C"

@@ -99,6 +99,35 @@ class QuantizedMatmul:
         return out
 
 
+class QuantizedMatmulBf16:
+    """(.., M, K) bf16 x Q8_0 (N, K) -> (.., M, N) bf16 with f32 accumulation on
+    the matrix cores (the prefill path; dispatch by dtype, where the Metal
+    backend dispatches matvec vs matmul by M,
+    crates/luminal_metal/src/quantized.rs:339-376)."""
+
+    def __init__(self, tile: int | None = None):
+        self.tile = tile
+
+    def process(self, x: torch.Tensor, w: Q8Weight) -> torch.Tensor:
+        lib = capi.load_library()
+        if x.dtype != torch.bfloat16 or not x.is_cuda:
+            raise TypeError("QuantizedMatmulBf16 expects bf16 activations on the GPU")
+        if x.shape[-1] != w.k:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "QuantizedMatmulBf16",
+                                 f"activation K {x.shape[-1]} != weight K {w.k}")
+        x = x.contiguous()
+        m = x.numel() // w.k
+        out = torch.empty(x.shape[:-1] + (w.n,), dtype=torch.bfloat16, device=x.device)
+        with torch.cuda.device(x.device):
+            if self.tile is None:
+                st = lib.lhip_q8_0_matmul_bf16(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, _stream())
+            else:
+                st = lib.lhip_q8_0_matmul_bf16_cfg(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, self.tile,
+                                                   _stream())
+        capi.check(st, "lhip_q8_0_matmul_bf16")
+        return out
+
+
 class QuantizedGather:
     """Row gather from a Q8_0 table; indices are f32 as in the reference
     (QuantizedGather<f32>::process, crates/luminal_cuda/src/quantized.rs:202-233)."""

@@ -1,0 +1,133 @@
+"""Parity of the Q8_0 prefill GEMM (bf16 activations, f32 accumulate on MFMA,
+bf16 out) with the CPU oracle, through the C ABI.
+
+Bar for bf16-output paths: max |y - t| / max(|t|, rms(t)) <= 1e-2 against the f64
+truth computed from the same bf16 activations and the exactly dequantised
+weights.  (The kernel rounds q*d to bf16, an error proportional to the size of
+the whole dot product, not of its possibly cancelled result; hence rms(t) in the
+denominator.)  The norm-wise error ||y - t|| / ||t|| is held to 4e-3.
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from luminal_amd import capi, synth  # noqa: E402
+from luminal_amd.quantized import Q8Weight, QuantizedMatmulBf16  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-2
+
+
+def bf16_err(y, truth):
+    y = np.asarray(y, np.float64)
+    t = np.asarray(truth, np.float64)
+    rms = float(np.sqrt(np.mean(t * t))) + 1e-300
+    elem = float(np.max(np.abs(y - t) / np.maximum(np.abs(t), rms)))
+    norm = float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300))
+    return elem, norm
+
+
+def upload(qs, d):
+    n, k = qs.shape
+    return Q8Weight.from_raw(synth.q8_0_raw_blocks(qs, d), n, k, DEV)
+
+
+def bf16_activations(oracle, m, k, seed):
+    x = synth.activations(m, k, seed)
+    bits = oracle.f32_to_bf16_bits(x)
+    return oracle.bf16_bits_to_f32(bits), bits
+
+
+def run(w, bits, tile=None):
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y = QuantizedMatmulBf16(tile).process(x, w)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+def truth_for(oracle, qs, d, xf):
+    wf = oracle.q8_0_dequant(synth.q8_0_raw_blocks(qs, d), qs.size).reshape(qs.shape)
+    return oracle.matmul_f64(xf, wf)
+
+
+@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (16, 512, 1024), (33, 67, 128), (130, 200, 256), (257, 129, 4096),
+                                   (128, 1024, 4096), (300, 96, 14336)])
+def test_gemm_vs_oracle_all_tiles_ragged(oracle, tile, m, n, k):
+    qs, d = synth.q8_0_random(n, k, seed=m + n + k)
+    xf, bits = bf16_activations(oracle, m, k, seed=m * n)
+    y = run(upload(qs, d), bits, tile)
+    assert y.shape == (m, n)
+    elem, norm = bf16_err(y, truth_for(oracle, qs, d, xf))
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+
+
+def test_gemm_integer_exact():
+    # small integers, power-of-two scales: q*d is exact in bf16 and every partial sum exact in f32,
+    # so the output must equal the bf16 rounding of the exact integer result bit for bit
+    rng = np.random.default_rng(5)
+    m, n, k = 70, 150, 512
+    qs = rng.integers(-8, 9, (n, k), dtype=np.int8)
+    d = (2.0 ** rng.integers(-2, 2, (n, k // 32))).astype(np.float16)
+    x = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    bits = (x.view(np.uint32) >> 16).astype(np.uint16)  # small ints are bf16-exact
+    want = x.astype(np.float64) @ (qs.astype(np.float64) * np.repeat(d.astype(np.float64), 32, axis=1)).T
+    want_bf16 = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).float().numpy()
+    w = upload(qs, d)
+    for tile in (None, 0, 1, 2, 3):
+        assert np.array_equal(run(w, bits, tile), want_bf16), tile
+
+
+def test_reference_metal_matmul_case(oracle):
+    """crates/luminal_metal/src/quantized.rs:937-986: W 512x1024 ints in 0..5, d = 1.0, x 16x1024 in
+    U(-0.5, 0.5); its fp16 variant (:988-1038) accepts an absolute error of 1.0 because it accumulates in
+    half; with f32 accumulation the bf16 result stays within bf16 rounding of the truth."""
+    rng = np.random.default_rng(6)
+    qs = rng.integers(0, 5, (512, 1024), dtype=np.int8)
+    d = np.ones((512, 32), np.float16)
+    x = rng.uniform(-0.5, 0.5, (16, 1024)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x)
+    xf = oracle.bf16_bits_to_f32(bits)
+    truth = xf.astype(np.float64) @ qs.T.astype(np.float64)
+    y = run(upload(qs, d), bits)
+    assert np.max(np.abs(y - truth) / np.maximum(np.abs(truth), 1.0)) < 2.0 ** -8
+
+
+@pytest.mark.parametrize("name,m", [("q", 128), ("k", 512), ("down", 128), ("gate", 2048)])
+def test_full_size_prefill_shapes(oracle, name, m):
+    """BASELINE config 2 shapes; the oracle runs on a sample of weight rows."""
+    n, k = synth.LLAMA3_8B_PROJ[name]
+    qs, d = synth.q8_0_random(n, k, seed=300 + m)
+    xf, bits = bf16_activations(oracle, m, k, seed=301)
+    y = run(upload(qs, d), bits)
+    rows = np.unique(np.concatenate([np.arange(40), np.arange(n - 40, n),
+                                     np.random.default_rng(7).integers(0, n, 176)]))
+    truth = truth_for(oracle, qs[rows], d[rows], xf)
+    elem, norm = bf16_err(y[:, rows], truth)
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+    # zero activations give exactly zero; one-hot activation row gives the bf16-rounded weight column
+    e = np.zeros((m, k), np.float32)
+    e[m // 2, 77] = 1.0
+    ye = run(upload(qs, d), (e.view(np.uint32) >> 16).astype(np.uint16))
+    col = (qs[:, 77].astype(np.float32) * d[:, 77 // 32].astype(np.float32))
+    want = torch.from_numpy(col).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(ye[m // 2], want)
+    assert not ye[np.arange(m) != m // 2].any()
+
+
+def test_gemm_argument_errors():
+    lib = capi.load_library()
+    w = upload(*synth.q8_0_random(64, 96, seed=1))
+    x = torch.zeros((4, 96), dtype=torch.bfloat16, device=DEV)
+    y = torch.zeros((4, 64), dtype=torch.bfloat16, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    # K = 96 is not a multiple of 64
+    assert lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 4, 64, 96, s) == \
+        capi.LHIP_ERR_UNSUPPORTED
+    assert lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), None, y.data_ptr(), 4, 64, 128, s) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 0, 64, 128, s) == \
+        capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 4, 64, 128, 9, s) == \
+        capi.LHIP_ERR_UNSUPPORTED
