@@ -12,8 +12,9 @@
 //   * activations go global -> registers -> LDS as bf16; weights go global
 //     (planar int8, 16-byte loads) -> registers -> dequantised q*d, rounded to
 //     bf16 (v_cvt_pk_bf16_f32, round-to-nearest-even) -> LDS;
-//   * LDS is double-buffered: the global loads of tile t+1 are in flight while
-//     the MFMAs of tile t run, and one barrier per tile separates them;
+//   * LDS is double-buffered and the global loads run D = 4 tiles ahead in
+//     rotating register sets, so HBM/L2 latency is covered by three tiles of
+//     MFMA work; one barrier per tile separates LDS writers from readers;
 //   * each wavefront computes a (BM/WM) x (BN/WN) sub-tile with
 //     v_mfma_f32_32x32x16_bf16; LDS rows are padded by 16 bytes so the 16-byte
 //     operand reads of 8 consecutive lanes hit all banks once;
@@ -45,7 +46,8 @@ __device__ __forceinline__ uint2 dequant4_bf16(uint32_t q4, float d) {
     return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
 }
 
-template <int BM, int BN, int WM, int WN>
+// D = register prefetch depth in K tiles (D > 1 needs K % (64*D) == 0 and D even).
+template <int BM, int BN, int WM, int WN, int D>
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
                                                                    const __half *__restrict__ ds,
                                                                    const __bf16 *__restrict__ x,
@@ -102,28 +104,30 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         b_dst[i] = row * kRowBytes + q16 * 32;
     }
 
-    gu32x4 a_reg[A_CHUNKS], b_reg[B_CHUNKS];
-    __half d_reg[B_CHUNKS];
-    auto load_tile = [&](int kt) {
-        const int k0 = kt * kBK;
+    // D register sets: tile t lives in set t % D from its load until it is written to LDS.
+    gu32x4 a_reg[D][A_CHUNKS], b_reg[D][B_CHUNKS];
+    __half d_reg[D][B_CHUNKS];
+    const int KT = K / kBK;
+    auto load_tile = [&](int set, int kt) {
+        const int k0 = min(kt, KT - 1) * kBK;  // tiles past the end re-read the last one (never used)
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) a_reg[i] = *reinterpret_cast<const gu32x4 *>(a_src[i] + k0);
+        for (int i = 0; i < A_CHUNKS; ++i) a_reg[set][i] = *reinterpret_cast<const gu32x4 *>(a_src[i] + k0);
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
-            b_reg[i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
-            d_reg[i] = d_src[i][k0 >> 5];
+            b_reg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
+            d_reg[set][i] = d_src[i][k0 >> 5];
         }
     };
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int set, int buf) {
         unsigned char *A = lds + buf * (A_BYTES + B_BYTES);
         unsigned char *B = A + A_BYTES;
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[i];
+        for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
-            const float d = __half2float(d_reg[i]);
-            const uint2 w0 = dequant4_bf16(b_reg[i].x, d), w1 = dequant4_bf16(b_reg[i].y, d);
-            const uint2 w2 = dequant4_bf16(b_reg[i].z, d), w3 = dequant4_bf16(b_reg[i].w, d);
+            const float d = __half2float(d_reg[set][i]);
+            const uint2 w0 = dequant4_bf16(b_reg[set][i].x, d), w1 = dequant4_bf16(b_reg[set][i].y, d);
+            const uint2 w2 = dequant4_bf16(b_reg[set][i].z, d), w3 = dequant4_bf16(b_reg[set][i].w, d);
             gu32x4 lo = {w0.x, w0.y, w1.x, w1.y}, hi = {w2.x, w2.y, w3.x, w3.y};
             *reinterpret_cast<gu32x4 *>(B + b_dst[i]) = lo;
             *reinterpret_cast<gu32x4 *>(B + b_dst[i] + 16) = hi;
@@ -138,16 +142,9 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    const int KT = K / kBK;
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
     // MFMA operand addresses inside a tile: lane l reads 8 consecutive k of row (l % 32), k group (l / 32).
     const int frag_off = (lane & 31) * kRowBytes + (lane >> 5) * 16;
-    for (int kt = 0; kt < KT; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < KT) load_tile(kt + 1);
+    auto compute_tile = [&](int buf) {
         const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
         const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
 #pragma unroll
@@ -163,8 +160,32 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
                 for (int j = 0; j < FN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < KT) store_tile(buf ^ 1);
-        __syncthreads();
+    };
+
+#pragma unroll
+    for (int j = 0; j < D; ++j) load_tile(j, j);
+    store_tile(0, 0);
+    __syncthreads();
+
+    if constexpr (D == 1) {
+        for (int kt = 0; kt < KT; ++kt) {
+            load_tile(0, kt + 1);
+            compute_tile(kt & 1);
+            store_tile(0, (kt + 1) & 1);
+            __syncthreads();
+        }
+    } else {
+        static_assert(D % 2 == 0, "LDS buffer parity must follow the register set");
+        for (int kt = 0; kt < KT; kt += D) {
+#pragma unroll
+            for (int j = 0; j < D; ++j) {
+                // set j held tile kt+j, already in LDS: refill it with tile kt+j+D
+                load_tile(j, kt + j + D);
+                compute_tile(j & 1);
+                store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
+                __syncthreads();
+            }
+        }
     }
 
     // Epilogue: acc element v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile.
@@ -181,13 +202,13 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int D>
 static lhip_status launch_gemm(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
                                hipStream_t s) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
-    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN>;
+    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D>;
     if (lds_bytes > 64 * 1024) {
         // Opting in to more than 64 KiB of dynamic LDS is a per-function attribute.
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -217,13 +238,19 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
     auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
     const int mi = static_cast<int>(m), ni = static_cast<int>(n), ki = static_cast<int>(k);
     hipStream_t s = as_stream(stream);
+    // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
+    const bool deep = (k % (kBK * 4)) == 0;
+#define LHIP_TILE(BM, BN, WM, WN)                                                                  \
+    return deep ? launch_gemm<BM, BN, WM, WN, 4>(qs, ds, x_dev, y_dev, mi, ni, ki, s)              \
+                : launch_gemm<BM, BN, WM, WN, 1>(qs, ds, x_dev, y_dev, mi, ni, ki, s)
     switch (tile) {
-        case 0: return launch_gemm<256, 128, 4, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
-        case 1: return launch_gemm<128, 128, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
-        case 2: return launch_gemm<128, 64, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
-        case 3: return launch_gemm<64, 64, 2, 2>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        case 0: LHIP_TILE(256, 128, 4, 2);
+        case 1: LHIP_TILE(128, 128, 2, 2);
+        case 2: LHIP_TILE(128, 64, 2, 2);
+        case 3: LHIP_TILE(64, 64, 2, 2);
         default: return LHIP_ERR_UNSUPPORTED;
     }
+#undef LHIP_TILE
 }
 
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
