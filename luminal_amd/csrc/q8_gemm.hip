@@ -92,7 +92,8 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         a_dst[i] = row * kRowBytes + col * 2;
     }
     const int8_t *b_src[B_CHUNKS];
-    const __half *d_src[B_CHUNKS];
+    const uint32_t *d_src[B_CHUNKS];  // the two scales of a K tile are one aligned dword (K/32 is even)
+    int d_shift[B_CHUNKS];
     int b_dst[B_CHUNKS];
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
@@ -100,13 +101,14 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         const int row = c >> 2, q16 = c & 3;
         const int grow = min(n0 + row, N - 1);
         b_src[i] = qs + static_cast<size_t>(grow) * K + q16 * 16;
-        d_src[i] = ds + static_cast<size_t>(grow) * nblk + (q16 >> 1);
+        d_src[i] = reinterpret_cast<const uint32_t *>(ds + static_cast<size_t>(grow) * nblk);
+        d_shift[i] = (q16 >> 1) * 16;
         b_dst[i] = row * kRowBytes + q16 * 32;
     }
 
     // D register sets: tile t lives in set t % D from its load until it is written to LDS.
     gu32x4 a_reg[D][A_CHUNKS], b_reg[D][B_CHUNKS];
-    __half d_reg[D][B_CHUNKS];
+    uint32_t d_reg[D][B_CHUNKS];  // both f16 scale codes of the tile
     const int KT = K / kBK;
     auto load_tile = [&](int set, int kt) {
         const int k0 = min(kt, KT - 1) * kBK;  // tiles past the end re-read the last one (never used)
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
             b_reg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
-            d_reg[set][i] = d_src[i][k0 >> 5];
+            d_reg[set][i] = d_src[i][k0 >> 6];
         }
     };
     auto store_tile = [&](int set, int buf) {
@@ -125,7 +127,10 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
-            const float d = __half2float(d_reg[set][i]);
+            // Opaque to the optimiser: keeps the unpacking of this set here, at its use,
+            // instead of next to its loads (where it would wait for data just requested).
+            asm volatile("" : "+v"(b_reg[set][i]), "+v"(d_reg[set][i]));
+            const float d = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[set][i] >> d_shift[i])));
             const uint2 w0 = dequant4_bf16(b_reg[set][i].x, d), w1 = dequant4_bf16(b_reg[set][i].y, d);
             const uint2 w2 = dequant4_bf16(b_reg[set][i].z, d), w3 = dequant4_bf16(b_reg[set][i].w, d);
             gu32x4 lo = {w0.x, w0.y, w1.x, w1.y}, hi = {w2.x, w2.y, w3.x, w3.y};
@@ -181,6 +186,10 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
             for (int j = 0; j < D; ++j) {
                 // set j held tile kt+j, already in LDS: refill it with tile kt+j+D
                 load_tile(j, kt + j + D);
+                // Keep the loads here, at the top of the step: if they sink towards the
+                // LDS stores below, the wait for the tile loaded D-1 steps ago also
+                // waits for them and the prefetch distance collapses.
+                __builtin_amdgcn_sched_barrier(0);
                 compute_tile(j & 1);
                 store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
                 __syncthreads();
