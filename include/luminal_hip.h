@@ -130,6 +130,41 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
 lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
                                  int64_t n, int64_t k, void *stream);
 
+/* ---- MXFP4 weights and the mixture-of-experts layer -------------------------
+ * No counterpart in the reference (it has no MXFP4 and no MoE op); built to its
+ * conventions: exact dequantisation, then f32-accumulated matmul
+ * (examples/llama/src/loader.rs:227-241), SwiGLU down(up(x) * swish(gate(x)))
+ * (examples/llama/src/model.rs:24-32).
+ *
+ * Raw MXFP4 (OCP Microscaling / gpt-oss packing): blocks of 17 bytes = 16 bytes
+ * of e2m1 nibbles (element 2i in the low nibble of byte i) + one e8m0 scale
+ * (2^(e-127)).  A weight (N, K) is N*K/32 blocks, row-major.  Planar form:
+ * nibble bytes uint8[N][K/2], padded to 256 B, then scales uint8[N][K/32]. */
+size_t lhip_mxfp4_raw_nbytes(int64_t n, int64_t k);
+size_t lhip_mxfp4_planar_nbytes(int64_t n, int64_t k);
+size_t lhip_mxfp4_planar_scale_offset(int64_t n, int64_t k);
+lhip_status lhip_mxfp4_repack(const void *raw_dev, void *planar_dev, int64_t n, int64_t k, void *stream);
+lhip_status lhip_mxfp4_unpack(const void *planar_dev, void *raw_dev, int64_t n, int64_t k, void *stream);
+/* Exact dequantisation to f32[N][K] (every e8m0 code, 0xff gives NaN). */
+lhip_status lhip_mxfp4_dequant_f32(const void *planar_dev, float *out_dev, int64_t n, int64_t k, void *stream);
+
+/* Router: for each of t tokens, the topk largest of its e logits (ties to the
+ * lower index) into sel[t][topk], and softmax over those k into wts[t][topk]. */
+lhip_status lhip_moe_route_topk(const float *logits_dev, int32_t *sel_dev, float *wts_dev, int64_t t, int64_t e,
+                                int64_t topk, void *stream);
+
+/* Expert layer: y[t] = sum_s wts[t][s] * down_e( up_e(x[t]) * swish(gate_e(x[t])) ), e = sel[t][s].
+ *   w_gate_up_planar : planar MXFP4 of shape (e*2*i, h): expert-major, rows [0,i) of an expert = gate, [i,2i) = up
+ *   w_down_planar    : planar MXFP4 of shape (e*h, i)
+ *   x, y             : bf16 (t, h); accumulation in f32 on the block-scaled matrix instruction
+ *   sel, wts         : routing as produced by lhip_moe_route_topk (an id outside [0,e) drops that term)
+ *   workspace_dev    : lhip_mxfp4_moe_workspace_nbytes(...) bytes, 256-byte aligned; contents are scratch
+ * h and i must be multiples of 32, e <= 1024.  e8m0 codes 0xff (NaN) in the weights are not supported here. */
+size_t lhip_mxfp4_moe_workspace_nbytes(int64_t t, int64_t h, int64_t i, int64_t e, int64_t topk);
+lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream);
+
 /* ---- calibration kernels ---------------------------------------------------
  * No counterpart in the reference.  A plain device-to-device copy and a
  * read-only pass with known byte counts, used to calibrate hardware counters

@@ -38,6 +38,15 @@ SIGNATURES = {
     "lhip_q8_0_matmul_bf16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_bf16_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_mxfp4_raw_nbytes": (_sz, [_i64, _i64]),
+    "lhip_mxfp4_planar_nbytes": (_sz, [_i64, _i64]),
+    "lhip_mxfp4_planar_scale_offset": (_sz, [_i64, _i64]),
+    "lhip_mxfp4_repack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_mxfp4_unpack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_mxfp4_dequant_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_moe_route_topk": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_mxfp4_moe_workspace_nbytes": (_sz, [_i64] * 5),
+    "lhip_mxfp4_moe_bf16": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp, _vp]),
     "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
     "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),
 }

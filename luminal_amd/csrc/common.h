@@ -45,4 +45,13 @@ static inline size_t q8_planar_nbytes(int64_t n, int64_t k) {
     return q8_scale_offset(n, k) + static_cast<size_t>(n) * static_cast<size_t>(k / 32) * 2;
 }
 
+// Planar MXFP4: [uint8 nibbles[N][K/2]] padded to 256 B, then [uint8 e8m0[N][K/32]].
+static inline size_t mx_scale_offset(int64_t n, int64_t k) {
+    size_t q = static_cast<size_t>(n) * static_cast<size_t>(k / 2);
+    return (q + 255) & ~size_t{255};
+}
+static inline size_t mx_planar_nbytes(int64_t n, int64_t k) {
+    return mx_scale_offset(n, k) + static_cast<size_t>(n) * static_cast<size_t>(k / 32);
+}
+
 }  // namespace lhip

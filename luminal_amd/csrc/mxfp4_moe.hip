@@ -1,0 +1,575 @@
+// MXFP4 mixture-of-experts layer on gfx950's block-scaled matrix instruction.
+//
+// Not in the reference (it has neither MXFP4 nor MoE); semantics follow its
+// conventions: weights dequantise exactly (e2m1 * 2^(e8m0-127)), the expert MLP is
+// luminal's SwiGLU  down( up(x) * swish(gate(x)) )  (examples/llama/src/model.rs:24-32,
+// src/hl_ops/unary.rs:169-177), routing is top-k of the logits with a softmax
+// over the selected k.
+//
+// v_mfma_scale_f32_16x16x128_f8f6f4 multiplies an fp8 operand by an fp4 operand
+// and applies one e8m0 scale per 32-element block to each — exactly the MXFP4
+// block structure — so the weights go from HBM into the instruction's
+// registers untouched: no dequantisation arithmetic, no LDS traffic for them.
+// Operand layout (measured on the part; lane l = (r, g) with r = l % 16,
+// g = l / 16; a K chunk is 128 elements):
+//   fp4 operand, 4 dwords : the 32 nibbles of block g (k in [32g, 32g+32)), even k low
+//   fp8 operand, 8 dwords : bytes 0-15 = k in [16g, 16g+16), bytes 16-31 = k in [64+16g, +16)
+//   scale (byte 0 of a VGPR): the e8m0 of (row r, block g), for either operand
+//   result, 4 floats      : C[4g + i][r], rows from the first operand, columns from the second
+// bf16 activations are not an MFMA input format here, so each activation is
+// split exactly into two fp8 numbers: per 32-block, scale 2^s with
+// max|x|/2^s in [128, 256); hi = fp8(x/2^s) keeps the top 4 significant bits,
+// lo = fp8(x/2^s - hi) the remaining 4 of bf16's 8 (exact down to 2^-10 of the
+// block maximum).  Two MFMAs (hi, lo) per weight fragment then give the exact
+// sum of exact products in f32, which is closer to the f32 semantics than a
+// bf16 MFMA over rounded weights would be.
+#include "common.h"
+
+namespace lhip {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t mu32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kChunk = 128;      // K elements per MFMA
+constexpr int kARow = 144;       // LDS bytes per activation row of a chunk: 128 fp8 + 16 padding
+
+static inline int64_t pad128(int64_t k) { return (k + 127) / 128 * 128; }
+
+// ---------------------------------------------------------------------------
+// Router: top-k of the logits (ties to the lower index), softmax over the k.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ logits, int T, int E, int topk,
+                                                        int *__restrict__ sel, float *__restrict__ wts) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= T) return;
+    const float *l = logits + static_cast<size_t>(t) * E;
+    int *s = sel + static_cast<size_t>(t) * topk;
+    float *w = wts + static_cast<size_t>(t) * topk;
+    for (int j = 0; j < topk; ++j) {
+        int best = -1;
+        float bv = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int r = 0; r < j; ++r) taken |= (s[r] == e);
+            if (taken) continue;
+            const float v = l[e];
+            if (best < 0 || v > bv) {
+                best = e;
+                bv = v;
+            }
+        }
+        s[j] = best;
+    }
+    const float mx = l[s[0]];
+    float sum = 0.f;
+    for (int j = 0; j < topk; ++j) {
+        w[j] = expf(l[s[j]] - mx);
+        sum += w[j];
+    }
+    const float inv = 1.0f / sum;
+    for (int j = 0; j < topk; ++j) w[j] *= inv;
+}
+
+// ---------------------------------------------------------------------------
+// Plan: group the R = T*topk routed entries by expert and cut each expert's rows
+// into tiles of BM.  One workgroup; E <= 1024.
+// ---------------------------------------------------------------------------
+struct MoePlan {
+    int *offsets;      // [E+1] first slot of each expert
+    int *slot_src;     // [R]   slot -> routed entry r = t*topk + s
+    int *slot_of;      // [R]   routed entry -> slot (-1 if its expert id is invalid)
+    int *tile_expert;  // [max_tiles]
+    int *tile_row0;    // [max_tiles] first slot of the tile
+    int *tile_rows;    // [max_tiles] valid rows in the tile
+    int *n_tiles;      // [1]
+};
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int *__restrict__ sel, int R, int E, int BM,
+                                                        MoePlan p) {
+    __shared__ int cnt[1024], off[1025], cur[1024];
+    for (int e = threadIdx.x; e < E; e += 1024) {
+        cnt[e] = 0;
+        cur[e] = 0;
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < R; r += 1024) {
+        const int e = sel[r];
+        if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int o = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            off[e] = o;
+            p.offsets[e] = o;
+            for (int m0 = 0; m0 < cnt[e]; m0 += BM) {
+                p.tile_expert[nt] = e;
+                p.tile_row0[nt] = o + m0;
+                p.tile_rows[nt] = min(BM, cnt[e] - m0);
+                ++nt;
+            }
+            o += cnt[e];
+        }
+        off[E] = o;
+        p.offsets[E] = o;
+        *p.n_tiles = nt;
+    }
+    __syncthreads();
+    // Order inside an expert's range is arbitrary (atomic): every row is computed
+    // independently, and slot_of lets the combine step find it again.
+    for (int r = threadIdx.x; r < R; r += 1024) {
+        const int e = sel[r];
+        if (e >= 0 && e < E) {
+            const int pos = off[e] + atomicAdd(&cur[e], 1);
+            p.slot_src[pos] = r;
+            p.slot_of[r] = pos;
+        } else {
+            p.slot_of[r] = -1;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Activation quantisation: bf16 rows -> fp8 hi plane, fp8 lo plane, e8m0 scales.
+// One thread per 8 elements; the 4 threads of a 32-block share the maximum.
+// Planes have row stride Kp = K rounded up to 128, zero-filled past K; the scale
+// plane has row stride Kp/32, filled with 127 (2^0) past K.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
+                                                              uint8_t *__restrict__ lo, uint8_t *__restrict__ sc,
+                                                              int rows, int K, int Kp) {
+    const int per_row = Kp / 8;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t row = idx / per_row;
+    const int c8 = static_cast<int>(idx - row * per_row);
+    const bool live = row < static_cast<size_t>(rows);
+    const int k = c8 * 8;
+    float v[8];
+    mu32x4 raw = {0, 0, 0, 0};
+    if (live && k < K) raw = *reinterpret_cast<const mu32x4 *>(x + row * K + k);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(raw[j] << 16);
+        v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    // scale 2^s with amax / 2^s in [128, 256): s = floor(log2 amax) - 7
+    int e = 127;
+    float inv = 1.0f;
+    if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
+        const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);  // biased exponent (0 = subnormal)
+        e = max(ex - 7, 1);                                                       // e8m0 code of 2^s
+        inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);              // 2^-s, exact
+    }
+    uint32_t ph[2], pl[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float a0 = v[4 * j] * inv, a1 = v[4 * j + 1] * inv, a2 = v[4 * j + 2] * inv, a3 = v[4 * j + 3] * inv;
+        int h = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0, false);
+        h = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, h, true);
+        const float r0 = a0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), r1 = a1 - __builtin_amdgcn_cvt_f32_fp8(h, 1);
+        const float r2 = a2 - __builtin_amdgcn_cvt_f32_fp8(h, 2), r3 = a3 - __builtin_amdgcn_cvt_f32_fp8(h, 3);
+        int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, 0, false);
+        l = __builtin_amdgcn_cvt_pk_fp8_f32(r2, r3, l, true);
+        ph[j] = static_cast<uint32_t>(h);
+        pl[j] = static_cast<uint32_t>(l);
+    }
+    if (!live) return;
+    *reinterpret_cast<uint2 *>(hi + row * Kp + k) = make_uint2(ph[0], ph[1]);
+    *reinterpret_cast<uint2 *>(lo + row * Kp + k) = make_uint2(pl[0], pl[1]);
+    if ((c8 & 3) == 0) sc[row * (Kp / 32) + (c8 >> 2)] = static_cast<uint8_t>(k < K ? e : 127);
+}
+
+// ---------------------------------------------------------------------------
+// Grouped expert GEMM.  grid = (column blocks, max tiles); a workgroup of 4 waves
+// owns one row tile (up to BM = 16*MT routed rows of one expert) and 4*NT column
+// fragments of 16.  GATED: NT == 2, fragment 0 = gate rows, fragment 1 = the
+// matching up rows, output bf16 up*swish(gate).  Otherwise f32 output.
+// ---------------------------------------------------------------------------
+struct MoeGemmArgs {
+    const uint8_t *a_hi, *a_lo, *a_sc;  // activation planes, row stride Kp / Kp/32
+    const int *a_index;                 // slot -> routed entry (GEMM 1) or nullptr (rows are slots)
+    int a_div;                          // routed entry / a_div = activation row
+    const uint8_t *w_nib, *w_sc;        // planar weights of all experts, rows_per_expert rows each
+    int rows_per_expert;
+    int K, Kp;
+    int N;                              // output columns per expert (I or H)
+    const int *tile_expert, *tile_row0, *tile_rows, *n_tiles;
+    void *out;                          // bf16 [R][N] (gated) or f32 [R][N]
+};
+
+template <int MT, int NT>
+struct BSet {
+    mu32x4 q[NT];
+    uint32_t s[NT];
+};
+
+template <int MT, int NT, bool GATED>
+__global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
+    static_assert(!GATED || NT == 2, "gated tiles pair one gate fragment with one up fragment");
+    constexpr int BM = 16 * MT;
+    constexpr int D = 4;  // weight prefetch distance in chunks
+    constexpr int A_PLANE = BM * kARow;
+    constexpr int A_BUF = 2 * A_PLANE + BM * 4;  // hi, lo, scales
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x A_BUF
+
+    const int tile = blockIdx.y;
+    if (tile >= *g.n_tiles) return;
+    const int expert = g.tile_expert[tile];
+    const int row0 = g.tile_row0[tile];
+    const int rows = g.tile_rows[tile];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, grp = lane >> 4;
+    const int K = g.K, Kp = g.Kp;
+    const int chunks = Kp / kChunk;
+    const int steps = (chunks + D - 1) / D * D;  // padded with dead chunks that add zero
+
+    // ---- weight fragments: straight from global memory into MFMA registers
+    const uint8_t *w_row[NT];
+    const uint8_t *s_row[NT];
+    int col[NT];
+#pragma unroll
+    for (int f = 0; f < NT; ++f) {
+        int n, wrow;
+        if (GATED) {
+            n = (blockIdx.x * 4 + wave) * 16 + r;  // i index
+            wrow = (f == 0 ? 0 : g.N) + min(n, g.N - 1);
+        } else {
+            n = ((blockIdx.x * 4 + wave) * NT + f) * 16 + r;
+            wrow = min(n, g.N - 1);
+        }
+        col[f] = n;
+        const size_t grow = static_cast<size_t>(expert) * g.rows_per_expert + wrow;
+        w_row[f] = g.w_nib + grow * (K / 2);
+        s_row[f] = g.w_sc + grow * (K / 32);
+    }
+    BSet<MT, NT> bs[D];
+    auto load_b = [&](int set, int c) {
+        // Block g of chunk c; lanes whose block lies past K (tail or dead chunk) read block 0 and are masked.
+        const int kb = c * 4 + grp;
+        const bool valid = kb * 32 < K;
+        const int kbc = valid ? kb : 0;
+#pragma unroll
+        for (int f = 0; f < NT; ++f) {
+            mu32x4 q = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_row[f] + kbc * 16));
+            uint32_t s = __builtin_nontemporal_load(s_row[f] + kbc);
+            const mu32x4 zero = {0, 0, 0, 0};
+            bs[set].q[f] = valid ? q : zero;
+            bs[set].s[f] = valid ? s : 127u;
+        }
+    };
+
+    // ---- activation tile: global -> registers -> LDS (double-buffered), shared by the 4 waves
+    const uint8_t *a_src[MT];
+    int a_dst[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int q = tid + i * 256;  // chunk of 16 bytes: plane, row, 16-byte column
+        const int plane = q / (BM * 8), rem = q - plane * (BM * 8);
+        const int row = rem >> 3, c16 = rem & 7;
+        const int slot = row0 + min(row, rows - 1);  // rows past the tile re-read its last row (not stored)
+        const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
+        a_src[i] = (plane ? g.a_lo : g.a_hi) + static_cast<size_t>(arow) * Kp + c16 * 16;
+        a_dst[i] = plane * A_PLANE + row * kARow + c16 * 16;
+    }
+    const uint8_t *as_src = nullptr;
+    if (tid < BM) {
+        const int slot = row0 + min(tid, rows - 1);
+        const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
+        as_src = g.a_sc + static_cast<size_t>(arow) * (Kp / 32);
+    }
+    mu32x4 a_reg[MT];
+    uint32_t as_reg = 0;
+    auto load_a = [&](int c) {
+        const int cc = min(c, chunks - 1);  // dead chunks re-read the last one; their weights are zero
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a_reg[i] = *reinterpret_cast<const mu32x4 *>(a_src[i] + cc * kChunk);
+        if (tid < BM) as_reg = *reinterpret_cast<const uint32_t *>(as_src + cc * 4);
+    };
+    auto store_a = [&](int buf) {
+        unsigned char *base = lds + buf * A_BUF;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            asm volatile("" : "+v"(a_reg[i]));
+            *reinterpret_cast<mu32x4 *>(base + a_dst[i]) = a_reg[i];
+        }
+        if (tid < BM) *reinterpret_cast<uint32_t *>(base + 2 * A_PLANE + tid * 4) = as_reg;
+    };
+
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int f = 0; f < NT; ++f) acc[i][f] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](int set, int buf) {
+        const unsigned char *base = lds + buf * A_BUF;
+        const unsigned char *ap = base + r * kARow + grp * 16;
+#pragma unroll
+        for (int f = 0; f < NT; ++f) asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const unsigned char *p = ap + i * 16 * kARow;
+            const mu32x4 h0 = *reinterpret_cast<const mu32x4 *>(p);
+            const mu32x4 h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
+            const mu32x4 l0 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE);
+            const mu32x4 l1 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE + 64);
+            const uint32_t sw = *reinterpret_cast<const uint32_t *>(base + 2 * A_PLANE + (i * 16 + r) * 4);
+            const int sa = static_cast<int>((sw >> (8 * grp)) & 0xff);
+            const v8i ah = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
+            const v8i al = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
+#pragma unroll
+            for (int f = 0; f < NT; ++f) {
+                const mu32x4 q = bs[set].q[f];
+                const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
+                const int sb = static_cast<int>(bs[set].s[f]);
+                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+            }
+        }
+    };
+
+    // ---- pipeline
+#pragma unroll
+    for (int j = 0; j < D; ++j) load_b(j, j);
+    load_a(0);
+    store_a(0);
+    __syncthreads();
+    for (int c0 = 0; c0 < steps; c0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int c = c0 + j;
+            load_a(c + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(j, j & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            load_b(j, c + D);  // refill the set just consumed
+            store_a((j + 1) & 1);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: acc[i][f][v] is row i*16 + 4*grp + v, column fragment f, column r
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int m = i * 16 + 4 * grp + v;
+            if (m >= rows) continue;
+            const size_t orow = static_cast<size_t>(row0 + m) * g.N;
+            if (GATED) {
+                if (col[0] < g.N) {
+                    const float gate = acc[i][0][v], up = acc[i][1][v];
+                    const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                    static_cast<__bf16 *>(g.out)[orow + col[0]] = static_cast<__bf16>(act);
+                }
+            } else {
+#pragma unroll
+                for (int f = 0; f < NT; ++f)
+                    if (col[f] < g.N) static_cast<float *>(g.out)[orow + col[f]] = acc[i][f][v];
+            }
+        }
+}
+
+// y[t][h] = bf16( sum_s wts[t][s] * out[slot_of[t*topk+s]][h] ), 4 columns per thread
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ out, const int *__restrict__ slot_of,
+                                                          const float *__restrict__ wts, __bf16 *__restrict__ y, int T,
+                                                          int H, int topk) {
+    const int h4 = H / 4;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<size_t>(T) * h4) return;
+    const int t = static_cast<int>(idx / h4), c = static_cast<int>(idx - static_cast<size_t>(t) * h4);
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < topk; ++s) {
+        const int slot = slot_of[t * topk + s];
+        if (slot < 0) continue;
+        const float w = wts[t * topk + s];
+        const float4 v = reinterpret_cast<const float4 *>(out + static_cast<size_t>(slot) * H)[c];
+        a.x = fmaf(w, v.x, a.x);
+        a.y = fmaf(w, v.y, a.y);
+        a.z = fmaf(w, v.z, a.z);
+        a.w = fmaf(w, v.w, a.w);
+    }
+    __bf16 *o = y + static_cast<size_t>(t) * H + c * 4;
+    o[0] = static_cast<__bf16>(a.x);
+    o[1] = static_cast<__bf16>(a.y);
+    o[2] = static_cast<__bf16>(a.z);
+    o[3] = static_cast<__bf16>(a.w);
+}
+
+// ---------------------------------------------------------------------------
+// Workspace carving (256-byte aligned pieces, in this order).
+// ---------------------------------------------------------------------------
+struct MoeWorkspace {
+    MoePlan plan;
+    uint8_t *x_hi, *x_lo, *x_sc;  // quantised x, T rows of Kp(H)
+    __bf16 *act;                  // [R][I]
+    uint8_t *a_hi, *a_lo, *a_sc;  // quantised act, R rows of Kp(I)
+    float *out;                   // [R][H]
+    size_t total;
+};
+
+static MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
+    MoeWorkspace w{};
+    const int64_t R = T * topk;
+    const int64_t max_tiles = R / 16 + E + 1;  // tiles of at least 16 rows, one partial tile per expert
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        uint8_t *p = base ? static_cast<uint8_t *>(base) + off : nullptr;
+        off += (bytes + 255) & ~size_t{255};
+        return p;
+    };
+    w.plan.offsets = reinterpret_cast<int *>(take((E + 1) * 4));
+    w.plan.slot_src = reinterpret_cast<int *>(take(R * 4));
+    w.plan.slot_of = reinterpret_cast<int *>(take(R * 4));
+    w.plan.tile_expert = reinterpret_cast<int *>(take(max_tiles * 4));
+    w.plan.tile_row0 = reinterpret_cast<int *>(take(max_tiles * 4));
+    w.plan.tile_rows = reinterpret_cast<int *>(take(max_tiles * 4));
+    w.plan.n_tiles = reinterpret_cast<int *>(take(4));
+    const int64_t Hp = pad128(H), Ip = pad128(I);
+    w.x_hi = take(T * Hp);
+    w.x_lo = take(T * Hp);
+    w.x_sc = take(T * (Hp / 32));
+    w.act = reinterpret_cast<__bf16 *>(take(R * I * 2));
+    w.a_hi = take(R * Ip);
+    w.a_lo = take(R * Ip);
+    w.a_sc = take(R * (Ip / 32));
+    w.out = reinterpret_cast<float *>(take(R * H * 4));
+    w.total = off;
+    return w;
+}
+
+template <int MT, int NT, bool GATED>
+static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
+    constexpr int BM = 16 * MT;
+    const size_t lds_bytes = 2 * (2 * static_cast<size_t>(BM) * kARow + BM * 4);
+    auto kern = mx_moe_gemm_kernel<MT, NT, GATED>;
+    if (lds_bytes > 64 * 1024)
+        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256),
+                       lds_bytes, s, a);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+static lhip_status check_moe_shape(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
+    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return LHIP_ERR_INVALID_SHAPE;
+    if (E > 1024 || topk > E || T * topk > (int64_t{1} << 24)) return LHIP_ERR_INVALID_SHAPE;
+    if (H % 32 != 0 || I % 32 != 0 || H > kMaxDim || I > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    return LHIP_OK;
+}
+
+}  // namespace lhip
+
+using namespace lhip;
+
+extern "C" {
+
+lhip_status lhip_moe_route_topk(const float *logits_dev, int32_t *sel_dev, float *wts_dev, int64_t t, int64_t e,
+                                int64_t topk, void *stream) {
+    if (!logits_dev || !sel_dev || !wts_dev) return LHIP_ERR_NULL_PTR;
+    if (t <= 0 || e <= 0 || topk <= 0 || topk > e || t > kMaxDim || e > 1024) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((t + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       logits_dev, static_cast<int>(t), static_cast<int>(e), static_cast<int>(topk), sel_dev, wts_dev);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+size_t lhip_mxfp4_moe_workspace_nbytes(int64_t t, int64_t h, int64_t i, int64_t e, int64_t topk) {
+    if (check_moe_shape(t, h, i, e, topk) != LHIP_OK) return 0;
+    return carve(nullptr, t, h, i, e, topk).total;
+}
+
+lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream) {
+    if (!w_gate_up_planar || !w_down_planar || !x_dev || !sel_dev || !wts_dev || !y_dev || !workspace_dev)
+        return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_moe_shape(t, h, i, e, topk)) return s;
+    if (h % 4 != 0) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(w_gate_up_planar, 256) || !aligned(w_down_planar, 256) || !aligned(x_dev, 16) ||
+        !aligned(workspace_dev, 256) || !aligned(y_dev, 2))
+        return LHIP_ERR_MISALIGNED;
+    hipStream_t s = as_stream(stream);
+    const int T = static_cast<int>(t), H = static_cast<int>(h), I = static_cast<int>(i), E = static_cast<int>(e);
+    const int topk_i = static_cast<int>(topk), R = T * topk_i;
+    MoeWorkspace w = carve(workspace_dev, t, h, i, e, topk);
+    const int Hp = static_cast<int>(pad128(h)), Ip = static_cast<int>(pad128(i));
+
+    // Row tile: as many routed rows per expert as there are on average, 16..128.
+    const int avg = (R + E - 1) / E;
+    const int mt = avg > 64 ? 8 : (avg > 32 ? 4 : (avg > 16 ? 2 : 1));
+    const int BM = 16 * mt;
+    const int max_tiles = R / BM + E;
+
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel_dev, R, E, BM, w.plan);
+    LHIP_CHECK_LAUNCH();
+    {
+        const size_t threads = static_cast<size_t>(T) * (Hp / 8);
+        hipLaunchKernelGGL(mx_quantize_act_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s,
+                           static_cast<const __bf16 *>(x_dev), w.x_hi, w.x_lo, w.x_sc, T, H, Hp);
+        LHIP_CHECK_LAUNCH();
+    }
+    auto *gu = static_cast<const uint8_t *>(w_gate_up_planar);
+    auto *dn = static_cast<const uint8_t *>(w_down_planar);
+
+    MoeGemmArgs a1{};
+    a1.a_hi = w.x_hi; a1.a_lo = w.x_lo; a1.a_sc = w.x_sc;
+    a1.a_index = w.plan.slot_src; a1.a_div = topk_i;
+    a1.w_nib = gu; a1.w_sc = gu + mx_scale_offset(e * 2 * i, h);
+    a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
+    a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
+    a1.n_tiles = w.plan.n_tiles; a1.out = w.act;
+    const int cb1 = (I + 63) / 64;  // 4 waves x 16 gate/up pairs
+    lhip_status st;
+    switch (mt) {
+        case 1: st = launch_moe_gemm<1, 2, true>(a1, cb1, max_tiles, s); break;
+        case 2: st = launch_moe_gemm<2, 2, true>(a1, cb1, max_tiles, s); break;
+        case 4: st = launch_moe_gemm<4, 2, true>(a1, cb1, max_tiles, s); break;
+        default: st = launch_moe_gemm<8, 2, true>(a1, cb1, max_tiles, s); break;
+    }
+    if (st) return st;
+    {
+        const size_t threads = static_cast<size_t>(R) * (Ip / 8);
+        hipLaunchKernelGGL(mx_quantize_act_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s,
+                           w.act, w.a_hi, w.a_lo, w.a_sc, R, I, Ip);
+        LHIP_CHECK_LAUNCH();
+    }
+    MoeGemmArgs a2{};
+    a2.a_hi = w.a_hi; a2.a_lo = w.a_lo; a2.a_sc = w.a_sc;
+    a2.a_index = nullptr; a2.a_div = 1;
+    a2.w_nib = dn; a2.w_sc = dn + mx_scale_offset(e * h, i);
+    a2.rows_per_expert = H; a2.K = I; a2.Kp = Ip; a2.N = H;
+    a2.tile_expert = w.plan.tile_expert; a2.tile_row0 = w.plan.tile_row0; a2.tile_rows = w.plan.tile_rows;
+    a2.n_tiles = w.plan.n_tiles; a2.out = w.out;
+    if (mt == 1) {
+        st = launch_moe_gemm<1, 1, false>(a2, (H + 63) / 64, max_tiles, s);
+    } else {
+        const int cb2 = (H + 127) / 128;  // 4 waves x 2 fragments of 16
+        switch (mt) {
+            case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
+            case 4: st = launch_moe_gemm<4, 2, false>(a2, cb2, max_tiles, s); break;
+            default: st = launch_moe_gemm<8, 2, false>(a2, cb2, max_tiles, s); break;
+        }
+    }
+    if (st) return st;
+    {
+        const size_t threads = static_cast<size_t>(T) * (H / 4);
+        hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s, w.out,
+                           w.plan.slot_of, wts_dev, static_cast<__bf16 *>(y_dev), T, H, topk_i);
+        LHIP_CHECK_LAUNCH();
+    }
+    return LHIP_OK;
+}
+
+}  // extern "C"

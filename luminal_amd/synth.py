@@ -48,3 +48,28 @@ LLAMA3_8B_LAYERS = 32
 def q8_0_gemv_bytes(n: int, k: int) -> int:
     """Algorithmic bytes of one batch-1 Q8_0 matvec: weights once, x and y in f32."""
     return n * k * 34 // 32 + 4 * k + 4 * n
+
+
+def mxfp4_random(n: int, k: int, seed: int, exp_lo: int = -8, exp_hi: int = 0):
+    """Random MXFP4 weight: e2m1 codes uniform over the 16 values, one e8m0 scale
+    per 32-value block with exponent uniform in [exp_lo, exp_hi].
+    Returns (codes uint8 (n,k) in 0..15, scales uint8 (n,k//32))."""
+    assert k % 32 == 0
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 16, size=(n, k), dtype=np.uint8)
+    scales = (127 + rng.integers(exp_lo, exp_hi + 1, size=(n, k // 32))).astype(np.uint8)
+    return codes, scales
+
+
+def mxfp4_raw_blocks(codes: np.ndarray, scales: np.ndarray) -> np.ndarray:
+    """Pack e2m1 codes + e8m0 scales into raw 17-byte blocks (even element in the low nibble)."""
+    n_blocks = codes.size // 32
+    c = np.ascontiguousarray(codes, dtype=np.uint8).reshape(n_blocks, 16, 2)
+    raw = np.empty((n_blocks, 17), np.uint8)
+    raw[:, :16] = c[:, :, 0] | (c[:, :, 1] << 4)
+    raw[:, 16] = np.ascontiguousarray(scales, dtype=np.uint8).reshape(-1)
+    return raw.reshape(-1)
+
+
+# gpt-oss-style expert layer of the benchmark configuration
+MOE_HIDDEN, MOE_INTER, MOE_EXPERTS, MOE_TOPK = 2880, 2880, 32, 4

@@ -1,0 +1,140 @@
+"""MXFP4 storage, router and mixture-of-experts layer against the CPU oracle.
+
+MXFP4 and MoE do not exist in the reference, so its tests hold nothing for
+them: parity here is against the oracle only (pinned by the OCP MX value table
+and closed forms, see tests/test_oracle.py).  Bars: storage and dequantised
+weights bit-exact; the bf16-output layer within 1e-2 (max |y-t| / max(|t|,
+rms(t))) and 4e-3 norm-wise of the f64 truth that rounds the SwiGLU activations
+to bf16 like the kernel pipeline does.
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from luminal_amd import capi, synth  # noqa: E402
+from luminal_amd.moe import Mxfp4Weight, MoEExperts, route_topk  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def bf16_err(y, truth):
+    y = np.asarray(y, np.float64)
+    t = np.asarray(truth, np.float64)
+    rms = float(np.sqrt(np.mean(t * t))) + 1e-300
+    return (float(np.max(np.abs(y - t) / np.maximum(np.abs(t), rms))),
+            float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300)))
+
+
+@pytest.mark.parametrize("n,k", [(1, 32), (5, 96), (64, 2880), (300, 128)])
+def test_repack_round_trip_and_layout(n, k):
+    codes, scales = synth.mxfp4_random(n, k, seed=n + k)
+    raw = synth.mxfp4_raw_blocks(codes, scales)
+    w = Mxfp4Weight.from_raw(raw, n, k, DEV)
+    planar = w.planar.cpu().numpy()
+    off = capi.load_library().lhip_mxfp4_planar_scale_offset(n, k)
+    nib = planar[: n * k // 2].reshape(n, k // 2)
+    assert np.array_equal(nib & 15, codes[:, 0::2]) and np.array_equal(nib >> 4, codes[:, 1::2])
+    assert np.array_equal(planar[off:off + n * k // 32].reshape(n, k // 32), scales)
+    assert np.array_equal(w.to_raw().cpu().numpy(), raw)
+
+
+def test_dequant_bit_exact_every_code_times_every_scale(oracle):
+    n, k = 256, 64  # row r uses scale code r; both blocks hold all 16 codes twice
+    codes = np.tile(np.arange(16, dtype=np.uint8), (n, k // 16))
+    scales = np.repeat(np.arange(256, dtype=np.uint8)[:, None], k // 32, axis=1)
+    raw = synth.mxfp4_raw_blocks(codes, scales)
+    got = Mxfp4Weight.from_raw(raw, n, k, DEV).dequantize().cpu().numpy()
+    want = oracle.mxfp4_dequant(raw, n * k).reshape(n, k)
+    nan = np.isnan(want)
+    assert nan[255].all() and not nan[:255].any()
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_router_matches_oracle(oracle):
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((1000, 32)).astype(np.float32)
+    logits[7, :] = 0.25  # all tied: lowest indices win
+    sel, wts = route_topk(torch.from_numpy(logits).to(DEV), 4)
+    osel, owts = oracle.moe_route(logits, 4)
+    assert np.array_equal(sel.cpu().numpy(), osel)
+    assert np.allclose(wts.cpu().numpy(), owts, rtol=2e-6, atol=0)
+    assert list(sel[7].cpu().numpy()) == [0, 1, 2, 3]
+
+
+def make_layer(oracle, e, h, i, seed):
+    gu_c, gu_s = synth.mxfp4_random(e * 2 * i, h, seed=seed)
+    dn_c, dn_s = synth.mxfp4_random(e * h, i, seed=seed + 1)
+    gu_raw, dn_raw = synth.mxfp4_raw_blocks(gu_c, gu_s), synth.mxfp4_raw_blocks(dn_c, dn_s)
+    layer = MoEExperts(Mxfp4Weight.from_raw(gu_raw, e * 2 * i, h, DEV), Mxfp4Weight.from_raw(dn_raw, e * h, i, DEV),
+                       e, h, i)
+    w_gu = oracle.mxfp4_dequant(gu_raw, gu_c.size).reshape(e, 2 * i, h)
+    w_dn = oracle.mxfp4_dequant(dn_raw, dn_c.size).reshape(e, h, i)
+    return layer, w_gu, w_dn
+
+
+def run_layer(oracle, layer, t, h, e, topk, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((t, h)) * scale).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x)
+    xf = oracle.bf16_bits_to_f32(bits)
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    sel, wts = route_topk(torch.from_numpy(logits).to(DEV), topk)
+    xd = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y = layer.process(xd, sel, wts)
+    torch.cuda.synchronize()
+    return xf, sel.cpu().numpy(), wts.cpu().numpy(), y.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("t,e,h,i,topk", [(1, 4, 64, 64, 2), (5, 4, 160, 96, 2), (40, 8, 128, 288, 4),
+                                          (300, 8, 256, 160, 4), (1500, 4, 128, 128, 2), (64, 32, 96, 64, 4)])
+def test_moe_small_layers_vs_oracle(oracle, t, e, h, i, topk):
+    # ragged K (not multiples of 128), every row-tile size (16..128 rows), experts with no tokens
+    layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=t + e + h)
+    xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t * 7 + 1, scale=0.05)
+    truth = oracle.moe_forward(xf, w_gu, w_dn, sel, wts, act_bf16=True)
+    elem, norm = bf16_err(y, truth)
+    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+
+
+def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
+    # activations spanning many binades inside one 32-block: the hi/lo fp8 split must not lose the small ones
+    e, h, i, t, topk = 2, 64, 64, 16, 1
+    layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=99)
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((t, h)) * 2.0 ** rng.integers(-7, 1, (t, h))).astype(np.float32) * 0.05
+    bits = oracle.f32_to_bf16_bits(x)
+    xf = oracle.bf16_bits_to_f32(bits)
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    sel, wts = route_topk(torch.from_numpy(logits).to(DEV), topk)
+    y = layer.process(torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16), sel, wts)
+    truth = oracle.moe_forward(xf, w_gu, w_dn, sel.cpu().numpy(), wts.cpu().numpy(), act_bf16=True)
+    elem, norm = bf16_err(y.float().cpu().numpy(), truth)
+    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+
+
+@pytest.mark.parametrize("t", [1, 64, 1024])
+def test_moe_benchmark_layer(oracle, t):
+    """BASELINE config 3: H = I = 2880, 32 experts, top-4; the oracle runs on a sample of tokens."""
+    e, h, i, topk = synth.MOE_EXPERTS, synth.MOE_HIDDEN, synth.MOE_INTER, synth.MOE_TOPK
+    layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=2024)
+    xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t, scale=1.0)
+    pick = np.unique(np.concatenate([[0, t - 1], np.random.default_rng(1).integers(0, t, 4)]))
+    truth = oracle.moe_forward(xf[pick], w_gu, w_dn, sel[pick], wts[pick], act_bf16=True)
+    elem, norm = bf16_err(y[pick], truth)
+    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+    assert np.isfinite(y).all()
+
+
+def test_moe_argument_errors():
+    lib = capi.load_library()
+    p = 0x1000
+    assert lib.lhip_mxfp4_moe_workspace_nbytes(4, 64, 64, 4, 2) > 0
+    assert lib.lhip_mxfp4_moe_workspace_nbytes(4, 65, 64, 4, 2) == 0
+    assert lib.lhip_mxfp4_moe_workspace_nbytes(4, 64, 64, 4, 5) == 0
+    assert lib.lhip_mxfp4_moe_bf16(None, p, p, p, p, p, 4, 64, 64, 4, 2, p, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_mxfp4_moe_bf16(p, p, p, p, p, p, 4, 64, 48, 4, 2, p, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_mxfp4_moe_bf16(p + 64, p, p, p, p, p, 4, 64, 64, 4, 2, p, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_moe_route_topk(p, p, p, 4, 4, 5, None) == capi.LHIP_ERR_INVALID_SHAPE
