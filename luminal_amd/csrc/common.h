@@ -45,13 +45,23 @@ static inline size_t q8_planar_nbytes(int64_t n, int64_t k) {
     return q8_scale_offset(n, k) + static_cast<size_t>(n) * static_cast<size_t>(k / 32) * 2;
 }
 
-// Planar MXFP4: [uint8 nibbles[N][K/2]] padded to 256 B, then [uint8 e8m0[N][K/32]].
+// Planar MXFP4, tiled for the block-scaled MFMA: rows are grouped into panels of
+// 16 and K into chunks of 128 (both padded with zero weights / scale 2^0).  Tile
+// (panel, chunk) is 1 KiB of nibble bytes: 64 pieces of 16 bytes, piece g*16 + r
+// holding block (chunk*4 + g) of row (panel*16 + r) — the order in which the 64
+// lanes of a wavefront consume them, so one wave load is one contiguous KiB.
+// The scale plane has the same order, one byte per piece.
+static inline int64_t mx_panels(int64_t n) { return (n + 15) / 16; }
+static inline int64_t mx_chunks(int64_t k) { return (k + 127) / 128; }
 static inline size_t mx_scale_offset(int64_t n, int64_t k) {
-    size_t q = static_cast<size_t>(n) * static_cast<size_t>(k / 2);
-    return (q + 255) & ~size_t{255};
+    return static_cast<size_t>(mx_panels(n)) * static_cast<size_t>(mx_chunks(k)) * 1024;
 }
 static inline size_t mx_planar_nbytes(int64_t n, int64_t k) {
-    return mx_scale_offset(n, k) + static_cast<size_t>(n) * static_cast<size_t>(k / 32);
+    return mx_scale_offset(n, k) + static_cast<size_t>(mx_panels(n)) * static_cast<size_t>(mx_chunks(k)) * 64;
+}
+// Piece index (in units of 16 nibble bytes / 1 scale byte) of block kb of row.
+__host__ __device__ static inline size_t mx_piece(int64_t row, int64_t kb, int64_t chunks) {
+    return (static_cast<size_t>(row >> 4) * chunks + (kb >> 2)) * 64 + (kb & 3) * 16 + (row & 15);
 }
 
 }  // namespace lhip

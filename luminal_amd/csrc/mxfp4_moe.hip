@@ -71,6 +71,40 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
     for (int j = 0; j < topk; ++j) w[j] *= inv;
 }
 
+// One wavefront per token for E <= 64: lane e holds logit e; k rounds of a
+// wave-wide arg-max (larger value wins, ties to the lower index).
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(const float *__restrict__ logits, int T, int E, int topk,
+                                                             int *__restrict__ sel, float *__restrict__ wts) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    float v = lane < E ? logits[static_cast<size_t>(t) * E + lane] : 0.f;
+    bool avail = lane < E;
+    float mx = 0.f, sum = 0.f, mine = 0.f;
+    for (int j = 0; j < topk; ++j) {
+        float bv = v;
+        int bi = avail ? lane : 64;  // 64 = nothing to offer
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o);
+            const int oi = __shfl_xor(bi, o);
+            const bool take = (oi < 64) && (bi == 64 || ov > bv || (ov == bv && oi < bi));
+            if (take) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (j == 0) mx = bv;
+        const float w = expf(bv - mx);
+        sum += w;
+        if (lane == j) {
+            mine = w;
+            sel[static_cast<size_t>(t) * topk + j] = bi;
+        }
+        if (lane == bi) avail = false;
+    }
+    if (lane < topk) wts[static_cast<size_t>(t) * topk + lane] = mine * (1.0f / sum);
+}
+
 // ---------------------------------------------------------------------------
 // Plan: group the R = T*topk routed entries by expert and cut each expert's rows
 // into tiles of BM.  One workgroup; E <= 1024.
@@ -207,6 +241,7 @@ template <int MT, int NT>
 struct BSet {
     mu32x4 q[NT];
     uint32_t s[NT];
+    bool valid;  // wave-uniform: false for a dead chunk past the padded K
 };
 
 template <int MT, int NT, bool GATED>
@@ -229,42 +264,41 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, grp = lane >> 4;
-    const int K = g.K, Kp = g.Kp;
+    const int Kp = g.Kp;
     const int chunks = Kp / kChunk;
     const int steps = (chunks + D - 1) / D * D;  // padded with dead chunks that add zero
 
-    // ---- weight fragments: straight from global memory into MFMA registers
-    const uint8_t *w_row[NT];
-    const uint8_t *s_row[NT];
+    // ---- weight fragments: straight from global memory into MFMA registers.
+    // The planar weights are tiled so that the 64 pieces a wave needs for one
+    // fragment and one chunk are one contiguous KiB (lane order).
+    const uint8_t *w_tile[NT];
+    const uint8_t *s_tile[NT];
     int col[NT];
 #pragma unroll
     for (int f = 0; f < NT; ++f) {
-        int n, wrow;
+        int n0, wrow0;  // first column of the fragment, first weight row inside the expert
         if (GATED) {
-            n = (blockIdx.x * 4 + wave) * 16 + r;  // i index
-            wrow = (f == 0 ? 0 : g.N) + min(n, g.N - 1);
+            n0 = (blockIdx.x * 4 + wave) * 16;  // i index
+            wrow0 = (f == 0 ? 0 : g.N) + min(n0, g.N - 16);
         } else {
-            n = ((blockIdx.x * 4 + wave) * NT + f) * 16 + r;
-            wrow = min(n, g.N - 1);
+            n0 = ((blockIdx.x * 4 + wave) * NT + f) * 16;
+            wrow0 = min(n0, g.N - 16);
         }
-        col[f] = n;
-        const size_t grow = static_cast<size_t>(expert) * g.rows_per_expert + wrow;
-        w_row[f] = g.w_nib + grow * (K / 2);
-        s_row[f] = g.w_sc + grow * (K / 32);
+        col[f] = n0 + r;
+        const size_t panel = (static_cast<size_t>(expert) * g.rows_per_expert + wrow0) >> 4;
+        w_tile[f] = g.w_nib + (panel * chunks * 64 + lane) * 16;
+        s_tile[f] = g.w_sc + panel * chunks * 64 + lane;
     }
     BSet<MT, NT> bs[D];
     auto load_b = [&](int set, int c) {
-        // Block g of chunk c; lanes whose block lies past K (tail or dead chunk) read block 0 and are masked.
-        const int kb = c * 4 + grp;
-        const bool valid = kb * 32 < K;
-        const int kbc = valid ? kb : 0;
+        // Dead chunks (past the padded K) re-read the last chunk; compute() zeroes them.
+        // (Masking here, next to the loads, would make the wave wait for data it has only just requested.)
+        bs[set].valid = c < chunks;
+        const int cc = min(c, chunks - 1);
 #pragma unroll
         for (int f = 0; f < NT; ++f) {
-            mu32x4 q = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_row[f] + kbc * 16));
-            uint32_t s = __builtin_nontemporal_load(s_row[f] + kbc);
-            const mu32x4 zero = {0, 0, 0, 0};
-            bs[set].q[f] = valid ? q : zero;
-            bs[set].s[f] = valid ? s : 127u;
+            bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
+            bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
         }
     };
 
@@ -311,30 +345,57 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
 #pragma unroll
         for (int f = 0; f < NT; ++f) acc[i][f] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    // One row fragment of activations: fp8 hi and lo operands and the scale byte.
+    struct AFrag {
+        mu32x4 h0, h1, l0, l1;
+        uint32_t sw;
+    };
+    auto load_frag = [&](const unsigned char *base, int i) {
+        const unsigned char *p = base + (i * 16 + r) * kARow + grp * 16;
+        AFrag a;
+        a.h0 = *reinterpret_cast<const mu32x4 *>(p);
+        a.h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
+        a.l0 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE);
+        a.l1 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE + 64);
+        a.sw = *reinterpret_cast<const uint32_t *>(base + 2 * A_PLANE + (i * 16 + r) * 4);
+        return a;
+    };
     auto compute = [&](int set, int buf) {
         const unsigned char *base = lds + buf * A_BUF;
-        const unsigned char *ap = base + r * kARow + grp * 16;
+        mu32x4 bq[NT];
+        int bsc[NT];
 #pragma unroll
-        for (int f = 0; f < NT; ++f) asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
+        for (int f = 0; f < NT; ++f) {
+            asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
+            const mu32x4 zero = {0, 0, 0, 0};
+            bq[f] = bs[set].valid ? bs[set].q[f] : zero;
+            bsc[f] = bs[set].valid ? static_cast<int>(bs[set].s[f]) : 127;
+        }
+        // The LDS reads of fragment i+1 are issued before the MFMAs of fragment i and
+        // fenced there, so two fragments are live at a time instead of all MT.
+        AFrag cur = load_frag(base, 0);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            const unsigned char *p = ap + i * 16 * kARow;
-            const mu32x4 h0 = *reinterpret_cast<const mu32x4 *>(p);
-            const mu32x4 h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
-            const mu32x4 l0 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE);
-            const mu32x4 l1 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE + 64);
-            const uint32_t sw = *reinterpret_cast<const uint32_t *>(base + 2 * A_PLANE + (i * 16 + r) * 4);
-            const int sa = static_cast<int>((sw >> (8 * grp)) & 0xff);
-            const v8i ah = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
-            const v8i al = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
+            AFrag nxt = cur;
+            if (i + 1 < MT) nxt = load_frag(base, i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const int sa = static_cast<int>((cur.sw >> (8 * grp)) & 0xff);
+            const v8i ah = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
+                            (int)cur.h1.x, (int)cur.h1.y, (int)cur.h1.z, (int)cur.h1.w};
+            const v8i al = {(int)cur.l0.x, (int)cur.l0.y, (int)cur.l0.z, (int)cur.l0.w,
+                            (int)cur.l1.x, (int)cur.l1.y, (int)cur.l1.z, (int)cur.l1.w};
 #pragma unroll
             for (int f = 0; f < NT; ++f) {
-                const mu32x4 q = bs[set].q[f];
-                const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
-                const int sb = static_cast<int>(bs[set].s[f]);
-                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, sb);
-                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+                const v8i b = {(int)bq[f].x, (int)bq[f].y, (int)bq[f].z, (int)bq[f].w, 0, 0, 0, 0};
+                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, bsc[f]);
+                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, bsc[f]);
+                // Pin the accumulation here: nothing else reads acc until the epilogue, and
+                // without this the optimiser sinks every MFMA of the unrolled pipeline to its
+                // end, keeping the fragments of all its steps alive.
+                asm volatile("" : "+a"(acc[i][f]));
             }
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
         }
     };
 
@@ -465,7 +526,7 @@ static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max
 static lhip_status check_moe_shape(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
     if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return LHIP_ERR_INVALID_SHAPE;
     if (E > 1024 || topk > E || T * topk > (int64_t{1} << 24)) return LHIP_ERR_INVALID_SHAPE;
-    if (H % 32 != 0 || I % 32 != 0 || H > kMaxDim || I > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (H % 32 != 0 || I % 32 != 0 || H > kMaxDim || I > kMaxDim) return LHIP_ERR_INVALID_SHAPE;  // so % 16 == 0 too
     return LHIP_OK;
 }
 
@@ -479,8 +540,14 @@ lhip_status lhip_moe_route_topk(const float *logits_dev, int32_t *sel_dev, float
                                 int64_t topk, void *stream) {
     if (!logits_dev || !sel_dev || !wts_dev) return LHIP_ERR_NULL_PTR;
     if (t <= 0 || e <= 0 || topk <= 0 || topk > e || t > kMaxDim || e > 1024) return LHIP_ERR_INVALID_SHAPE;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((t + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       logits_dev, static_cast<int>(t), static_cast<int>(e), static_cast<int>(topk), sel_dev, wts_dev);
+    if (e <= 64 && topk <= 64)
+        hipLaunchKernelGGL(moe_route_wave_kernel, dim3(static_cast<unsigned>((t + 3) / 4)), dim3(256), 0,
+                           as_stream(stream), logits_dev, static_cast<int>(t), static_cast<int>(e),
+                           static_cast<int>(topk), sel_dev, wts_dev);
+    else
+        hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((t + 255) / 256)), dim3(256), 0,
+                           as_stream(stream), logits_dev, static_cast<int>(t), static_cast<int>(e),
+                           static_cast<int>(topk), sel_dev, wts_dev);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }

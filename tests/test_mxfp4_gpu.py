@@ -33,10 +33,19 @@ def test_repack_round_trip_and_layout(n, k):
     raw = synth.mxfp4_raw_blocks(codes, scales)
     w = Mxfp4Weight.from_raw(raw, n, k, DEV)
     planar = w.planar.cpu().numpy()
-    off = capi.load_library().lhip_mxfp4_planar_scale_offset(n, k)
-    nib = planar[: n * k // 2].reshape(n, k // 2)
-    assert np.array_equal(nib & 15, codes[:, 0::2]) and np.array_equal(nib >> 4, codes[:, 1::2])
-    assert np.array_equal(planar[off:off + n * k // 32].reshape(n, k // 32), scales)
+    lib = capi.load_library()
+    off = lib.lhip_mxfp4_planar_scale_offset(n, k)
+    panels, chunks = (n + 15) // 16, (k + 127) // 128
+    assert off == panels * chunks * 1024 and planar.size == off + panels * chunks * 64
+    # tiled order: piece (panel, chunk, g, r) holds block (chunk*4+g) of row (panel*16+r); padding = 0 / scale 127
+    nib = planar[:off].reshape(panels, chunks, 4, 16, 16)
+    sc = planar[off:].reshape(panels, chunks, 4, 16)
+    want_nib = np.zeros((panels * 16, chunks * 4, 16), np.uint8)
+    want_sc = np.full((panels * 16, chunks * 4), 127, np.uint8)
+    want_nib[:n, : k // 32] = (codes[:, 0::2] | (codes[:, 1::2] << 4)).reshape(n, k // 32, 16)
+    want_sc[:n, : k // 32] = scales
+    assert np.array_equal(nib, want_nib.reshape(panels, 16, chunks, 4, 16).transpose(0, 2, 3, 1, 4))
+    assert np.array_equal(sc, want_sc.reshape(panels, 16, chunks, 4).transpose(0, 2, 3, 1))
     assert np.array_equal(w.to_raw().cpu().numpy(), raw)
 
 
@@ -62,6 +71,12 @@ def test_router_matches_oracle(oracle):
     assert np.array_equal(sel.cpu().numpy(), osel)
     assert np.allclose(wts.cpu().numpy(), owts, rtol=2e-6, atol=0)
     assert list(sel[7].cpu().numpy()) == [0, 1, 2, 3]
+    # more experts than a wavefront has lanes: the per-thread kernel
+    big = rng.standard_normal((50, 100)).astype(np.float32)
+    sel, wts = route_topk(torch.from_numpy(big).to(DEV), 6)
+    osel, owts = oracle.moe_route(big, 6)
+    assert np.array_equal(sel.cpu().numpy(), osel)
+    assert np.allclose(wts.cpu().numpy(), owts, rtol=2e-6, atol=0)
 
 
 def make_layer(oracle, e, h, i, seed):
