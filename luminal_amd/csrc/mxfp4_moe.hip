@@ -222,8 +222,8 @@ __global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__re
 // ---------------------------------------------------------------------------
 // Grouped expert GEMM.  grid = (column blocks, max tiles); a workgroup of 4 waves
 // owns one row tile (up to BM = 16*MT routed rows of one expert) and 4*NT column
-// fragments of 16.  GATED: NT == 2, fragment 0 = gate rows, fragment 1 = the
-// matching up rows, output bf16 up*swish(gate).  Otherwise f32 output.
+// fragments of 16.  GATED: fragments come in pairs, gate rows and the matching
+// up rows, output bf16 up*swish(gate).  Otherwise f32 output.
 // ---------------------------------------------------------------------------
 struct MoeGemmArgs {
     const uint8_t *a_hi, *a_lo, *a_sc;  // activation planes, row stride Kp / Kp/32
@@ -246,7 +246,7 @@ struct BSet {
 
 template <int MT, int NT, bool GATED>
 __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
-    static_assert(!GATED || NT == 2, "gated tiles pair one gate fragment with one up fragment");
+    static_assert(!GATED || NT % 2 == 0, "gated tiles pair each gate fragment with its up fragment");
     constexpr int BM = 16 * MT;
     constexpr int D = 4;  // weight prefetch distance in chunks
     constexpr int A_PLANE = BM * kARow;
@@ -277,9 +277,9 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
 #pragma unroll
     for (int f = 0; f < NT; ++f) {
         int n0, wrow0;  // first column of the fragment, first weight row inside the expert
-        if (GATED) {
-            n0 = (blockIdx.x * 4 + wave) * 16;  // i index
-            wrow0 = (f == 0 ? 0 : g.N) + min(n0, g.N - 16);
+        if (GATED) {  // fragments 2p / 2p+1 = gate / up rows of the same 16 intermediate columns
+            n0 = ((blockIdx.x * 4 + wave) * (NT / 2) + (f >> 1)) * 16;
+            wrow0 = ((f & 1) ? g.N : 0) + min(n0, g.N - 16);
         } else {
             n0 = ((blockIdx.x * 4 + wave) * NT + f) * 16;
             wrow0 = min(n0, g.N - 16);
@@ -428,17 +428,165 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
             if (m >= rows) continue;
             const size_t orow = static_cast<size_t>(row0 + m) * g.N;
             if (GATED) {
-                if (col[0] < g.N) {
-                    const float gate = acc[i][0][v], up = acc[i][1][v];
-                    const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
-                    static_cast<__bf16 *>(g.out)[orow + col[0]] = static_cast<__bf16>(act);
-                }
+#pragma unroll
+                for (int p = 0; p < NT / 2; ++p)
+                    if (col[2 * p] < g.N) {
+                        const float gate = acc[i][2 * p][v], up = acc[i][2 * p + 1][v];
+                        const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                        static_cast<__bf16 *>(g.out)[orow + col[2 * p]] = static_cast<__bf16>(act);
+                    }
             } else {
 #pragma unroll
                 for (int f = 0; f < NT; ++f)
                     if (col[f] < g.N) static_cast<float *>(g.out)[orow + col[f]] = acc[i][f][v];
             }
         }
+}
+
+// ---------------------------------------------------------------------------
+// Decode-sized variant: row tiles of at most 16 routed rows (one row fragment).
+// The tile's whole quantised activation rows (all of K) are staged in LDS once,
+// so the K loop is nothing but the weight stream — no activation loads, no
+// barriers — with D = 8 chunks of weights in flight per wave.  Needs
+// 2 * 16 * (Kp + 16) + 16 * Kp/32 bytes of LDS (K up to ~4.6k).
+// ---------------------------------------------------------------------------
+template <int NT, bool GATED>
+__global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
+    static_assert(!GATED || NT % 2 == 0, "gated tiles pair each gate fragment with its up fragment");
+    constexpr int D = 8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int tile = blockIdx.y;
+    if (tile >= *g.n_tiles) return;
+    const int expert = g.tile_expert[tile];
+    const int row0 = g.tile_row0[tile];
+    const int rows = g.tile_rows[tile];  // 1..16
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, grp = lane >> 4;
+    const int Kp = g.Kp;
+    const int chunks = Kp / kChunk;
+    const int steps = (chunks + D - 1) / D * D;
+    const int a_row = Kp + 16;             // LDS bytes per activation row (padded against bank conflicts)
+    const int a_plane = 16 * a_row;
+    const int sc_row = Kp / 32;            // scale bytes per row
+    unsigned char *lds_sc = lds + 2 * a_plane;
+
+    const uint8_t *w_tile[NT];
+    const uint8_t *s_tile[NT];
+    int col[NT];
+#pragma unroll
+    for (int f = 0; f < NT; ++f) {
+        int n0, wrow0;
+        if (GATED) {
+            n0 = ((blockIdx.x * 4 + wave) * (NT / 2) + (f >> 1)) * 16;
+            wrow0 = ((f & 1) ? g.N : 0) + min(n0, g.N - 16);
+        } else {
+            n0 = ((blockIdx.x * 4 + wave) * NT + f) * 16;
+            wrow0 = min(n0, g.N - 16);
+        }
+        col[f] = n0 + r;
+        const size_t panel = (static_cast<size_t>(expert) * g.rows_per_expert + wrow0) >> 4;
+        w_tile[f] = g.w_nib + (panel * chunks * 64 + lane) * 16;
+        s_tile[f] = g.w_sc + panel * chunks * 64 + lane;
+    }
+    BSet<1, NT> bs[D];
+    auto load_b = [&](int set, int c) {
+        bs[set].valid = c < chunks;
+        const int cc = min(c, chunks - 1);
+#pragma unroll
+        for (int f = 0; f < NT; ++f) {
+            bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
+            bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+        }
+    };
+    // Weights first: their HBM round trip overlaps the staging of the activations.
+#pragma unroll
+    for (int j = 0; j < D; ++j) load_b(j, j);
+
+    {
+        const int per_row = Kp / 16;  // 16-byte pieces per row and plane
+        const int pieces = rows * per_row * 2;
+        for (int q = tid; q < pieces; q += 256) {
+            const int plane = q / (rows * per_row), rem = q - plane * (rows * per_row);
+            const int row = rem / per_row, c16 = rem - row * per_row;
+            const int slot = row0 + row;
+            const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
+            const mu32x4 v = *reinterpret_cast<const mu32x4 *>((plane ? g.a_lo : g.a_hi) +
+                                                                static_cast<size_t>(arow) * Kp + c16 * 16);
+            *reinterpret_cast<mu32x4 *>(lds + plane * a_plane + row * a_row + c16 * 16) = v;
+        }
+        const int sc_words = rows * (sc_row / 4);
+        for (int q = tid; q < sc_words; q += 256) {
+            const int row = q / (sc_row / 4), w4 = q - row * (sc_row / 4);
+            const int slot = row0 + row;
+            const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
+            reinterpret_cast<uint32_t *>(lds_sc + row * sc_row)[w4] =
+                reinterpret_cast<const uint32_t *>(g.a_sc + static_cast<size_t>(arow) * sc_row)[w4];
+        }
+    }
+    __syncthreads();
+
+    v4f acc[NT];
+#pragma unroll
+    for (int f = 0; f < NT; ++f) acc[f] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // Rows past the tile hold stale LDS bytes; their results are never stored.
+    const unsigned char *ap = lds + r * a_row + grp * 16;
+    const unsigned char *sp = lds_sc + r * sc_row + grp;
+    auto compute = [&](int set, int c) {
+        const int cc = min(c, chunks - 1);
+        const unsigned char *p = ap + cc * kChunk;
+        const mu32x4 h0 = *reinterpret_cast<const mu32x4 *>(p);
+        const mu32x4 h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
+        const mu32x4 l0 = *reinterpret_cast<const mu32x4 *>(p + a_plane);
+        const mu32x4 l1 = *reinterpret_cast<const mu32x4 *>(p + a_plane + 64);
+        const int sa = sp[cc * 4];
+        const v8i ah = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
+        const v8i al = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
+#pragma unroll
+        for (int f = 0; f < NT; ++f) {
+            asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
+            const mu32x4 zero = {0, 0, 0, 0};
+            const mu32x4 q = bs[set].valid ? bs[set].q[f] : zero;
+            const int sb = bs[set].valid ? static_cast<int>(bs[set].s[f]) : 127;
+            const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
+            acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[f], 0, 4, 0, sa, 0, sb);
+            acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[f], 0, 4, 0, sa, 0, sb);
+            asm volatile("" : "+a"(acc[f]));
+        }
+    };
+    for (int c0 = 0; c0 < steps; c0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            compute(j, c0 + j);
+            __builtin_amdgcn_sched_barrier(0);
+            load_b(j, c0 + j + D);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int m = 4 * grp + v;
+        if (m >= rows) continue;
+        const size_t orow = static_cast<size_t>(row0 + m) * g.N;
+        if (GATED) {
+#pragma unroll
+            for (int p = 0; p < NT / 2; ++p)
+                if (col[2 * p] < g.N) {
+                    const float gate = acc[2 * p][v], up = acc[2 * p + 1][v];
+                    const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                    static_cast<__bf16 *>(g.out)[orow + col[2 * p]] = static_cast<__bf16>(act);
+                }
+        } else {
+#pragma unroll
+            for (int f = 0; f < NT; ++f)
+                if (col[f] < g.N) static_cast<float *>(g.out)[orow + col[f]] = acc[f][v];
+        }
+    }
 }
 
 // y[t][h] = bf16( sum_s wts[t][s] * out[slot_of[t*topk+s]][h] ), 4 columns per thread
@@ -523,6 +671,21 @@ static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max
     return LHIP_OK;
 }
 
+static inline size_t moe_small_lds_bytes(int Kp) { return 2 * 16 * static_cast<size_t>(Kp + 16) + 16 * (Kp / 32); }
+
+template <int NT, bool GATED>
+static lhip_status launch_moe_gemm_small(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
+    const size_t lds_bytes = moe_small_lds_bytes(a.Kp);
+    auto kern = mx_moe_gemm_small_kernel<NT, GATED>;
+    if (lds_bytes > 64 * 1024)
+        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256),
+                       lds_bytes, s, a);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
 static lhip_status check_moe_shape(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
     if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return LHIP_ERR_INVALID_SHAPE;
     if (E > 1024 || topk > E || T * topk > (int64_t{1} << 24)) return LHIP_ERR_INVALID_SHAPE;
@@ -578,6 +741,10 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     const int mt = avg > 64 ? 8 : (avg > 32 ? 4 : (avg > 16 ? 2 : 1));
     const int BM = 16 * mt;
     const int max_tiles = R / BM + E;
+    // A handful of routed rows in total (batch-1 decode and the like): stage each tile's
+    // activation rows whole and run the barrier-free weight stream.  With more rows per expert
+    // that staging costs more than it saves (measured at T = 64: 168 us against 108 us).
+    const bool decode_sized = R <= 4 * E / 2;
 
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel_dev, R, E, BM, w.plan);
     LHIP_CHECK_LAUNCH();
@@ -597,13 +764,19 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
     a1.n_tiles = w.plan.n_tiles; a1.out = w.act;
-    const int cb1 = (I + 63) / 64;  // 4 waves x 16 gate/up pairs
+    // Column blocks: 4 waves x (NT/2) gate/up pairs of 16.  Tall row tiles take 4 weight
+    // fragments per wave, so each activation fragment read from LDS feeds twice the MFMAs.
+    const int cb1 = (I + 63) / 64, cb1w = (I + 127) / 128;
     lhip_status st;
     switch (mt) {
-        case 1: st = launch_moe_gemm<1, 2, true>(a1, cb1, max_tiles, s); break;
+        case 1:
+            st = decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024
+                     ? launch_moe_gemm_small<2, true>(a1, cb1, max_tiles, s)
+                                                       : launch_moe_gemm<1, 2, true>(a1, cb1, max_tiles, s);
+            break;
         case 2: st = launch_moe_gemm<2, 2, true>(a1, cb1, max_tiles, s); break;
-        case 4: st = launch_moe_gemm<4, 2, true>(a1, cb1, max_tiles, s); break;
-        default: st = launch_moe_gemm<8, 2, true>(a1, cb1, max_tiles, s); break;
+        case 4: st = launch_moe_gemm<4, 4, true>(a1, cb1w, max_tiles, s); break;
+        default: st = launch_moe_gemm<8, 4, true>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
     {
@@ -620,13 +793,15 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a2.tile_expert = w.plan.tile_expert; a2.tile_row0 = w.plan.tile_row0; a2.tile_rows = w.plan.tile_rows;
     a2.n_tiles = w.plan.n_tiles; a2.out = w.out;
     if (mt == 1) {
-        st = launch_moe_gemm<1, 1, false>(a2, (H + 63) / 64, max_tiles, s);
+        st = decode_sized && moe_small_lds_bytes(Ip) <= 150 * 1024
+                 ? launch_moe_gemm_small<1, false>(a2, (H + 63) / 64, max_tiles, s)
+                                                   : launch_moe_gemm<1, 1, false>(a2, (H + 63) / 64, max_tiles, s);
     } else {
-        const int cb2 = (H + 127) / 128;  // 4 waves x 2 fragments of 16
+        const int cb2 = (H + 127) / 128, cb2w = (H + 255) / 256;  // 4 waves x NT fragments of 16
         switch (mt) {
             case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
-            case 4: st = launch_moe_gemm<4, 2, false>(a2, cb2, max_tiles, s); break;
-            default: st = launch_moe_gemm<8, 2, false>(a2, cb2, max_tiles, s); break;
+            case 4: st = launch_moe_gemm<4, 4, false>(a2, cb2w, max_tiles, s); break;
+            default: st = launch_moe_gemm<8, 4, false>(a2, cb2w, max_tiles, s); break;
         }
     }
     if (st) return st;
