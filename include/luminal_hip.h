@@ -165,6 +165,46 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
                                 const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                 int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream);
 
+/* ---- the operators around the matmuls in the Llama-3 decode loop (f32) --------
+ * What the reference assembles from primitive ops in examples/llama/src/model.rs,
+ * as single kernels.  Positions live in device memory (pos_dev) so that a decode
+ * step can be captured in a HIP graph and replayed. */
+
+/* out[t][:] = table[(int)idx[t]][:]; fp32 embedding lookup with ids carried as f32
+ * (crates/luminal_nn/src/embedding.rs:40-58, crates/luminal_cpu/src/binary.rs:175-191).
+ * dim % 4 == 0; an id outside [0, n_rows) gives a zero row. */
+lhip_status lhip_gather_rows_f32(const float *table_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
+                                 int64_t n_rows, int64_t dim, void *stream);
+/* RMS norm as luminal's LayerNorm(mean_norm = false): y = v * 1/sqrt(mean(v^2) + eps) * w
+ * (crates/luminal_nn/src/norm.rs:56-71, src/hl_ops/unary.rs:93-104).  With residual_dev
+ * given, v = x + residual and v is also written to x_out_dev (the residual adds of
+ * model.rs:173-187 fused into the norm that follows them); otherwise v = x. */
+lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
+                              float *y_dev, int64_t rows, int64_t dim, float eps, void *stream);
+/* Rotary embedding (adjacent pairs, model.rs:52-72) applied in place to the q and k heads
+ * of fused rows qkv[tokens][(q_heads + 2*kv_heads)*head_dim] at positions *pos_dev + t, then
+ * k and v appended to the caches [kv_heads][max_seq][head_dim] (model.rs:108-110). */
+lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v_cache_dev, const int32_t *pos_dev,
+                                    int64_t tokens, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
+                                    int64_t max_seq, float theta, void *stream);
+/* Causal grouped-query attention of the q heads in qkv over the caches (model.rs:112-139):
+ * out[tokens][q_heads*head_dim].  head_dim <= 256, max_seq <= 16000. */
+lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
+                               float *out_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
+                               int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
+/* out[r][j] = up * swish(gate) with gate = gate_up[r][j], up = gate_up[r][f + j] (model.rs:24-32). */
+lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, void *stream);
+/* Element-wise casts between f32 and bf16 (round to nearest even), for feeding f32
+ * activations to the bf16 prefill GEMM. */
+lhip_status lhip_cast_f32_to_bf16(const float *x_dev, void *y_dev, int64_t n, void *stream);
+lhip_status lhip_cast_bf16_to_f32(const void *x_dev, float *y_dev, int64_t n, void *stream);
+/* x += y */
+lhip_status lhip_add_f32(float *x_dev, const float *y_dev, int64_t n, void *stream);
+/* Greedy pick (examples/llama/src/main.rs:194-198; the last index wins exact ties): the index
+ * goes to *id_f32_dev and/or *id_i32_dev, and *pos_dev (if given) is advanced by `advance`. */
+lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                            int32_t advance, void *stream);
+
 /* ---- calibration kernels ---------------------------------------------------
  * No counterpart in the reference.  A plain device-to-device copy and a
  * read-only pass with known byte counts, used to calibrate hardware counters

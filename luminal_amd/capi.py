@@ -47,6 +47,15 @@ SIGNATURES = {
     "lhip_moe_route_topk": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_mxfp4_moe_workspace_nbytes": (_sz, [_i64] * 5),
     "lhip_mxfp4_moe_bf16": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp, _vp]),
+    "lhip_gather_rows_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_rms_norm_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
+    "lhip_rope_kv_append_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp]),
+    "lhip_attention_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "lhip_swiglu_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_cast_f32_to_bf16": (C.c_int32, [_vp, _vp, _i64, _vp]),
+    "lhip_cast_bf16_to_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),
+    "lhip_add_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),
+    "lhip_argmax_f32": (C.c_int32, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _vp]),
     "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
     "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),
 }

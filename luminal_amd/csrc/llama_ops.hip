@@ -1,0 +1,332 @@
+// The non-matmul operators of the Llama-3 decode loop, in f32, so that a
+// Q8_0 model can run end to end on the device around the quantized matmuls.
+// Each restates what the reference builds from primitive ops
+// (examples/llama/src/model.rs; crates/luminal_nn/src/norm.rs:56-71;
+// src/hl_ops/unary.rs:93-104,126-130,169-177).  They are small, memory-bound
+// and written for correctness first: at batch 1 more than 95 % of the bytes a
+// decode step touches are the quantized weights.
+//
+// Positions are read from device memory (`pos_dev`), so a whole decode step can
+// be captured once in a HIP graph and replayed while the position advances on
+// the device.
+#include "common.h"
+
+namespace lhip {
+
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();  // protect red against the previous use
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) t += red[w];
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float *red) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int w = 1; w < static_cast<int>(blockDim.x >> 6); ++w) t = fmaxf(t, red[w]);
+    return t;
+}
+
+// out[t][:] = table[(int)idx[t]][:]   (Embedding / CPU Gather, crates/luminal_cpu/src/binary.rs:175-191)
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float4 *__restrict__ table,
+                                                          const float *__restrict__ idx, float4 *__restrict__ out,
+                                                          int n_rows, int dim4) {
+    const int t = blockIdx.x;
+    const float fi = idx[t];
+    const long row = (fi >= 0.0f && fi < 2147483648.0f) ? static_cast<long>(fi) : -1;
+    float4 *o = out + static_cast<size_t>(t) * dim4;
+    for (int j = threadIdx.x; j < dim4; j += 256)
+        o[j] = (row >= 0 && row < n_rows) ? table[static_cast<size_t>(row) * dim4 + j] : make_float4(0, 0, 0, 0);
+}
+
+// y = (x [+ res]) * 1/sqrt(mean(x^2) + eps) * w ; if res is given, x_out receives x + res
+// (LayerNorm with mean_norm = false: std_norm then weight, norm.rs:56-71, unary.rs:93-104).
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ res,
+                                                       float *__restrict__ x_out, const float *__restrict__ w,
+                                                       float *__restrict__ y, int dim, float eps) {
+    __shared__ float red[4];
+    const size_t base = static_cast<size_t>(blockIdx.x) * dim;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < dim; j += 256) {
+        float v = x[base + j];
+        if (res) {
+            v += res[base + j];
+            x_out[base + j] = v;
+        }
+        ss += v * v;
+    }
+    const float total = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+    for (int j = threadIdx.x; j < dim; j += 256) {
+        const float v = res ? x_out[base + j] : x[base + j];
+        y[base + j] = v * scale * w[j];
+    }
+}
+
+// Rotary embedding on adjacent pairs (the ggml layout of model.rs:52-72) for the q and k
+// parts of a fused qkv row, then k and v are appended to the cache at position pos0 + s.
+// qkv: [S][(hq + 2*hkv) * hd]; caches: [hkv][max_seq][hd].  One block per (token, head).
+__global__ __launch_bounds__(64) void rope_kv_kernel(float *__restrict__ qkv, float *__restrict__ k_cache,
+                                                     float *__restrict__ v_cache, const int *__restrict__ pos_dev,
+                                                     int hq, int hkv, int hd, int max_seq, float theta) {
+    const int s = blockIdx.x, head = blockIdx.y;  // head in [0, hq + 2*hkv)
+    const int pos = *pos_dev + s;
+    float *row = qkv + (static_cast<size_t>(s) * (hq + 2 * hkv) + head) * hd;
+    const int half = hd / 2;
+    if (head < hq + hkv) {  // q or k: rotate
+        for (int j = threadIdx.x; j < half; j += 64) {
+            const float inv_freq = 1.0f / powf(theta, static_cast<float>(2 * j) / static_cast<float>(hd));
+            const float ang = static_cast<float>(pos) * inv_freq;
+            float sn, cs;
+            sincosf(ang, &sn, &cs);
+            const float x0 = row[2 * j], x1 = row[2 * j + 1];
+            const float y0 = x0 * cs - x1 * sn, y1 = x0 * sn + x1 * cs;
+            row[2 * j] = y0;
+            row[2 * j + 1] = y1;
+            if (head >= hq && pos < max_seq) {
+                float *kc = k_cache + (static_cast<size_t>(head - hq) * max_seq + pos) * hd;
+                kc[2 * j] = y0;
+                kc[2 * j + 1] = y1;
+            }
+        }
+    } else if (pos < max_seq) {  // v: copy
+        float *vc = v_cache + (static_cast<size_t>(head - hq - hkv) * max_seq + pos) * hd;
+        for (int j = threadIdx.x; j < hd; j += 64) vc[j] = row[j];
+    }
+}
+
+// Causal grouped-query attention for S query tokens at positions pos0 .. pos0+S-1 over the
+// cache (model.rs:112-139): scores = q.k / sqrt(hd), masked positions get f16::MIN added (they
+// vanish in the softmax, so they are skipped), softmax, times V.  One block per (token, q head).
+// q is read from the fused qkv rows; out: [S][hq*hd].  Dynamic LDS: (pos0 + S) floats.
+__global__ __launch_bounds__(256) void attention_kernel(const float *__restrict__ qkv, const float *__restrict__ k_cache,
+                                                        const float *__restrict__ v_cache, float *__restrict__ out,
+                                                        const int *__restrict__ pos_dev, int hq, int hkv, int hd,
+                                                        int max_seq) {
+    extern __shared__ float sc[];  // scores of this query
+    __shared__ float red[4];
+    __shared__ float qs[256];
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int n_keys = min(*pos_dev + s + 1, max_seq);
+    const int kvh = h / (hq / hkv);
+    const float *q = qkv + (static_cast<size_t>(s) * (hq + 2 * hkv) + h) * hd;
+    for (int j = threadIdx.x; j < hd; j += 256) qs[j] = q[j];
+    __syncthreads();
+    const float *kc = k_cache + static_cast<size_t>(kvh) * max_seq * hd;
+    const float *vc = v_cache + static_cast<size_t>(kvh) * max_seq * hd;
+    const float inv_sqrt = 1.0f / sqrtf(static_cast<float>(hd));
+    // one wave per key: 64 lanes cover hd (<= 256) elements
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mx = -3.0e38f;
+    for (int p = wave; p < n_keys; p += 4) {
+        float d = 0.f;
+        for (int j = lane; j < hd; j += 64) d += qs[j] * kc[static_cast<size_t>(p) * hd + j];
+        for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o);
+        d *= inv_sqrt;
+        if (lane == 0) sc[p] = d;
+        mx = fmaxf(mx, d);
+    }
+    mx = block_max(mx, red);
+    float sum = 0.f;
+    for (int p = threadIdx.x; p < n_keys; p += 256) {
+        const float e = expf(sc[p] - mx);
+        sc[p] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, red);
+    const float inv = 1.0f / sum;
+    float *o = out + (static_cast<size_t>(s) * hq + h) * hd;
+    for (int j = threadIdx.x; j < hd; j += 256) {
+        float a = 0.f;
+        for (int p = 0; p < n_keys; ++p) a += sc[p] * vc[static_cast<size_t>(p) * hd + j];
+        o[j] = a * inv;
+    }
+}
+
+// out[s][j] = up * swish(gate), gate = gu[s][j], up = gu[s][f + j]   (model.rs:24-32)
+__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gu, float *__restrict__ out, int f,
+                                                     size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const size_t s = i / f;
+    const int j = static_cast<int>(i - s * f);
+    const float g = gu[s * 2 * f + j], u = gu[s * 2 * f + f + j];
+    out[i] = u * (g * (1.0f / (1.0f + expf(-g))));
+}
+
+__global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ y,
+                                                            size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) y[i] = static_cast<__bf16>(x[i]);  // round to nearest even
+}
+
+__global__ __launch_bounds__(256) void cast_bf16_f32_kernel(const __bf16 *__restrict__ x, float *__restrict__ y,
+                                                            size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) y[i] = static_cast<float>(x[i]);
+}
+
+__global__ __launch_bounds__(256) void add_kernel(float *__restrict__ x, const float *__restrict__ y, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) x[i] += y[i];
+}
+
+// Greedy pick: index of the largest value; on exact ties the last one, as itertools'
+// position_max_by does in the reference's loop (examples/llama/src/main.rs:194-198).  The
+// index is written as f32 (token ids travel as f32 in luminal) and as int32, and the position
+// counter is advanced by `advance`.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ x, int n, float *__restrict__ id_f32,
+                                                      int *__restrict__ id_i32, int *__restrict__ pos_dev,
+                                                      int advance) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    float v = -3.4e38f;
+    int idx = -1;
+    for (int j = threadIdx.x; j < n; j += 1024) {
+        const float c = x[j];
+        if (idx < 0 || c >= v) {  // j increases, so >= keeps the last of equals
+            v = c;
+            idx = j;
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o);
+        const int oi = __shfl_xor(idx, o);
+        if (oi >= 0 && (idx < 0 || ov > v || (ov == v && oi > idx))) {
+            v = ov;
+            idx = oi;
+        }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        bv[wave] = v;
+        bi[wave] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (bi[w] >= 0 && (bi[0] < 0 || bv[w] > bv[0] || (bv[w] == bv[0] && bi[w] > bi[0]))) {
+                bv[0] = bv[w];
+                bi[0] = bi[w];
+            }
+        if (id_f32) *id_f32 = static_cast<float>(bi[0]);
+        if (id_i32) *id_i32 = bi[0];
+        if (pos_dev) *pos_dev += advance;
+    }
+}
+
+}  // namespace lhip
+
+using namespace lhip;
+
+extern "C" {
+
+lhip_status lhip_gather_rows_f32(const float *table_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
+                                 int64_t n_rows, int64_t dim, void *stream) {
+    if (!table_dev || !idx_dev || !out_dev) return LHIP_ERR_NULL_PTR;
+    if (n_idx <= 0 || n_rows <= 0 || dim <= 0 || dim % 4 != 0 || n_idx > kMaxDim || n_rows > kMaxDim || dim > kMaxDim)
+        return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(table_dev, 16) || !aligned(out_dev, 16)) return LHIP_ERR_MISALIGNED;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(static_cast<unsigned>(n_idx)), dim3(256), 0, as_stream(stream),
+                       reinterpret_cast<const float4 *>(table_dev), idx_dev, reinterpret_cast<float4 *>(out_dev),
+                       static_cast<int>(n_rows), static_cast<int>(dim / 4));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
+                              float *y_dev, int64_t rows, int64_t dim, float eps, void *stream) {
+    if (!x_dev || !w_dev || !y_dev || (residual_dev && !x_out_dev)) return LHIP_ERR_NULL_PTR;
+    if (rows <= 0 || dim <= 0 || rows > kMaxDim || dim > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, as_stream(stream), x_dev,
+                       residual_dev, x_out_dev, w_dev, y_dev, static_cast<int>(dim), eps);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v_cache_dev, const int32_t *pos_dev,
+                                    int64_t tokens, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
+                                    int64_t max_seq, float theta, void *stream) {
+    if (!qkv_dev || !k_cache_dev || !v_cache_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
+    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 2 != 0 || max_seq <= 0 ||
+        q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads + 2 * kv_heads > 65535 || max_seq > kMaxDim)
+        return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(rope_kv_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads + 2 * kv_heads)),
+                       dim3(64), 0, as_stream(stream), qkv_dev, k_cache_dev, v_cache_dev, pos_dev,
+                       static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
+                       static_cast<int>(max_seq), theta);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
+                               float *out_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
+                               int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream) {
+    if (!qkv_dev || !k_cache_dev || !v_cache_dev || !out_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
+    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || max_seq <= 0 ||
+        q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 16000)
+        return LHIP_ERR_INVALID_SHAPE;  // the score row of one query lives in LDS
+    hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)), dim3(256),
+                       static_cast<size_t>(max_seq) * sizeof(float), as_stream(stream), qkv_dev, k_cache_dev,
+                       v_cache_dev, out_dev, pos_dev, static_cast<int>(q_heads), static_cast<int>(kv_heads),
+                       static_cast<int>(head_dim), static_cast<int>(max_seq));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, void *stream) {
+    if (!gate_up_dev || !out_dev) return LHIP_ERR_NULL_PTR;
+    if (rows <= 0 || f <= 0 || rows > kMaxDim || f > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    const size_t total = static_cast<size_t>(rows) * static_cast<size_t>(f);
+    hipLaunchKernelGGL(swiglu_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       gate_up_dev, out_dev, static_cast<int>(f), total);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_add_f32(float *x_dev, const float *y_dev, int64_t n, void *stream) {
+    if (!x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
+    if (n <= 0) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(add_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream), x_dev,
+                       y_dev, static_cast<size_t>(n));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_cast_f32_to_bf16(const float *x_dev, void *y_dev, int64_t n, void *stream) {
+    if (!x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
+    if (n <= 0) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), x_dev, static_cast<__bf16 *>(y_dev), static_cast<size_t>(n));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_cast_bf16_to_f32(const void *x_dev, float *y_dev, int64_t n, void *stream) {
+    if (!x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
+    if (n <= 0) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(cast_bf16_f32_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), static_cast<const __bf16 *>(x_dev), y_dev, static_cast<size_t>(n));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                            int32_t advance, void *stream) {
+    if (!x_dev || (!id_f32_dev && !id_i32_dev)) return LHIP_ERR_NULL_PTR;
+    if (n <= 0 || n > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x_dev, static_cast<int>(n), id_f32_dev,
+                       id_i32_dev, pos_dev, advance);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,220 @@
+"""Llama-3 decode loop over the luminal_hip C ABI.
+
+Host-side counterpart of examples/llama/src/{model.rs,main.rs}: the same layer
+stack and generation loop (prefill, then greedy decode with a KV cache), with
+every tensor op running in libluminal_hip.so.  torch holds the device buffers
+and, optionally, replays a captured HIP graph of one decode step.  Linear
+weights are Q8_0; q|k|v and gate|up are stored row-concatenated so each is one
+matvec (row-wise the same arithmetic as the reference's separate matmuls).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import capi
+from .quantized import Q8Weight
+
+
+@dataclass(frozen=True)
+class LlamaConfig:
+    """Constants of examples/llama/src/model.rs:5-14."""
+    vocab: int = 128256
+    dim: int = 4096
+    layers: int = 32
+    q_heads: int = 32
+    kv_heads: int = 8
+    ffn: int = 14336
+    eps: float = 1e-5
+    theta: float = 500000.0
+
+    @property
+    def head_dim(self) -> int:
+        return self.dim // self.q_heads
+
+    @property
+    def qkv_rows(self) -> int:
+        return (self.q_heads + 2 * self.kv_heads) * self.head_dim
+
+
+LLAMA3_8B = LlamaConfig()
+
+
+def _s() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+class LlamaQ8:
+    def __init__(self, cfg: LlamaConfig, weights: dict, max_seq: int, device="cuda:0"):
+        """weights: 'embed' f32 (vocab, dim); 'out_norm' f32 (dim); 'lm_head' Q8Weight (vocab, dim); and per
+        layer i: f'{i}.attn_norm', f'{i}.ffn_norm' f32 (dim); f'{i}.qkv' Q8Weight (qkv_rows, dim);
+        f'{i}.o' (dim, dim); f'{i}.gate_up' (2*ffn, dim); f'{i}.down' (dim, ffn)."""
+        self.cfg, self.w, self.max_seq, self.dev = cfg, weights, max_seq, torch.device(device)
+        self.lib = capi.load_library()
+        kv = (cfg.kv_heads, max_seq, cfg.head_dim)
+        self.k_cache = [torch.zeros(kv, dtype=torch.float32, device=self.dev) for _ in range(cfg.layers)]
+        self.v_cache = [torch.zeros(kv, dtype=torch.float32, device=self.dev) for _ in range(cfg.layers)]
+        self.pos = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        self.tok = torch.zeros(1, dtype=torch.float32, device=self.dev)      # next token id, as f32
+        self.tok_i = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        self._bufs = {}
+        self._graph = None
+
+    # ---- buffers -----------------------------------------------------------
+    def _buf(self, name, shape, dtype=torch.float32):
+        key = (name, tuple(shape), dtype)
+        if key not in self._bufs:
+            self._bufs[key] = torch.empty(shape, dtype=dtype, device=self.dev)
+        return self._bufs[key]
+
+    def reset(self):
+        self.pos.zero_()
+
+    # ---- ops ---------------------------------------------------------------
+    def _matmul(self, w: Q8Weight, x, y, m, bf16):
+        lib = self.lib
+        if not bf16:
+            capi.check(lib.lhip_q8_0_matmul_f32(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), m, w.n, w.k, _s()),
+                       "lhip_q8_0_matmul_f32")
+            return
+        xb = self._buf("xb", (m, w.k), torch.bfloat16)
+        yb = self._buf("yb", (m, w.n), torch.bfloat16)
+        capi.check(lib.lhip_cast_f32_to_bf16(x.data_ptr(), xb.data_ptr(), m * w.k, _s()), "cast")
+        capi.check(lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), xb.data_ptr(), yb.data_ptr(), m, w.n, w.k, _s()),
+                   "lhip_q8_0_matmul_bf16")
+        capi.check(lib.lhip_cast_bf16_to_f32(yb.data_ptr(), y.data_ptr(), m * w.n, _s()), "cast")
+
+    def _norm(self, x, res, x_out, w, y, rows):
+        capi.check(self.lib.lhip_rms_norm_f32(x.data_ptr(), res.data_ptr() if res is not None else None,
+                                              x_out.data_ptr() if x_out is not None else None, w.data_ptr(),
+                                              y.data_ptr(), rows, self.cfg.dim, self.cfg.eps, _s()), "lhip_rms_norm_f32")
+
+    def forward(self, tokens_f32: torch.Tensor, s: int, bf16: bool = False, all_logits: bool = False):
+        """Runs s tokens (ids as f32 on the device) at positions pos .. pos+s-1, appends to the KV cache and
+        returns the logits of the last position ((vocab,)), or of all positions ((s, vocab)).
+        Does not advance the position."""
+        cfg, lib, w = self.cfg, self.lib, self.w
+        d, hd = cfg.dim, cfg.head_dim
+        h = self._buf("h", (s, d))
+        n = self._buf("n", (s, d))
+        qkv = self._buf("qkv", (s, cfg.qkv_rows))
+        att = self._buf("att", (s, d))
+        o = self._buf("o", (s, d))
+        gu = self._buf("gu", (s, 2 * cfg.ffn))
+        act = self._buf("act", (s, cfg.ffn))
+        dn = self._buf("dn", (s, d))
+        capi.check(lib.lhip_gather_rows_f32(w["embed"].data_ptr(), tokens_f32.data_ptr(), h.data_ptr(), s, cfg.vocab,
+                                            d, _s()), "lhip_gather_rows_f32")
+        for i in range(cfg.layers):
+            if i == 0:
+                self._norm(h, None, None, w["0.attn_norm"], n, s)
+            else:  # residual of the previous layer's MLP, fused into this norm
+                self._norm(h, dn, h, w[f"{i}.attn_norm"], n, s)
+            self._matmul(w[f"{i}.qkv"], n, qkv, s, bf16)
+            capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                   self.v_cache[i].data_ptr(), self.pos.data_ptr(), s, cfg.q_heads,
+                                                   cfg.kv_heads, hd, self.max_seq, cfg.theta, _s()), "rope")
+            capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                              att.data_ptr(), self.pos.data_ptr(), s, cfg.q_heads, cfg.kv_heads, hd,
+                                              self.max_seq, _s()), "attention")
+            self._matmul(w[f"{i}.o"], att, o, s, bf16)
+            self._norm(h, o, h, w[f"{i}.ffn_norm"], n, s)          # h += attn out; n = norm(h)
+            self._matmul(w[f"{i}.gate_up"], n, gu, s, bf16)
+            capi.check(lib.lhip_swiglu_f32(gu.data_ptr(), act.data_ptr(), s, cfg.ffn, _s()), "swiglu")
+            self._matmul(w[f"{i}.down"], act, dn, s, bf16)
+        self._norm(h, dn, h, w["out_norm"], n, s)                    # last residual + final norm
+        if all_logits:
+            logits = self._buf("logits_all", (s, cfg.vocab))
+            self._matmul(w["lm_head"], n, logits, s, bf16)
+            return logits
+        logits = self._buf("logits", (cfg.vocab,))
+        last = n[s - 1]
+        self._matmul(w["lm_head"], last, logits, 1, False)  # only the last position is read (main.rs:58-61)
+        return logits
+
+    def _pick(self, logits, advance):
+        capi.check(self.lib.lhip_argmax_f32(logits.data_ptr(), self.cfg.vocab, self.tok.data_ptr(),
+                                            self.tok_i.data_ptr(), self.pos.data_ptr(), advance, _s()), "argmax")
+
+    # ---- generation loop (examples/llama/src/main.rs:101-190) ----------------
+    def prefill(self, tokens, bf16: bool = False):
+        t = torch.as_tensor(np.asarray(tokens, dtype=np.float32)).to(self.dev)
+        logits = self.forward(t, t.numel(), bf16=bf16)
+        self._pick(logits, t.numel())
+        return logits
+
+    def decode_step(self):
+        logits = self.forward(self.tok, 1)
+        self._pick(logits, 1)
+        return logits
+
+    def decode(self, steps: int, use_graph: bool = True):
+        """Greedy decode of `steps` tokens after a prefill; returns the token ids (first = the prefill's pick)."""
+        out = torch.empty(steps, dtype=torch.int32, device=self.dev)
+        if not use_graph:
+            for i in range(steps):
+                out[i:i + 1].copy_(self.tok_i)
+                self.decode_step()
+            return out
+        if self._graph is None:
+            pos0, tok0, toki0 = self.pos.clone(), self.tok.clone(), self.tok_i.clone()
+            st = torch.cuda.Stream(device=self.dev)
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                self.decode_step()  # warm-up outside capture (allocates the step's buffers)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=st):
+                    self.decode_step()
+            torch.cuda.current_stream().wait_stream(st)
+            self._graph = g
+            # undo the two steps above: the cache rows they wrote are rewritten by the replays
+            self.pos.copy_(pos0)
+            self.tok.copy_(tok0)
+            self.tok_i.copy_(toki0)
+        for i in range(steps):
+            out[i:i + 1].copy_(self.tok_i)
+            self._graph.replay()
+        return out
+
+
+def fuse_rows(*raws: np.ndarray) -> np.ndarray:
+    """Row-concatenate Q8_0 weights with the same K: their raw block streams simply follow each other."""
+    return np.concatenate([np.ascontiguousarray(r, dtype=np.uint8).reshape(-1) for r in raws])
+
+
+def random_weights(cfg: LlamaConfig, seed: int, device="cuda:0", scale_sigma: float | None = None) -> dict:
+    """Random Q8_0 model built on the device (quants U{-127..127}; block scales |N(0, sigma)|/127 with sigma
+    chosen so activations stay O(1): sigma ~ sqrt(3 / fan_in) / 0.8); norms 1 + small noise; embeddings N(0, 1)."""
+    lib = capi.load_library()
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+
+    def q8(n, k):
+        nb = n * k // 32
+        sigma = scale_sigma if scale_sigma is not None else float(np.sqrt(3.0 / k) / 0.8)
+        qs = torch.randint(-127, 128, (nb, 32), dtype=torch.int8, device=dev, generator=gen)
+        d = (torch.randn((nb, 1), device=dev, generator=gen).abs() * (sigma / 127.0)).to(torch.float16)
+        raw = torch.empty((nb, 34), dtype=torch.uint8, device=dev)
+        raw[:, :2] = d.view(torch.uint8)
+        raw[:, 2:] = qs.view(torch.uint8)
+        planar = torch.empty(lib.lhip_q8_0_planar_nbytes(n, k), dtype=torch.uint8, device=dev)
+        capi.check(lib.lhip_q8_0_repack(raw.data_ptr(), planar.data_ptr(), n, k, _s()), "lhip_q8_0_repack")
+        torch.cuda.synchronize()
+        return Q8Weight(planar, n, k)
+
+    def norm():
+        return 1.0 + 0.05 * torch.randn(cfg.dim, device=dev, generator=gen)
+
+    w = {"embed": torch.randn((cfg.vocab, cfg.dim), device=dev, generator=gen), "out_norm": norm(),
+         "lm_head": q8(cfg.vocab, cfg.dim)}
+    for i in range(cfg.layers):
+        w[f"{i}.attn_norm"], w[f"{i}.ffn_norm"] = norm(), norm()
+        w[f"{i}.qkv"] = q8(cfg.qkv_rows, cfg.dim)
+        w[f"{i}.o"] = q8(cfg.dim, cfg.dim)
+        w[f"{i}.gate_up"] = q8(2 * cfg.ffn, cfg.dim)
+        w[f"{i}.down"] = q8(cfg.dim, cfg.ffn)
+    return w

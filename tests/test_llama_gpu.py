@@ -1,0 +1,187 @@
+"""The Llama-3 decode loop through the C ABI against the numpy oracle, on small
+configurations of the same architecture (the oracle cannot run 8B parameters in
+test time): single operators, f32 prefill + decode logits within 2e-3, graph
+replay equal to eager stepping, bf16 prefill within the bf16 bar."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from conftest import rel_err  # noqa: E402
+from luminal_amd import capi, synth  # noqa: E402
+from luminal_amd.llama import LlamaConfig, LlamaQ8, fuse_rows  # noqa: E402
+from luminal_amd.quantized import Q8Weight  # noqa: E402
+from oracle import llama_oracle as lo  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def s():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def build_model(oracle, cfg, seed, max_seq=64):
+    """Random Q8_0 model: returns (engine, dequantised f32 weights for the oracle)."""
+    rng = np.random.default_rng(seed)
+    hd = cfg.head_dim
+    wf, raws = {}, {}
+
+    def q8(name, n, k, i):
+        qs, d = synth.q8_0_random(n, k, seed=seed * 1000 + i, scale_sigma=float(np.sqrt(3.0 / k) / 0.8))
+        raw = synth.q8_0_raw_blocks(qs, d)
+        raws[name] = raw
+        wf[name] = oracle.q8_0_dequant(raw, n * k).reshape(n, k)
+
+    wf["embed"] = rng.standard_normal((cfg.vocab, cfg.dim)).astype(np.float32)
+    wf["out_norm"] = (1 + 0.05 * rng.standard_normal(cfg.dim)).astype(np.float32)
+    q8("lm_head", cfg.vocab, cfg.dim, 0)
+    for i in range(cfg.layers):
+        wf[f"{i}.attn_norm"] = (1 + 0.05 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        wf[f"{i}.ffn_norm"] = (1 + 0.05 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        for j, (nm, n, k) in enumerate([("q", cfg.dim, cfg.dim), ("k", cfg.kv_heads * hd, cfg.dim),
+                                        ("v", cfg.kv_heads * hd, cfg.dim), ("o", cfg.dim, cfg.dim),
+                                        ("gate", cfg.ffn, cfg.dim), ("up", cfg.ffn, cfg.dim),
+                                        ("down", cfg.dim, cfg.ffn)]):
+            q8(f"{i}.{nm}", n, k, 10 * i + j + 1)
+    w = {"embed": torch.from_numpy(wf["embed"]).to(DEV), "out_norm": torch.from_numpy(wf["out_norm"]).to(DEV),
+         "lm_head": Q8Weight.from_raw(raws["lm_head"], cfg.vocab, cfg.dim, DEV)}
+    for i in range(cfg.layers):
+        w[f"{i}.attn_norm"] = torch.from_numpy(wf[f"{i}.attn_norm"]).to(DEV)
+        w[f"{i}.ffn_norm"] = torch.from_numpy(wf[f"{i}.ffn_norm"]).to(DEV)
+        w[f"{i}.qkv"] = Q8Weight.from_raw(fuse_rows(raws[f"{i}.q"], raws[f"{i}.k"], raws[f"{i}.v"]), cfg.qkv_rows,
+                                          cfg.dim, DEV)
+        w[f"{i}.o"] = Q8Weight.from_raw(raws[f"{i}.o"], cfg.dim, cfg.dim, DEV)
+        w[f"{i}.gate_up"] = Q8Weight.from_raw(fuse_rows(raws[f"{i}.gate"], raws[f"{i}.up"]), 2 * cfg.ffn, cfg.dim, DEV)
+        w[f"{i}.down"] = Q8Weight.from_raw(raws[f"{i}.down"], cfg.dim, cfg.ffn, DEV)
+    return LlamaQ8(cfg, w, max_seq, DEV), wf
+
+
+def empty_cache(cfg):
+    return [np.zeros((cfg.kv_heads, 0, cfg.head_dim)) for _ in range(cfg.layers)]
+
+
+# ------------------------------------------------------------------ single operators
+
+def test_rms_norm_and_fused_residual():
+    lib = capi.load_library()
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 4096)).astype(np.float32)
+    r = rng.standard_normal((5, 4096)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    xd, rd, wd = (torch.from_numpy(a).to(DEV) for a in (x, r, w))
+    y = torch.empty_like(xd)
+    assert lib.lhip_rms_norm_f32(xd.data_ptr(), None, None, wd.data_ptr(), y.data_ptr(), 5, 4096, 1e-5, s()) == 0
+    assert rel_err(y.cpu().numpy(), lo.rms_norm(x, w, 1e-5)) < 1e-5
+    xo = torch.empty_like(xd)
+    assert lib.lhip_rms_norm_f32(xd.data_ptr(), rd.data_ptr(), xo.data_ptr(), wd.data_ptr(), y.data_ptr(), 5, 4096,
+                                 1e-5, s()) == 0
+    assert np.array_equal(xo.cpu().numpy(), x + r)
+    assert rel_err(y.cpu().numpy(), lo.rms_norm(x + r, w, 1e-5)) < 1e-5
+
+
+def test_rope_attention_swiglu_gather_argmax():
+    lib = capi.load_library()
+    rng = np.random.default_rng(2)
+    hq, hkv, hd, max_seq, S, pos0 = 8, 2, 128, 40, 6, 9
+    qkv = rng.standard_normal((S, (hq + 2 * hkv) * hd)).astype(np.float32)
+    kc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    vc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    qd, kd, vd = (torch.from_numpy(a.copy()).to(DEV) for a in (qkv, kc, vc))
+    pos = torch.tensor([pos0], dtype=torch.int32, device=DEV)
+    assert lib.lhip_rope_kv_append_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), pos.data_ptr(), S, hq, hkv, hd,
+                                       max_seq, 500000.0, s()) == 0
+    rows = qkv.reshape(S, hq + 2 * hkv, hd)
+    q_want = lo.rope(rows[:, :hq].astype(np.float64), pos0, 500000.0)
+    k_want = lo.rope(rows[:, hq:hq + hkv].astype(np.float64), pos0, 500000.0)
+    got = qd.cpu().numpy().reshape(S, hq + 2 * hkv, hd)
+    assert np.max(np.abs(got[:, :hq] - q_want)) < 2e-5 and np.max(np.abs(got[:, hq:hq + hkv] - k_want)) < 2e-5
+    assert np.array_equal(got[:, hq + hkv:], rows[:, hq + hkv:])  # v untouched
+    kc2, vc2 = kd.cpu().numpy(), vd.cpu().numpy()
+    assert np.max(np.abs(kc2[:, pos0:pos0 + S] - k_want.transpose(1, 0, 2))) < 2e-5
+    assert np.array_equal(vc2[:, pos0:pos0 + S], rows[:, hq + hkv:].transpose(1, 0, 2))
+    assert np.array_equal(kc2[:, :pos0], kc[:, :pos0]) and np.array_equal(kc2[:, pos0 + S:], kc[:, pos0 + S:])
+    # attention over the updated cache
+    out = torch.empty((S, hq * hd), dtype=torch.float32, device=DEV)
+    assert lib.lhip_attention_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), pos.data_ptr(), S, hq,
+                                  hkv, hd, max_seq, s()) == 0
+    want = np.empty((S, hq, hd))
+    for t in range(S):
+        n_keys = pos0 + t + 1
+        for h in range(hq):
+            sc = kc2[h // (hq // hkv), :n_keys].astype(np.float64) @ got[t, h].astype(np.float64) / np.sqrt(hd)
+            p = np.exp(sc - sc.max())
+            want[t, h] = (p / p.sum()) @ vc2[h // (hq // hkv), :n_keys].astype(np.float64)
+    assert rel_err(out.cpu().numpy(), want.reshape(S, -1)) < 1e-4
+    # swiglu
+    gu = rng.standard_normal((3, 2 * 96)).astype(np.float32)
+    o = torch.empty((3, 96), dtype=torch.float32, device=DEV)
+    assert lib.lhip_swiglu_f32(torch.from_numpy(gu).to(DEV).data_ptr(), o.data_ptr(), 3, 96, s()) == 0
+    assert rel_err(o.cpu().numpy(), gu[:, 96:] * lo.swish(gu[:, :96].astype(np.float64))) < 1e-5
+    # fp32 row gather with f32 ids, argmax with the reference's tie rule (last maximum wins)
+    table = rng.standard_normal((50, 64)).astype(np.float32)
+    ids = torch.tensor([3.0, 49.0, 0.0, 7.9], device=DEV)
+    g = torch.empty((4, 64), dtype=torch.float32, device=DEV)
+    assert lib.lhip_gather_rows_f32(torch.from_numpy(table).to(DEV).data_ptr(), ids.data_ptr(), g.data_ptr(), 4, 50,
+                                    64, s()) == 0
+    assert np.array_equal(g.cpu().numpy(), table[[3, 49, 0, 7]])
+    v = rng.standard_normal(5000).astype(np.float32)
+    v[[17, 4021, 333]] = 9.5
+    idf = torch.zeros(1, device=DEV)
+    idi = torch.zeros(1, dtype=torch.int32, device=DEV)
+    assert lib.lhip_argmax_f32(torch.from_numpy(v).to(DEV).data_ptr(), 5000, idf.data_ptr(), idi.data_ptr(),
+                               pos.data_ptr(), 3, s()) == 0
+    assert int(idi.item()) == 4021 == lo.argmax_last(v) and idf.item() == 4021.0 and int(pos.item()) == pos0 + 3
+
+
+# ------------------------------------------------------------------ end to end
+
+@pytest.mark.parametrize("cfg", [LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512),
+                                 LlamaConfig(vocab=1000, dim=1024, layers=3, q_heads=8, kv_heads=2, ffn=2048)])
+def test_prefill_and_decode_logits_vs_oracle(oracle, cfg):
+    eng, wf = build_model(oracle, cfg, seed=cfg.dim)
+    rng = np.random.default_rng(3)
+    prompt = [int(t) for t in rng.integers(0, cfg.vocab, 12)]
+    kc, vc = empty_cache(cfg), empty_cache(cfg)
+    want = lo.forward(cfg, wf, prompt, kc, vc, 0)
+    got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
+    assert rel_err(got.cpu().numpy(), want) < 2e-3
+    # generation loop: prefill picks a token, then teacher-forced comparison of every decode step's logits
+    eng.reset()
+    eng.prefill(prompt)
+    tok = lo.argmax_last(want[-1])
+    assert int(eng.tok_i.item()) == tok and int(eng.pos.item()) == len(prompt)
+    for step in range(6):
+        want_step = lo.forward(cfg, wf, [tok], kc, vc, len(prompt) + step)[0]
+        logits = eng.decode_step()
+        assert rel_err(logits.cpu().numpy(), want_step) < 2e-3, step
+        tok = lo.argmax_last(want_step)
+        # keep both sides on the oracle's token even if a near-tie flipped the pick
+        eng.tok.fill_(float(tok))
+        eng.tok_i.fill_(tok)
+
+
+def test_graph_replay_equals_eager_decode(oracle):
+    cfg = LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)
+    eng, _ = build_model(oracle, cfg, seed=7)
+    prompt = [1, 2, 3, 4, 5]
+    eng.prefill(prompt)
+    eager = eng.decode(10, use_graph=False).cpu().numpy()
+    eng.reset()
+    eng.prefill(prompt)
+    graphed = eng.decode(10, use_graph=True).cpu().numpy()
+    assert np.array_equal(eager, graphed)
+    # a second run re-uses the captured graph
+    eng.reset()
+    eng.prefill(prompt)
+    assert np.array_equal(eng.decode(10, use_graph=True).cpu().numpy(), eager)
+
+
+def test_bf16_prefill_then_f32_decode(oracle):
+    cfg = LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)
+    eng, wf = build_model(oracle, cfg, seed=9)
+    prompt = [int(t) for t in np.random.default_rng(4).integers(0, cfg.vocab, 20)]
+    want = lo.forward(cfg, wf, prompt, empty_cache(cfg), empty_cache(cfg), 0)[-1]
+    got = eng.prefill(prompt, bf16=True).cpu().numpy()
+    t = np.asarray(want)
+    assert np.max(np.abs(got - t)) / np.sqrt(np.mean(t * t)) < 5e-2  # bf16 matmuls through the whole stack
