@@ -178,7 +178,8 @@ lhip_status lhip_gather_rows_f32(const float *table_dev, const float *idx_dev, f
 /* RMS norm as luminal's LayerNorm(mean_norm = false): y = v * 1/sqrt(mean(v^2) + eps) * w
  * (crates/luminal_nn/src/norm.rs:56-71, src/hl_ops/unary.rs:93-104).  With residual_dev
  * given, v = x + residual and v is also written to x_out_dev (the residual adds of
- * model.rs:173-187 fused into the norm that follows them); otherwise v = x. */
+ * model.rs:173-187 fused into the norm that follows them; x_out may be x itself); otherwise
+ * v = x.  dim % 4 == 0, dim <= 16384, 16-byte aligned pointers. */
 lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
                               float *y_dev, int64_t rows, int64_t dim, float eps, void *stream);
 /* Rotary embedding (adjacent pairs, model.rs:52-72) applied in place to the q and k heads
@@ -188,7 +189,8 @@ lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v
                                     int64_t tokens, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
                                     int64_t max_seq, float theta, void *stream);
 /* Causal grouped-query attention of the q heads in qkv over the caches (model.rs:112-139):
- * out[tokens][q_heads*head_dim].  head_dim <= 256, max_seq <= 16000. */
+ * out[tokens][q_heads*head_dim].  head_dim in {64, 128, 192, 256}, max_seq <= 12000;
+ * qkv, caches and out 16-byte aligned. */
 lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
                                float *out_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
                                int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);

@@ -49,25 +49,48 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float4 *__restri
 
 // y = (x [+ res]) * 1/sqrt(mean(x^2) + eps) * w ; if res is given, x_out receives x + res
 // (LayerNorm with mean_norm = false: std_norm then weight, norm.rs:56-71, unary.rs:93-104).
-__global__ __launch_bounds__(256) void rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ res,
-                                                       float *__restrict__ x_out, const float *__restrict__ w,
-                                                       float *__restrict__ y, int dim, float eps) {
-    __shared__ float red[4];
+// One block of 1024 threads per row; each thread keeps up to 4 float4 of the row in
+// registers between the two passes (dim <= 16384, dim % 4 == 0); x_out may alias x.
+__global__ __launch_bounds__(1024) void rms_norm_kernel(const float *x, const float *res, float *x_out,
+                                                        const float *__restrict__ w, float *__restrict__ y, int dim,
+                                                        float eps) {
+    __shared__ float red[16];
     const size_t base = static_cast<size_t>(blockIdx.x) * dim;
+    const int dim4 = dim >> 2;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x + base);
+    const float4 *r4 = res ? reinterpret_cast<const float4 *>(res + base) : nullptr;
+    float4 v[4];
     float ss = 0.f;
-    for (int j = threadIdx.x; j < dim; j += 256) {
-        float v = x[base + j];
-        if (res) {
-            v += res[base + j];
-            x_out[base + j] = v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int j = threadIdx.x + i * 1024;
+        v[i] = make_float4(0, 0, 0, 0);
+        if (j < dim4) {
+            v[i] = x4[j];
+            if (r4) {
+                const float4 r = r4[j];
+                v[i].x += r.x; v[i].y += r.y; v[i].z += r.z; v[i].w += r.w;
+            }
         }
-        ss += v * v;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int j = threadIdx.x + i * 1024;
+        if (j < dim4) {
+            if (r4) reinterpret_cast<float4 *>(x_out + base)[j] = v[i];
+            ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+        }
     }
     const float total = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
-    for (int j = threadIdx.x; j < dim; j += 256) {
-        const float v = res ? x_out[base + j] : x[base + j];
-        y[base + j] = v * scale * w[j];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int j = threadIdx.x + i * 1024;
+        if (j < dim4) {
+            const float4 g = reinterpret_cast<const float4 *>(w)[j];
+            reinterpret_cast<float4 *>(y + base)[j] =
+                make_float4(v[i].x * scale * g.x, v[i].y * scale * g.y, v[i].z * scale * g.z, v[i].w * scale * g.w);
+        }
     }
 }
 
@@ -106,33 +129,63 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float *__restrict__ qkv, fl
 // Causal grouped-query attention for S query tokens at positions pos0 .. pos0+S-1 over the
 // cache (model.rs:112-139): scores = q.k / sqrt(hd), masked positions get f16::MIN added (they
 // vanish in the softmax, so they are skipped), softmax, times V.  One block per (token, q head).
-// q is read from the fused qkv rows; out: [S][hq*hd].  Dynamic LDS: (pos0 + S) floats.
+// q is read from the fused qkv rows; out: [S][hq*hd].  Dynamic LDS: max_seq floats.
+//
+// Scores: 16 lanes share a key (each holds hd/16 elements of q in registers), so a wave
+// scores 4 keys at once and the block 16, four independent groups of loads in flight per lane.
+// P.V: 32 lanes cover hd as float4 and 8 such groups split the keys, partial sums meet in LDS.
+// Requires hd % 64 == 0 (hd = 64, 128, 192, 256).
 __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict__ qkv, const float *__restrict__ k_cache,
                                                         const float *__restrict__ v_cache, float *__restrict__ out,
                                                         const int *__restrict__ pos_dev, int hq, int hkv, int hd,
                                                         int max_seq) {
     extern __shared__ float sc[];  // scores of this query
     __shared__ float red[4];
-    __shared__ float qs[256];
+    __shared__ float4 part[8][64];  // P.V partial sums: 8 key groups x hd/4 float4
     const int s = blockIdx.x, h = blockIdx.y;
     const int n_keys = min(*pos_dev + s + 1, max_seq);
     const int kvh = h / (hq / hkv);
     const float *q = qkv + (static_cast<size_t>(s) * (hq + 2 * hkv) + h) * hd;
-    for (int j = threadIdx.x; j < hd; j += 256) qs[j] = q[j];
-    __syncthreads();
     const float *kc = k_cache + static_cast<size_t>(kvh) * max_seq * hd;
     const float *vc = v_cache + static_cast<size_t>(kvh) * max_seq * hd;
     const float inv_sqrt = 1.0f / sqrtf(static_cast<float>(hd));
-    // one wave per key: 64 lanes cover hd (<= 256) elements
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    // ---- scores
+    const int sub = threadIdx.x & 15;   // which slice of hd
+    const int kslot = threadIdx.x >> 4;  // which of the 16 keys of a round
+    const int per = hd / 16;             // 4, 8, 12 or 16 floats per lane, as float4s
+    float4 qr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        qr[j] = (j * 4 < per) ? *reinterpret_cast<const float4 *>(q + sub * per + j * 4) : make_float4(0, 0, 0, 0);
     float mx = -3.0e38f;
-    for (int p = wave; p < n_keys; p += 4) {
-        float d = 0.f;
-        for (int j = lane; j < hd; j += 64) d += qs[j] * kc[static_cast<size_t>(p) * hd + j];
-        for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o);
-        d *= inv_sqrt;
-        if (lane == 0) sc[p] = d;
-        mx = fmaxf(mx, d);
+    for (int p0 = 0; p0 < n_keys; p0 += 64) {  // 4 rounds of 16 keys per trip: independent loads
+        float d[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int p = p0 + u * 16 + kslot;
+            d[u] = 0.f;
+            if (p < n_keys) {
+                const float *kr = kc + static_cast<size_t>(p) * hd + sub * per;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (j * 4 < per) {
+                        const float4 kv = *reinterpret_cast<const float4 *>(kr + j * 4);
+                        d[u] += qr[j].x * kv.x + qr[j].y * kv.y + qr[j].z * kv.z + qr[j].w * kv.w;
+                    }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            float v = d[u];
+            for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
+            v *= inv_sqrt;
+            const int p = p0 + u * 16 + kslot;
+            if (p < n_keys) {
+                if (sub == 0) sc[p] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
     }
     mx = block_max(mx, red);
     float sum = 0.f;
@@ -141,13 +194,44 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
         sc[p] = e;
         sum += e;
     }
-    sum = block_sum(sum, red);
+    sum = block_sum(sum, red);  // also makes the exponentials visible to every thread
     const float inv = 1.0f / sum;
-    float *o = out + (static_cast<size_t>(s) * hq + h) * hd;
-    for (int j = threadIdx.x; j < hd; j += 256) {
-        float a = 0.f;
-        for (int p = 0; p < n_keys; ++p) a += sc[p] * vc[static_cast<size_t>(p) * hd + j];
-        o[j] = a * inv;
+
+    // ---- P.V
+    const int c4 = threadIdx.x & 31;  // float4 column (and c4 + 32 when hd > 128)
+    const int kg = threadIdx.x >> 5;  // key group 0..7
+    const int hd4 = hd / 4;
+    float4 a0 = make_float4(0, 0, 0, 0), a1 = make_float4(0, 0, 0, 0);
+    const bool lo_col = c4 < hd4, hi_col = c4 + 32 < hd4;
+    for (int p0 = kg; p0 < n_keys; p0 += 32) {  // 4 keys per trip and group: their loads are independent
+        float w[4];
+        float4 v0[4], v1[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int p = p0 + 8 * u;
+            const bool live = p < n_keys;
+            const float4 *vr = reinterpret_cast<const float4 *>(vc + static_cast<size_t>(live ? p : 0) * hd);
+            w[u] = live ? sc[p] : 0.f;
+            v0[u] = lo_col ? vr[c4] : make_float4(0, 0, 0, 0);
+            v1[u] = hi_col ? vr[c4 + 32] : make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            a0.x += w[u] * v0[u].x; a0.y += w[u] * v0[u].y; a0.z += w[u] * v0[u].z; a0.w += w[u] * v0[u].w;
+            a1.x += w[u] * v1[u].x; a1.y += w[u] * v1[u].y; a1.z += w[u] * v1[u].z; a1.w += w[u] * v1[u].w;
+        }
+    }
+    part[kg][c4] = a0;
+    part[kg][c4 + 32] = a1;
+    __syncthreads();
+    if (threadIdx.x < hd4) {
+        float4 t = part[0][threadIdx.x];
+        for (int g = 1; g < 8; ++g) {
+            const float4 u = part[g][threadIdx.x];
+            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
+        float4 *o = reinterpret_cast<float4 *>(out + (static_cast<size_t>(s) * hq + h) * hd);
+        o[threadIdx.x] = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
     }
 }
 
@@ -190,13 +274,30 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     __shared__ int bi[16];
     float v = -3.4e38f;
     int idx = -1;
-    for (int j = threadIdx.x; j < n; j += 1024) {
-        const float c = x[j];
-        if (idx < 0 || c >= v) {  // j increases, so >= keeps the last of equals
+    auto take = [&](float c, int j) {
+        if (idx < 0 || c > v || (c == v && j > idx)) {
             v = c;
             idx = j;
         }
+    };
+    const int n4 = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) ? n >> 2 : 0;  // vector part
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    for (int j0 = threadIdx.x; j0 < n4; j0 += 4096) {  // four independent loads per trip
+        float4 c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = j0 + u * 1024;
+            c[u] = j < n4 ? x4[j] : make_float4(-3.4e38f, -3.4e38f, -3.4e38f, -3.4e38f);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = (j0 + u * 1024) * 4;
+            if (j0 + u * 1024 < n4) {
+                take(c[u].x, j); take(c[u].y, j + 1); take(c[u].z, j + 2); take(c[u].w, j + 3);
+            }
+        }
     }
+    for (int j = n4 * 4 + threadIdx.x; j < n; j += 1024) take(x[j], j);
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(v, o);
         const int oi = __shfl_xor(idx, o);
@@ -245,8 +346,11 @@ lhip_status lhip_gather_rows_f32(const float *table_dev, const float *idx_dev, f
 lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
                               float *y_dev, int64_t rows, int64_t dim, float eps, void *stream) {
     if (!x_dev || !w_dev || !y_dev || (residual_dev && !x_out_dev)) return LHIP_ERR_NULL_PTR;
-    if (rows <= 0 || dim <= 0 || rows > kMaxDim || dim > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, as_stream(stream), x_dev,
+    if (rows <= 0 || dim <= 0 || rows > kMaxDim || dim > 16384 || dim % 4 != 0) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(x_dev, 16) || !aligned(w_dev, 16) || !aligned(y_dev, 16) ||
+        (residual_dev && (!aligned(residual_dev, 16) || !aligned(x_out_dev, 16))))
+        return LHIP_ERR_MISALIGNED;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<unsigned>(rows)), dim3(1024), 0, as_stream(stream), x_dev,
                        residual_dev, x_out_dev, w_dev, y_dev, static_cast<int>(dim), eps);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
@@ -271,8 +375,8 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
                                float *out_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
                                int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream) {
     if (!qkv_dev || !k_cache_dev || !v_cache_dev || !out_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
-    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || max_seq <= 0 ||
-        q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 16000)
+    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || head_dim % 64 != 0 ||
+        max_seq <= 0 || q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 12000)
         return LHIP_ERR_INVALID_SHAPE;  // the score row of one query lives in LDS
     hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)), dim3(256),
                        static_cast<size_t>(max_seq) * sizeof(float), as_stream(stream), qkv_dev, k_cache_dev,

@@ -112,7 +112,7 @@ def test_rope_attention_swiglu_gather_argmax():
             sc = kc2[h // (hq // hkv), :n_keys].astype(np.float64) @ got[t, h].astype(np.float64) / np.sqrt(hd)
             p = np.exp(sc - sc.max())
             want[t, h] = (p / p.sum()) @ vc2[h // (hq // hkv), :n_keys].astype(np.float64)
-    assert rel_err(out.cpu().numpy(), want.reshape(S, -1)) < 1e-4
+    assert rel_err(out.cpu().numpy(), want.reshape(S, -1)) < 1e-3
     # swiglu
     gu = rng.standard_normal((3, 2 * 96)).astype(np.float32)
     o = torch.empty((3, 96), dtype=torch.float32, device=DEV)
