@@ -39,6 +39,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end Llama-3-8B decode section")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
 
@@ -107,6 +108,47 @@ def cpu_baseline(seconds: float):
         "all_cores": {"value": round(q8_bytes / tn / 1e9, 3), "cores": ncpu, "passes": repsn,
                       "ms_per_pass": round(tn * 1e3, 2)},
     }
+
+
+def llama_decode(torch):
+    """BASELINE config 4: random-weight Llama-3-8B, all linears Q8_0, norms and embeddings f32;
+    512-token prefill (bf16 GEMM path), then 256 greedy batch-1 decode steps (f32 matvec path,
+    one captured HIP graph per step, token and position stay on the device)."""
+    import numpy as np
+
+    from luminal_amd.llama import LLAMA3_8B, LlamaQ8, random_weights
+
+    cfg = LLAMA3_8B
+    w = random_weights(cfg, seed=4, device="cuda:0")
+    eng = LlamaQ8(cfg, w, max_seq=1024)
+    prompt = np.random.default_rng(0).integers(0, cfg.vocab, 512)
+    eng.prefill(prompt, bf16=True)          # warm-up (allocates buffers)
+    eng.decode(4, use_graph=True)           # captures the decode graph
+    eng.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.prefill(prompt, bf16=True)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    toks = eng.decode(256, use_graph=True)
+    torch.cuda.synchronize()
+    t_decode = time.perf_counter() - t0
+    weight_bytes = cfg.layers * sum(synth_bytes(n, k) for n, k in
+                                    [(cfg.qkv_rows, cfg.dim), (cfg.dim, cfg.dim), (2 * cfg.ffn, cfg.dim),
+                                     (cfg.dim, cfg.ffn)]) + synth_bytes(cfg.vocab, cfg.dim)
+    ms = t_decode / 256 * 1e3
+    return {"tok_s": round(256 / t_decode, 1), "ms_per_token": round(ms, 3),
+            "prefill_tokens": 512, "prefill_ms": round(t_prefill * 1e3, 2),
+            "prefill_tok_s": round(512 / t_prefill, 1), "decode_steps": 256,
+            "q8_0_weight_bytes_per_token": weight_bytes,
+            "weight_stream_gbs": round(weight_bytes / (t_decode / 256) / 1e9, 1),
+            "frac_hbm_peak": round(weight_bytes / (t_decode / 256) / 1e9 / HBM_PEAK_GBS, 4),
+            "first_tokens": [int(t) for t in toks[:4].tolist()]}
+
+
+def synth_bytes(n, k):
+    return n * k * 34 // 32
 
 
 def main():
@@ -285,9 +327,12 @@ def main():
         "calibration": calibration,
         "roofline": roofline,
     }
-    if not args.no_cpu_baseline:
-        del weights
+    del weights
+    torch.cuda.empty_cache()
+    if not args.no_decode and layers == 32:
+        out["llama3_8b_q8_0_decode"] = llama_decode(torch)
         torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
     print(json.dumps(out))
 

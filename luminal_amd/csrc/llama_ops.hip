@@ -131,17 +131,23 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float *__restrict__ qkv, fl
 // vanish in the softmax, so they are skipped), softmax, times V.  One block per (token, q head).
 // q is read from the fused qkv rows; out: [S][hq*hd].  Dynamic LDS: max_seq floats.
 //
-// Scores: 16 lanes share a key (each holds hd/16 elements of q in registers), so a wave
-// scores 4 keys at once and the block 16, four independent groups of loads in flight per lane.
-// P.V: 32 lanes cover hd as float4 and 8 such groups split the keys, partial sums meet in LDS.
-// Requires hd % 64 == 0 (hd = 64, 128, 192, 256).
-__global__ __launch_bounds__(256) void attention_kernel(const float *__restrict__ qkv, const float *__restrict__ k_cache,
-                                                        const float *__restrict__ v_cache, float *__restrict__ out,
-                                                        const int *__restrict__ pos_dev, int hq, int hkv, int hd,
-                                                        int max_seq) {
+// Scores: 16 lanes share a key (each holds hd/16 elements of q in registers); the block's
+// 1024 threads score 64 keys per round and 8 rounds per trip, so up to 512 key rows are
+// requested before the first one is used — a decode step over a few hundred keys is one or
+// two memory round trips instead of one per key.
+// P.V: 32 lanes cover hd as float4 and 32 such groups split the keys, 8 keys per group and
+// trip; partial sums meet in LDS.  Requires hd % 64 == 0 (hd = 64, 128, 192, 256).
+constexpr int kAttnThreads = 1024;
+
+__global__ __launch_bounds__(kAttnThreads) void attention_kernel(const float *__restrict__ qkv,
+                                                                  const float *__restrict__ k_cache,
+                                                                  const float *__restrict__ v_cache,
+                                                                  float *__restrict__ out,
+                                                                  const int *__restrict__ pos_dev, int hq, int hkv,
+                                                                  int hd, int max_seq) {
     extern __shared__ float sc[];  // scores of this query
-    __shared__ float red[4];
-    __shared__ float4 part[8][64];  // P.V partial sums: 8 key groups x hd/4 float4
+    __shared__ float red[16];
+    __shared__ float4 part[32][64];  // P.V partial sums: 32 key groups x hd/4 float4
     const int s = blockIdx.x, h = blockIdx.y;
     const int n_keys = min(*pos_dev + s + 1, max_seq);
     const int kvh = h / (hq / hkv);
@@ -151,19 +157,19 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
     const float inv_sqrt = 1.0f / sqrtf(static_cast<float>(hd));
 
     // ---- scores
-    const int sub = threadIdx.x & 15;   // which slice of hd
-    const int kslot = threadIdx.x >> 4;  // which of the 16 keys of a round
+    const int sub = threadIdx.x & 15;    // which slice of hd
+    const int kslot = threadIdx.x >> 4;  // which of the 64 keys of a round
     const int per = hd / 16;             // 4, 8, 12 or 16 floats per lane, as float4s
     float4 qr[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
         qr[j] = (j * 4 < per) ? *reinterpret_cast<const float4 *>(q + sub * per + j * 4) : make_float4(0, 0, 0, 0);
     float mx = -3.0e38f;
-    for (int p0 = 0; p0 < n_keys; p0 += 64) {  // 4 rounds of 16 keys per trip: independent loads
-        float d[4];
+    for (int p0 = 0; p0 < n_keys; p0 += 512) {
+        float d[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int p = p0 + u * 16 + kslot;
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + u * 64 + kslot;
             d[u] = 0.f;
             if (p < n_keys) {
                 const float *kr = kc + static_cast<size_t>(p) * hd + sub * per;
@@ -176,11 +182,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 8; ++u) {
             float v = d[u];
             for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
             v *= inv_sqrt;
-            const int p = p0 + u * 16 + kslot;
+            const int p = p0 + u * 64 + kslot;
             if (p < n_keys) {
                 if (sub == 0) sc[p] = v;
                 mx = fmaxf(mx, v);
@@ -189,7 +195,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
     }
     mx = block_max(mx, red);
     float sum = 0.f;
-    for (int p = threadIdx.x; p < n_keys; p += 256) {
+    for (int p = threadIdx.x; p < n_keys; p += kAttnThreads) {
         const float e = expf(sc[p] - mx);
         sc[p] = e;
         sum += e;
@@ -199,16 +205,16 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
 
     // ---- P.V
     const int c4 = threadIdx.x & 31;  // float4 column (and c4 + 32 when hd > 128)
-    const int kg = threadIdx.x >> 5;  // key group 0..7
+    const int kg = threadIdx.x >> 5;  // key group 0..31
     const int hd4 = hd / 4;
     float4 a0 = make_float4(0, 0, 0, 0), a1 = make_float4(0, 0, 0, 0);
     const bool lo_col = c4 < hd4, hi_col = c4 + 32 < hd4;
-    for (int p0 = kg; p0 < n_keys; p0 += 32) {  // 4 keys per trip and group: their loads are independent
-        float w[4];
-        float4 v0[4], v1[4];
+    for (int p0 = kg; p0 < n_keys; p0 += 256) {  // 8 keys per trip and group: their loads are independent
+        float w[8];
+        float4 v0[8], v1[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int p = p0 + 8 * u;
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + 32 * u;
             const bool live = p < n_keys;
             const float4 *vr = reinterpret_cast<const float4 *>(vc + static_cast<size_t>(live ? p : 0) * hd);
             w[u] = live ? sc[p] : 0.f;
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
             v1[u] = hi_col ? vr[c4 + 32] : make_float4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 8; ++u) {
             a0.x += w[u] * v0[u].x; a0.y += w[u] * v0[u].y; a0.z += w[u] * v0[u].z; a0.w += w[u] * v0[u].w;
             a1.x += w[u] * v1[u].x; a1.y += w[u] * v1[u].y; a1.z += w[u] * v1[u].z; a1.w += w[u] * v1[u].w;
         }
@@ -226,7 +232,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float *__restrict_
     __syncthreads();
     if (threadIdx.x < hd4) {
         float4 t = part[0][threadIdx.x];
-        for (int g = 1; g < 8; ++g) {
+        for (int g = 1; g < 32; ++g) {
             const float4 u = part[g][threadIdx.x];
             t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
         }
@@ -378,7 +384,8 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
     if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || head_dim % 64 != 0 ||
         max_seq <= 0 || q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 12000)
         return LHIP_ERR_INVALID_SHAPE;  // the score row of one query lives in LDS
-    hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)), dim3(256),
+    hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)),
+                       dim3(kAttnThreads),
                        static_cast<size_t>(max_seq) * sizeof(float), as_stream(stream), qkv_dev, k_cache_dev,
                        v_cache_dev, out_dev, pos_dev, static_cast<int>(q_heads), static_cast<int>(kv_heads),
                        static_cast<int>(head_dim), static_cast<int>(max_seq));
