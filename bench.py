@@ -37,6 +37,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="decode_projection_set",
+                    choices=["decode_projection_set", "prefill_gemm", "moe"],
+                    help="decode_projection_set (default, the headline metric), prefill_gemm (BASELINE config 2), "
+                         "moe (BASELINE config 3)")
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end Llama-3-8B decode section")
@@ -110,6 +114,180 @@ def cpu_baseline(seconds: float):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP8_PEAK_TFLOPS = 5000.0
+MFMA_FP4_PEAK_TFLOPS = 10100.0
+
+
+def _event_us(torch, fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def bench_prefill_gemm(args):
+    """BASELINE config 2: the seven Llama-3-8B weight shapes in Q8_0 against bf16 activations,
+    M in {128, 512, 2048}, f32 accumulation, bf16 output.  A step is one pass over all shapes at
+    all three M; weights rotate over distinct buffers."""
+    import torch
+
+    from luminal_amd import capi, synth
+
+    lib = capi.load_library()
+    dev = torch.device("cuda:0")
+    capi.check(lib.lhip_init(0), "lhip_init")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0x5EED + 2)
+    stream = torch.cuda.current_stream().cuda_stream
+    shapes = {"q/o": (4096, 4096), "k/v": (1024, 4096), "gate/up": (14336, 4096), "down": (4096, 14336),
+              "lm_head": (128256, 4096)}
+    ms_list = (128, 512, 2048)
+    bufs, xs, ys = {}, {}, {}
+    for nm, (n, k) in shapes.items():
+        nbuf = 1 if nm == "lm_head" else 4
+        bufs[nm] = [make_weight(torch, lib, capi, n, k, gen, dev) for _ in range(nbuf)]
+    for m in ms_list:
+        for k in (4096, 14336):
+            xs[(m, k)] = torch.randn((m, k), device=dev, generator=gen).to(torch.bfloat16)
+        for n in (4096, 1024, 14336, 128256):
+            ys[(m, n)] = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+
+    def run(nm, m, b):
+        n, k = shapes[nm]
+        st = lib.lhip_q8_0_matmul_bf16(b.data_ptr(), xs[(m, k)].data_ptr(), ys[(m, n)].data_ptr(), m, n, k, stream)
+        if st:
+            capi.check(st, "lhip_q8_0_matmul_bf16")
+
+    def step():
+        for nm in shapes:
+            for m in ms_list:
+                run(nm, m, bufs[nm][0])
+
+    flops_step = sum(2.0 * m * n * k for (n, k) in shapes.values() for m in ms_list)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = {}
+    for nm, (n, k) in shapes.items():
+        for m in ms_list:
+            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3) / len(bufs[nm])
+            fl = 2.0 * m * n * k
+            by = n * k * 34 // 32 + 2 * m * k + 2 * m * n
+            per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                                  "frac_mfma_bf16": round(fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                  "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4> on the M = 2048 gate/up shape
+    n, k, m = 14336, 4096, 2048
+    us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5) / len(bufs["gate/up"])
+    ach = 2.0 * m * n * k / us / 1e6
+    value = flops_step / (wall / args.steps) / 1e12
+    print(json.dumps({
+        "metric": "Q8_0 prefill GEMM TFLOP/s (MFMA utilisation), 1 GPU", "value": round(value, 1), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 weights dequantised to bf16 x bf16 activations, f32 accumulate, bf16 out", "data": "synthetic",
+        "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list)},
+        "per_shape": per,
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4> (gate/up, M=2048)",
+                     "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_us": round(us, 1)}}))
+
+
+def bench_moe(args):
+    """BASELINE config 3: gpt-oss-style MXFP4 expert layer, H = I = 2880, 32 experts, top-4,
+    T in {1, 64, 1024}; a step is one layer pass at each T (routing rotates so T = 1 streams
+    different experts from HBM every pass)."""
+    import torch
+
+    from luminal_amd import capi, synth
+    from luminal_amd.moe import Mxfp4Weight, MoEExperts, route_topk
+
+    lib = capi.load_library()
+    dev = torch.device("cuda:0")
+    capi.check(lib.lhip_init(0), "lhip_init")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0x5EED + 3)
+    E, H, I, K4 = synth.MOE_EXPERTS, synth.MOE_HIDDEN, synth.MOE_INTER, synth.MOE_TOPK
+
+    def weight(n, k):  # random e2m1 codes, e8m0 exponents uniform in [-8, 0], built raw then repacked by the library
+        nb = n * k // 32
+        raw = torch.empty((nb, 17), dtype=torch.uint8, device=dev)
+        raw[:, :16] = torch.randint(0, 256, (nb, 16), dtype=torch.uint8, device=dev, generator=gen)
+        raw[:, 16] = torch.randint(119, 128, (nb,), dtype=torch.uint8, device=dev, generator=gen)
+        planar = torch.empty(lib.lhip_mxfp4_planar_nbytes(n, k), dtype=torch.uint8, device=dev)
+        capi.check(lib.lhip_mxfp4_repack(raw.data_ptr(), planar.data_ptr(), n, k,
+                                         torch.cuda.current_stream().cuda_stream), "lhip_mxfp4_repack")
+        torch.cuda.synchronize()
+        return Mxfp4Weight(planar, n, k)
+
+    layer = MoEExperts(weight(E * 2 * I, H), weight(E * H, I), E, H, I)
+    cases = {}
+    for T in (1, 64, 1024):
+        x = torch.randn((T, H), device=dev, generator=gen).to(torch.bfloat16)
+        routes = []
+        for r in range(8):
+            logits = torch.randn((T, E), device=dev, generator=gen)
+            if T == 1:
+                logits[0, 4 * r:4 * r + 4] += 100.0
+            routes.append(route_topk(logits, K4))
+        cases[T] = (x, routes)
+    it = [0]
+
+    def run(T):
+        x, routes = cases[T]
+        sel, wts = routes[it[0] % 8]
+        it[0] += 1
+        layer.process(x, sel, wts)
+
+    def step():
+        for T in cases:
+            run(T)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = {}
+    flops_step = 0.0
+    for T in cases:
+        us = _event_us(torch, lambda: run(T), 16)
+        touched = E if T >= 64 else K4
+        by = touched * 13219200 + 2 * 2 * T * H
+        fl = T * 199065600.0
+        flops_step += fl
+        per[f"T={T}"] = {"us": round(us, 1), "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
+                         "tflops": round(fl / us / 1e6, 1), "frac_mfma_fp4": round(fl / us / 1e6 / MFMA_FP4_PEAK_TFLOPS, 5),
+                         "frac_mfma_fp8_two_pass": round(2 * fl / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 5)}
+    t64 = per["T=64"]
+    print(json.dumps({
+        "metric": "MXFP4 MoE expert layer (H=I=2880, 32 experts, top-4): GB/s and TFLOP/s, 1 GPU",
+        "value": round(flops_step / (wall / args.steps) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp4 (e2m1, e8m0 block scales) weights x bf16 activations split exactly into two fp8 operands, "
+                 "f32 accumulate on v_mfma_scale_f32_16x16x128_f8f6f4, bf16 out",
+        "data": "synthetic", "config": {"workload": "gpt_oss_style_mxfp4_moe_layer", "tokens": [1, 64, 1024]},
+        "per_tokens": per,
+        "roofline": {"bound": "hbm", "kernel": "whole layer at T=64 (plan, quantise, 2 grouped GEMMs, combine)",
+                     "achieved": t64["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": t64["frac_hbm"],
+                     "traffic": None}}))
+
+
 def llama_decode(torch):
     """BASELINE config 4: random-weight Llama-3-8B, all linears Q8_0, norms and embeddings f32;
     512-token prefill (bf16 GEMM path), then 256 greedy batch-1 decode steps (f32 matvec path,
@@ -157,6 +335,10 @@ def main():
         print("bench.py: this build measures ONE GPU's share of the path (no collectives, no sharding); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "prefill_gemm":
+        return bench_prefill_gemm(args)
+    if args.workload == "moe":
+        return bench_moe(args)
 
     import torch
 
