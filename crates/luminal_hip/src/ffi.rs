@@ -1,0 +1,30 @@
+//! `extern "C"` surface of libluminal_hip.so (include/luminal_hip.h), plus the status-to-panic bridge:
+//! luminal's backends `unwrap()` every driver call, so a non-zero status becomes a panic here.
+use std::ffi::{c_char, c_void, CStr};
+
+pub type Status = i32;
+pub type Stream = *mut c_void;
+
+extern "C" {
+    pub fn lhip_status_string(s: Status) -> *const c_char;
+    pub fn lhip_last_hip_error() -> i32;
+    pub fn lhip_init(device: i32) -> Status;
+    pub fn lhip_malloc(dptr: *mut *mut c_void, nbytes: usize) -> Status;
+    pub fn lhip_free(dptr: *mut c_void) -> Status;
+    pub fn lhip_memcpy_h2d(dst: *mut c_void, src: *const c_void, nbytes: usize, s: Stream) -> Status;
+    pub fn lhip_memcpy_d2h(dst: *mut c_void, src: *const c_void, nbytes: usize, s: Stream) -> Status;
+    pub fn lhip_stream_sync(s: Stream) -> Status;
+    pub fn lhip_q8_0_raw_nbytes(n: i64, k: i64) -> usize;
+    pub fn lhip_q8_0_planar_nbytes(n: i64, k: i64) -> usize;
+    pub fn lhip_q8_0_repack(raw: *const c_void, planar: *mut c_void, n: i64, k: i64, s: Stream) -> Status;
+    pub fn lhip_q8_0_matmul_f32(w: *const c_void, x: *const f32, y: *mut f32, m: i64, n: i64, k: i64, s: Stream) -> Status;
+    pub fn lhip_q8_0_gather_f32(w: *const c_void, idx: *const f32, out: *mut f32, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;
+}
+
+#[track_caller]
+pub fn check(status: Status, what: &str) {
+    if status != 0 {
+        let name = unsafe { CStr::from_ptr(lhip_status_string(status)) }.to_string_lossy().into_owned();
+        panic!("{what}: {name} (hipError_t {})", unsafe { lhip_last_hip_error() });
+    }
+}

@@ -185,3 +185,53 @@ def test_bf16_prefill_then_f32_decode(oracle):
     got = eng.prefill(prompt, bf16=True).cpu().numpy()
     t = np.asarray(want)
     assert np.max(np.abs(got - t)) / np.sqrt(np.mean(t * t)) < 5e-2  # bf16 matmuls through the whole stack
+
+
+def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
+    """A synthetic GGUF with the reference's tensor names, read back through the loader
+    (examples/llama/src/loader.rs:99-165), must produce exactly the engine built from the same blocks."""
+    from luminal_amd import gguf
+
+    cfg = LlamaConfig(vocab=256, dim=128, layers=2, q_heads=4, kv_heads=2, ffn=256)
+    rng = np.random.default_rng(5)
+    hd = cfg.head_dim
+    tensors = {"token_embd.weight": ("F32", (cfg.dim, cfg.vocab), rng.standard_normal((cfg.vocab, cfg.dim)).astype("<f4").tobytes()),
+               "output_norm.weight": ("F32", (cfg.dim,), (1 + 0.05 * rng.standard_normal(cfg.dim)).astype("<f4").tobytes())}
+
+    def q8(name, n, k, i):
+        qs, d = synth.q8_0_random(n, k, seed=500 + i, scale_sigma=float(np.sqrt(3.0 / k) / 0.8))
+        tensors[name] = ("Q8_0", (k, n), synth.q8_0_raw_blocks(qs, d).tobytes())
+
+    q8("output.weight", cfg.vocab, cfg.dim, 0)
+    for i in range(cfg.layers):
+        for nm in ("attn_norm", "ffn_norm"):
+            tensors[f"blk.{i}.{nm}.weight"] = ("F32", (cfg.dim,), (1 + 0.05 * rng.standard_normal(cfg.dim)).astype("<f4").tobytes())
+        for j, (nm, n, k) in enumerate([("attn_q", cfg.dim, cfg.dim), ("attn_k", cfg.kv_heads * hd, cfg.dim),
+                                        ("attn_v", cfg.kv_heads * hd, cfg.dim), ("attn_output", cfg.dim, cfg.dim),
+                                        ("ffn_gate", cfg.ffn, cfg.dim), ("ffn_up", cfg.ffn, cfg.dim),
+                                        ("ffn_down", cfg.dim, cfg.ffn)]):
+            q8(f"blk.{i}.{nm}.weight", n, k, 10 * i + j + 1)
+    path = tmp_path / "tiny_llama.gguf"
+    gguf.write_gguf(path, {"general.architecture": "llama"}, tensors)
+    eng = LlamaQ8(cfg, gguf.q8_load(path, cfg, DEV), max_seq=32)
+    # oracle weights straight from the same bytes
+    wf = {}
+    for name, (dt, dims, data) in tensors.items():
+        arr = np.frombuffer(data, dtype="<f4") if dt == "F32" else oracle.q8_0_dequant(np.frombuffer(data, np.uint8), int(np.prod(dims)))
+        wf[name] = arr
+    ow = {"embed": wf["token_embd.weight"].reshape(cfg.vocab, cfg.dim), "out_norm": wf["output_norm.weight"],
+          "lm_head": wf["output.weight"].reshape(cfg.vocab, cfg.dim)}
+    for i in range(cfg.layers):
+        b = f"blk.{i}."
+        ow[f"{i}.attn_norm"], ow[f"{i}.ffn_norm"] = wf[b + "attn_norm.weight"], wf[b + "ffn_norm.weight"]
+        ow[f"{i}.q"] = wf[b + "attn_q.weight"].reshape(cfg.dim, cfg.dim)
+        ow[f"{i}.k"] = wf[b + "attn_k.weight"].reshape(cfg.kv_heads * hd, cfg.dim)
+        ow[f"{i}.v"] = wf[b + "attn_v.weight"].reshape(cfg.kv_heads * hd, cfg.dim)
+        ow[f"{i}.o"] = wf[b + "attn_output.weight"].reshape(cfg.dim, cfg.dim)
+        ow[f"{i}.gate"] = wf[b + "ffn_gate.weight"].reshape(cfg.ffn, cfg.dim)
+        ow[f"{i}.up"] = wf[b + "ffn_up.weight"].reshape(cfg.ffn, cfg.dim)
+        ow[f"{i}.down"] = wf[b + "ffn_down.weight"].reshape(cfg.dim, cfg.ffn)
+    prompt = [3, 200, 17, 5]
+    want = lo.forward(cfg, ow, prompt, empty_cache(cfg), empty_cache(cfg), 0)
+    got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
+    assert rel_err(got.cpu().numpy(), want) < 2e-3
