@@ -192,7 +192,7 @@ def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
     (examples/llama/src/loader.rs:99-165), must produce exactly the engine built from the same blocks."""
     from luminal_amd import gguf
 
-    cfg = LlamaConfig(vocab=256, dim=128, layers=2, q_heads=4, kv_heads=2, ffn=256)
+    cfg = LlamaConfig(vocab=256, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)  # head_dim 64
     rng = np.random.default_rng(5)
     hd = cfg.head_dim
     tensors = {"token_embd.weight": ("F32", (cfg.dim, cfg.vocab), rng.standard_normal((cfg.vocab, cfg.dim)).astype("<f4").tobytes()),
