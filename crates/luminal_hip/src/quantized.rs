@@ -63,6 +63,26 @@ fn device_ptr(t: &InputTensor) -> *mut c_void {
     t.borrowed().downcast_ref::<HipData>().expect("operand is not a HIP buffer").ptr
 }
 
+/// Activation operand: already on the device, or a host vector that is uploaded for this call.
+enum Activation<'a> {
+    Device(&'a HipData),
+    Staged(HipData),
+}
+
+impl Activation<'_> {
+    fn of(t: &InputTensor) -> Activation<'_> {
+        let any = t.borrowed();
+        if let Some(d) = any.downcast_ref::<HipData>() {
+            Activation::Device(d)
+        } else {
+            Activation::Staged(HipData::from_host(any.downcast_ref::<Vec<f32>>().expect("activation is neither HipData nor Vec<f32>")))
+        }
+    }
+    fn ptr(&self) -> *const f32 {
+        (match self { Activation::Device(d) => d.ptr, Activation::Staged(d) => d.ptr }) as _
+    }
+}
+
 fn usize_dims(s: &ShapeTracker) -> Vec<usize> {
     s.dims().into_iter().map(|d| d.to_usize().unwrap()).collect()
 }
@@ -78,13 +98,14 @@ impl Operator for QuantizedMatmul<f32> {
         let rows: usize = a[..a.len() - 1].iter().product::<usize>().max(1); // batch * m
         let (k, n) = (b[b.len() - 2], b[b.len() - 1]);
         let out = HipData::alloc(rows * n * 4);
+        let x = Activation::of(&inp[0].0);
         check(
             unsafe {
-                ffi::lhip_q8_0_matmul_f32(device_ptr(&inp[1].0), device_ptr(&inp[0].0) as _, out.ptr as _, rows as i64,
-                                          n as i64, k as i64, null_mut())
+                ffi::lhip_q8_0_matmul_f32(device_ptr(&inp[1].0), x.ptr(), out.ptr as _, rows as i64, n as i64, k as i64, null_mut())
             },
             "lhip_q8_0_matmul_f32",
         );
+        check(unsafe { ffi::lhip_stream_sync(null_mut()) }, "lhip_stream_sync"); // a staged activation is freed on return
         vec![Tensor::new(out)]
     }
 }
@@ -93,19 +114,19 @@ impl Operator for QuantizedMatmul<f32> {
 #[derive(Clone, Debug)]
 pub struct QuantizedGather<T> {
     pub embed_dim: usize,
-    pub vocab: usize,
     _t: PhantomData<T>,
 }
 
 impl Operator for QuantizedGather<f32> {
     fn process(&mut self, inp: Vec<(InputTensor, ShapeTracker)>) -> Vec<Tensor> {
         let idx = inp[0].0.borrowed().downcast_ref::<Vec<f32>>().expect("gather indices are host f32");
+        let vocab = inp[1].1.dims().into_iter().map(|d| d.to_usize().unwrap()).product::<usize>() / self.embed_dim;
         let idx_dev = HipData::from_host(idx);
         let out = HipData::alloc(idx.len() * self.embed_dim * 4);
         check(
             unsafe {
                 ffi::lhip_q8_0_gather_f32(device_ptr(&inp[1].0), idx_dev.ptr as _, out.ptr as _, idx.len() as i64,
-                                          self.vocab as i64, self.embed_dim as i64, null_mut())
+                                          vocab as i64, self.embed_dim as i64, null_mut())
             },
             "lhip_q8_0_gather_f32",
         );
@@ -115,6 +136,13 @@ impl Operator for QuantizedGather<f32> {
 }
 
 /// Rewrites the consumers of the given Q8_0 weight nodes into HIP quantized operators.
+///
+/// Runs after the CPU backend's pattern passes (`luminal_cpu::MatMulCompiler`, `GatherCompiler`), which turn
+/// Mul -> SumReduce and the one-hot lookup into `MatMul2D` / `BatchedMatMul2D` / `Gather` nodes; those are the nodes
+/// replaced here, as the CUDA pass replaces `Matmul<T>` / `CudaGather<T>` (crates/luminal_cuda/src/quantized.rs:244-272).
+/// Activations entering and leaving the quantized nodes are host `Vec<f32>` in that pipeline, so the operators below
+/// accept either a `HipData` or a host vector as the activation operand and always return `HipData`; a graph that
+/// keeps activations on the device needs `HipData`-aware neighbours (copy nodes or dense HIP operators).
 #[derive(Debug, Default)]
 pub struct HipQuantizedCompiler<T> {
     weights: Vec<NodeIndex>,
@@ -138,57 +166,15 @@ impl Compiler for HipQuantizedCompiler<f32> {
                 .collect();
             for (consumer, slot) in uses {
                 assert_eq!(slot, 1, "Quantized weight {consumer:?} is the wrong input!");
-                // With only GenericCompiler in front, the consumer is still the primitive Mul feeding a
-                // SumReduce(2) (the pattern crates/luminal_cpu/src/matmul.rs matches) or the one-hot gather
-                // pattern; `fuse_into` replaces that pair by one node and returns it.
-                match crate::quantized::patterns::classify(graph, consumer) {
-                    patterns::Use::Matmul(node) => *graph.node_weight_mut(node).unwrap() = Box::new(QuantizedMatmul::<f32>::default()),
-                    patterns::Use::Gather { node, embed_dim, vocab } => {
-                        *graph.node_weight_mut(node).unwrap() = Box::new(QuantizedGather::<f32> { embed_dim, vocab, _t: PhantomData })
-                    }
-                    patterns::Use::Other(op) => panic!("Quantized weight {consumer:?} feeds a node that is neither a matmul nor a gather ({op})"),
+                let op = graph.node_weight_mut(consumer).unwrap();
+                if let Some(g) = op.as_any().downcast_ref::<luminal_cpu::Gather>() {
+                    *op = Box::new(QuantizedGather::<f32> { embed_dim: g.embed_dim, _t: PhantomData });
+                } else if op.as_any().is::<luminal_cpu::MatMul2D>() || op.as_any().is::<luminal_cpu::BatchedMatMul2D>() {
+                    *op = Box::new(QuantizedMatmul::<f32>::default());
+                } else {
+                    panic!("Quantized weight {consumer:?} is an input to a node that isn't a matmul or gather ({op:?})");
                 }
             }
         }
-    }
-}
-
-/// Pattern recognition the pass needs when no dense HIP compiler ran before it.
-pub(crate) mod patterns {
-    use luminal::{op::{Mul, SumReduce}, prelude::*};
-    use petgraph::{visit::EdgeRef, Direction};
-
-    pub enum Use {
-        Matmul(NodeIndex),
-        Gather { node: NodeIndex, embed_dim: usize, vocab: usize },
-        Other(String),
-    }
-
-    /// `consumer` is the node that reads the weight.  A matmul is `Mul` whose only reader is `SumReduce` over the
-    /// last axis; the pair is collapsed onto the `SumReduce` node, which keeps its outgoing edges.
-    pub fn classify(graph: &mut Graph, consumer: NodeIndex) -> Use {
-        let is_mul = graph.node_weight(consumer).map(|o| o.as_any().is::<Mul>()).unwrap_or(false);
-        if is_mul {
-            let readers: Vec<_> = graph.edges_directed(consumer, Direction::Outgoing).map(|e| e.target()).collect();
-            if let [reduce] = readers[..] {
-                let over_last = graph.node_weight(reduce).and_then(|o| o.as_any().downcast_ref::<SumReduce>().map(|s| s.0));
-                if let Some(axis) = over_last {
-                    let srcs = graph.get_sources(consumer);
-                    if axis + 1 == srcs[0].2.len() {
-                        // Re-point the Mul's inputs at the SumReduce node with the un-expanded shapes, then drop the Mul.
-                        let (mut a, mut b) = (srcs[0].2, srcs[1].2);
-                        a.remove_dim(a.len() - 2);
-                        b.remove_dim(0);
-                        b.permute(&[1, 0]);
-                        graph.graph.remove_node(consumer);
-                        graph.graph.add_edge(srcs[0].0, reduce, Dependency::Data { input_order: 0, output_order: srcs[0].1, shape: a });
-                        graph.graph.add_edge(srcs[1].0, reduce, Dependency::Data { input_order: 1, output_order: srcs[1].1, shape: b });
-                        return Use::Matmul(reduce);
-                    }
-                }
-            }
-        }
-        let name = format!("{:?}", graph.node_weight(consumer));
-        Use::Other(name)
     }
 }
