@@ -107,6 +107,30 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
                                      int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu,
                                      int waves_per_block, void *stream);
 
+/* Batch-1 decode matvec with fusions.  No counterpart in the reference, whose graph runs
+ * each piece as its own operator (RMSNorm: examples/llama/src/model.rs:150-160 through
+ * luminal_nn, the sibling projections model.rs:95-100 and :24-32, the residual adds
+ * model.rs:163-172); a compiler pass that finds those patterns around QuantizedMatmul
+ * nodes emits one call instead.
+ *   count (1..4) weights planar_dev[i] of shape (n[i], K) read the same x (K floats) and
+ *   write y_dev[i] (n[i] floats);
+ *   norm_weight_dev != NULL: x is replaced by x * (1/sqrt(mean(x^2) + eps)) * norm_weight;
+ *   epilogue 0: y = W x;  1: y = residual + W x (count == 1; y may be residual itself);
+ *   2: rows are (gate, up) pairs, row 2j = gate_j and row 2j+1 = up_j, and
+ *      y[j] = up_j * gate_j / (1 + exp(-gate_j)) for j < n/2 (n even).
+ * K must be a multiple of 1024 and at most 16384 (LHIP_ERR_UNSUPPORTED otherwise: run
+ * the separate operators).  x and norm_weight 16-byte aligned. */
+lhip_status lhip_q8_0_matvec_fused_f32(const void *const *planar_dev, float *const *y_dev, const int64_t *n, int count,
+                                       const float *x_dev, int64_t k, const float *norm_weight_dev, float eps,
+                                       const float *residual_dev, int epilogue, void *stream);
+/* Same with an explicit launch shape: (rows_per_wave, k_unroll, waves_per_block) one of
+ * (2,4,4) (1,2,4) (2,2,4) (1,1,4) (2,1,4) (1,2,16) (2,2,8) (1,1,16) (2,1,8), epilogue 2
+ * needs rows_per_wave 2; blocks_per_cu in 1..16. */
+lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float *const *y_dev, const int64_t *n,
+                                           int count, const float *x_dev, int64_t k, const float *norm_weight_dev,
+                                           float eps, const float *residual_dev, int epilogue, int rows_per_wave,
+                                           int k_unroll, int waves_per_block, int blocks_per_cu, void *stream);
+
 /* Prefill GEMM: y[m][n] = sum_k x[m][k] * W[n][k] with bf16 activations
  * (x (m, K) row-major, 16-byte aligned), f32 accumulation on the matrix cores
  * and bf16 output (y (m, N) row-major).  The reference has no bf16 type and no
@@ -194,8 +218,21 @@ lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v
 lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
                                float *out_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
                                int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
-/* out[r][j] = up * swish(gate) with gate = gate_up[r][j], up = gate_up[r][f + j] (model.rs:24-32). */
-lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, void *stream);
+/* Batch-1 decode: rotary + cache append + attention of the previous two operators as one call, for one new
+ * token at position *pos_dev (model.rs:52-72, :108-139).  qkv_dev holds the un-rotated fused row
+ * [(q_heads + 2*kv_heads)*head_dim] and is not modified; out_dev [q_heads*head_dim].  The keys of every KV head
+ * are split over several workgroups whose partial softmax states meet in workspace_dev
+ * (lhip_attention_decode_workspace_nbytes bytes, 256-byte aligned, contents irrelevant on entry; calls sharing a
+ * workspace must be ordered on one stream) and are merged by a second small kernel.  Built for head_dim 64 or 128 and
+ * q_heads / kv_heads in {1, 2, 4, 8}: LHIP_ERR_UNSUPPORTED otherwise (the workspace size is then 0). */
+size_t lhip_attention_decode_workspace_nbytes(int64_t q_heads, int64_t kv_heads, int64_t head_dim);
+lhip_status lhip_attention_decode_f32(const float *qkv_dev, float *k_cache_dev, float *v_cache_dev, float *out_dev,
+                                      const int32_t *pos_dev, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
+                                      int64_t max_seq, float theta, void *workspace_dev, void *stream);
+/* out[r][j] = up * swish(gate) (model.rs:24-32) with gate = gate_up[r][j], up = gate_up[r][f + j], or, with
+ * interleaved != 0, gate = gate_up[r][2j], up = gate_up[r][2j + 1] (the row order the fused matvec epilogue uses). */
+lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,
+                            void *stream);
 /* Element-wise casts between f32 and bf16 (round to nearest even), for feeding f32
  * activations to the bf16 prefill GEMM. */
 lhip_status lhip_cast_f32_to_bf16(const float *x_dev, void *y_dev, int64_t n, void *stream);

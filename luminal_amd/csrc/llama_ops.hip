@@ -243,12 +243,13 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(const float *__
 
 // out[s][j] = up * swish(gate), gate = gu[s][j], up = gu[s][f + j]   (model.rs:24-32)
 __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gu, float *__restrict__ out, int f,
-                                                     size_t total) {
+                                                     size_t total, int interleaved) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= total) return;
     const size_t s = i / f;
     const int j = static_cast<int>(i - s * f);
-    const float g = gu[s * 2 * f + j], u = gu[s * 2 * f + f + j];
+    const float g = gu[s * 2 * f + (interleaved ? 2 * j : j)];
+    const float u = gu[s * 2 * f + (interleaved ? 2 * j + 1 : f + j)];
     out[i] = u * (g * (1.0f / (1.0f + expf(-g))));
 }
 
@@ -393,12 +394,13 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
     return LHIP_OK;
 }
 
-lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, void *stream) {
+lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,
+                            void *stream) {
     if (!gate_up_dev || !out_dev) return LHIP_ERR_NULL_PTR;
     if (rows <= 0 || f <= 0 || rows > kMaxDim || f > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     const size_t total = static_cast<size_t>(rows) * static_cast<size_t>(f);
     hipLaunchKernelGGL(swiglu_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       gate_up_dev, out_dev, static_cast<int>(f), total);
+                       gate_up_dev, out_dev, static_cast<int>(f), total, interleaved);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }

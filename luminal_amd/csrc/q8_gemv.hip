@@ -19,6 +19,7 @@
 //     16 lanes and four readlanes; there are no atomics and the result does
 //     not depend on the launch shape of other rows.
 #include <hip/hip_fp16.h>
+#include <limits.h>
 
 #include "common.h"
 
@@ -295,6 +296,186 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_pipe_kernel(const int8_t *
     }
 }
 
+// ---------------------------------------------------------------------------
+// Fused decode variant of the pipelined kernel (batch 1):
+//   * up to four weights that read the same activations run as one launch
+//     (sibling projections q|k|v, gate|up): one launch overhead, one staging
+//     of x per workgroup, and the short problems fill the tail of the long one;
+//   * optional RMS-norm prologue: y = W (x * g) / sqrt(mean(x^2) + eps), the
+//     sum of squares recomputed by every workgroup while it stages x, which
+//     removes the norm launch and its round trip through HBM;
+//   * epilogues: none, y = residual + W x, or SwiGLU on interleaved rows
+//     (row 2j = gate_j, row 2j+1 = up_j, y[j] = up * gate * sigmoid(gate)).
+// The per-row arithmetic is that of the plain kernel, so results agree with
+// it bit for bit when no prologue or epilogue is selected.
+// ---------------------------------------------------------------------------
+
+constexpr int kMaxGroup = 4;
+
+struct GemvGroup {
+    const int8_t *qs[kMaxGroup];
+    const unsigned short *ds[kMaxGroup];
+    float *y[kMaxGroup];
+    int n[kMaxGroup];
+    int group_end[kMaxGroup];  // running total of row groups; unused entries hold INT_MAX
+};
+
+struct GemvFuse {
+    const float *norm_w;    // NORM: gain of the RMS norm, K floats
+    float eps;
+    const float *residual;  // EPI_ADD: N floats (single weight only)
+};
+
+enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+
+struct Located {
+    const int8_t *qs;
+    const unsigned short *ds;
+    float *y;
+    int n;
+    int row0;
+};
+
+// Row group -> (weight, first row).  All operands are wave-uniform.
+template <int R>
+__device__ __forceinline__ Located locate(const GemvGroup &p, int gg) {
+    Located o{p.qs[0], p.ds[0], p.y[0], p.n[0], gg * R};
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i) {
+        if (gg >= p.group_end[i - 1]) {
+            o.qs = p.qs[i];
+            o.ds = p.ds[i];
+            o.y = p.y[i];
+            o.n = p.n[i];
+            o.row0 = (gg - p.group_end[i - 1]) * R;
+        }
+    }
+    return o;
+}
+
+template <int R, int S, int W, bool NORM, int EPI>
+__global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p, const GemvFuse f,
+                                                               const float *__restrict__ x, int k, int n_groups) {
+    static_assert(EPI != EPI_SWIGLU || R % 2 == 0, "SwiGLU pairs live in one wave");
+    extern __shared__ float4 xs4[];
+    __shared__ float red[W];
+    const unsigned lane = threadIdx.x & 63u;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave_global = blockIdx.x * W + wave;
+    const int total_waves = gridDim.x * W;
+
+    const int chunks = k / (S * 1024);
+    const int my_groups = wave_global < n_groups ? (n_groups - wave_global + total_waves - 1) / total_waves : 0;
+    const int T = my_groups * chunks;
+
+    StepBuf<R, S> a, b;
+    {
+        const Located l = locate<R>(p, wave_global < n_groups ? wave_global : 0);
+        load_step(a, l.qs, l.ds, l.row0, l.n, k, 0, lane, T > 0);
+    }
+
+    // The norm's scalar factor commutes with the matrix product, so x * g is staged at once and the row sums
+    // are multiplied by 1/sqrt(mean(x^2) + eps) at the end: the sum of squares rides on the staging loads and
+    // is published by the staging barrier.
+    {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
+        const float4 *g4 = reinterpret_cast<const float4 *>(f.norm_w);
+        const int k4 = k >> 2;
+        float ss = 0.f;
+#pragma unroll 4
+        for (int i = threadIdx.x; i < k4; i += W * 64) {
+            const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
+            float4 v = x4[src];
+            if (NORM) {
+                const float4 g = g4[src];
+                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                v = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+            }
+            xs4[i] = v;
+        }
+        if (NORM) {
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+        }
+    }
+    __syncthreads();
+    if (T == 0) return;
+    float scale = 1.f;
+    if (NORM) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < W; ++w) total += red[w];
+        scale = 1.0f / sqrtf(total / static_cast<float>(k) + f.eps);
+    }
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+    int t = 0, g = wave_global, c = 0;
+    auto next = [&](int &gg, int &cc) {
+        if (++cc == chunks) {
+            cc = 0;
+            gg += total_waves;
+        }
+    };
+    auto issue = [&](StepBuf<R, S> &buf, int gg, int cc, bool live) {
+        const Located l = locate<R>(p, live ? gg : 0);
+        load_step(buf, l.qs, l.ds, l.row0, l.n, k, cc * S, lane, live);
+    };
+    auto finish_group = [&](int gg) {
+        const Located l = locate<R>(p, gg);
+        float sum[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            sum[r] = wave_sum(acc[r]);
+            if (NORM) sum[r] *= scale;
+            acc[r] = 0.f;
+        }
+        if (EPI == EPI_SWIGLU) {
+            float out = 0.f;
+#pragma unroll
+            for (int j = 0; j < R / 2; ++j) {
+                const float gate = sum[2 * j], up = sum[2 * j + 1];
+                const float v = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                if (lane == static_cast<unsigned>(j)) out = v;
+            }
+            const int pair = l.row0 / 2 + static_cast<int>(lane);
+            if (lane < static_cast<unsigned>(R / 2) && 2 * pair + 1 < l.n) l.y[pair] = out;
+        } else {
+            float out = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (lane == static_cast<unsigned>(r)) out = sum[r];
+            const int row = l.row0 + static_cast<int>(lane);
+            if (lane < static_cast<unsigned>(R) && row < l.n) {
+                if (EPI == EPI_ADD) out += f.residual[row];
+                l.y[row] = out;
+            }
+        }
+    };
+
+    while (true) {
+        int g1 = g, c1 = c;
+        next(g1, c1);
+        issue(b, g1, c1, t + 1 < T);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(a, xs4, c * S, lane, acc);
+        if (c == chunks - 1) finish_group(g);
+        if (++t >= T) break;
+        g = g1;
+        c = c1;
+        next(g1, c1);
+        issue(a, g1, c1, t + 1 < T);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(b, xs4, c * S, lane, acc);
+        if (c == chunks - 1) finish_group(g);
+        if (++t >= T) break;
+        g = g1;
+        c = c1;
+    }
+}
+
 constexpr int kNumCUs = 256;
 constexpr int kMaxLdsK = 16384;  // 64 KiB of staged activations
 
@@ -390,6 +571,64 @@ static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_
     }
 }
 
+template <int R, int S, int W, bool NORM, int EPI>
+static lhip_status launch_fused(const GemvGroup &p, const GemvFuse &f, const float *x, int k, int n_groups,
+                                int blocks_per_cu, hipStream_t s) {
+    int grid = (n_groups + W - 1) / W;
+    const int cap = kNumCUs * blocks_per_cu;
+    if (grid > cap) grid = cap;
+    hipLaunchKernelGGL((q8_gemv_fused_kernel<R, S, W, NORM, EPI>), dim3(static_cast<unsigned>(grid)), dim3(W * 64),
+                       static_cast<size_t>(k) * sizeof(float), s, p, f, x, k, n_groups);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+template <int R, int S, int W>
+static lhip_status launch_fused_variant(bool norm, int epi, const GemvGroup &p, const GemvFuse &f, const float *x, int k,
+                                        int n_groups, int blocks_per_cu, hipStream_t s) {
+    if (epi == EPI_SWIGLU) {
+        if constexpr (R % 2 == 0) {
+            return norm ? launch_fused<R, S, W, true, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s)
+                        : launch_fused<R, S, W, false, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s);
+        } else {
+            return LHIP_ERR_UNSUPPORTED;
+        }
+    }
+    if (epi == EPI_ADD)
+        return norm ? launch_fused<R, S, W, true, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s)
+                    : launch_fused<R, S, W, false, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s);
+    return norm ? launch_fused<R, S, W, true, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s)
+                : launch_fused<R, S, W, false, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s);
+}
+
+// Launch shapes of the fused kernel: (rows per wave, slices per step, waves per workgroup, workgroups per CU).
+static lhip_status dispatch_fused(int r, int sl, int w, int bpc, bool norm, int epi, const GemvGroup &p,
+                                  const GemvFuse &f, const float *x, int k, int n_groups, hipStream_t s) {
+#define LHIP_CASE(R, S, W) \
+    if (r == R && sl == S && w == W) return launch_fused_variant<R, S, W>(norm, epi, p, f, x, k, n_groups, bpc, s);
+    LHIP_CASE(2, 4, 4) LHIP_CASE(1, 2, 4) LHIP_CASE(2, 2, 4) LHIP_CASE(1, 1, 4) LHIP_CASE(2, 1, 4)
+    LHIP_CASE(1, 2, 16) LHIP_CASE(2, 2, 8) LHIP_CASE(1, 1, 16) LHIP_CASE(2, 1, 8)
+#undef LHIP_CASE
+    return LHIP_ERR_UNSUPPORTED;
+}
+
+// Default launch shape of the fused kernel for n_total rows (all weights together).
+static void choose_fused(int64_t n_total, int k, int epi, int *r, int *sl, int *w, int *bpc) {
+    const int slices = k % 4096 == 0 ? 4 : (k % 2048 == 0 ? 2 : 1);
+    const int fit = (160 * 1024) / (k * 4);
+    if (n_total >= 16384 && slices == 4 && fit >= 1) {
+        *r = 2, *sl = 4, *w = 4, *bpc = 1;
+        return;
+    }
+    const bool pairs = epi == EPI_SWIGLU;
+    *sl = slices >= 2 ? 2 : 1;
+    if (fit >= 3) {
+        *r = pairs ? 2 : 1, *w = 4, *bpc = pairs ? 2 : 3;
+    } else {
+        *r = pairs ? 2 : 1, *w = pairs ? 8 : 16, *bpc = 1;
+    }
+}
+
 static lhip_status check_args(const void *planar, const float *x, float *y, int64_t m, int64_t n, int64_t k) {
     if (!planar || !x || !y) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_q8_shape(n, k)) return s;
@@ -421,6 +660,58 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
     int r, u, b, w;
     choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
     return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, b, w, stream);
+}
+
+lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float *const *y_dev, const int64_t *n,
+                                           int count, const float *x_dev, int64_t k, const float *norm_weight_dev,
+                                           float eps, const float *residual_dev, int epilogue, int rows_per_wave,
+                                           int k_unroll, int waves_per_block, int blocks_per_cu, void *stream) {
+    if (!planar_dev || !y_dev || !n || !x_dev) return LHIP_ERR_NULL_PTR;
+    if (count < 1 || count > kMaxGroup) return LHIP_ERR_INVALID_SHAPE;
+    if (epilogue != EPI_NONE && epilogue != EPI_ADD && epilogue != EPI_SWIGLU) return LHIP_ERR_UNSUPPORTED;
+    if (epilogue == EPI_ADD && (!residual_dev || count != 1)) return residual_dev ? LHIP_ERR_UNSUPPORTED : LHIP_ERR_NULL_PTR;
+    if (!aligned(x_dev, 16) || (norm_weight_dev && !aligned(norm_weight_dev, 16))) return LHIP_ERR_MISALIGNED;
+    if (k <= 0 || k % 1024 != 0 || k > kMaxLdsK) return k > 0 && k % 32 == 0 ? LHIP_ERR_UNSUPPORTED : LHIP_ERR_INVALID_SHAPE;
+    if (rows_per_wave < 1 || k_unroll < 1 || blocks_per_cu < 1 || blocks_per_cu > 16 || k % (k_unroll * 1024) != 0)
+        return LHIP_ERR_UNSUPPORTED;
+    GemvGroup p;
+    int64_t groups = 0;
+    for (int i = 0; i < kMaxGroup; ++i) {
+        if (i < count) {
+            if (!planar_dev[i] || !y_dev[i]) return LHIP_ERR_NULL_PTR;
+            if (lhip_status st = check_q8_shape(n[i], k)) return st;
+            if (epilogue == EPI_SWIGLU && n[i] % 2 != 0) return LHIP_ERR_INVALID_SHAPE;
+            if (!aligned(planar_dev[i], 256) || !aligned(y_dev[i], 4)) return LHIP_ERR_MISALIGNED;
+            auto *base = static_cast<const uint8_t *>(planar_dev[i]);
+            p.qs[i] = reinterpret_cast<const int8_t *>(base);
+            p.ds[i] = reinterpret_cast<const unsigned short *>(base + q8_scale_offset(n[i], k));
+            p.y[i] = y_dev[i];
+            p.n[i] = static_cast<int>(n[i]);
+            groups += (n[i] + rows_per_wave - 1) / rows_per_wave;
+            if (groups > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+            p.group_end[i] = static_cast<int>(groups);
+        } else {
+            p.qs[i] = p.qs[0], p.ds[i] = p.ds[0], p.y[i] = p.y[0], p.n[i] = p.n[0];
+            p.group_end[i] = INT_MAX;
+        }
+    }
+    const GemvFuse f{norm_weight_dev, eps, residual_dev};
+    return dispatch_fused(rows_per_wave, k_unroll, waves_per_block, blocks_per_cu, norm_weight_dev != nullptr, epilogue,
+                          p, f, x_dev, static_cast<int>(k), static_cast<int>(groups), as_stream(stream));
+}
+
+lhip_status lhip_q8_0_matvec_fused_f32(const void *const *planar_dev, float *const *y_dev, const int64_t *n, int count,
+                                       const float *x_dev, int64_t k, const float *norm_weight_dev, float eps,
+                                       const float *residual_dev, int epilogue, void *stream) {
+    if (!n) return LHIP_ERR_NULL_PTR;
+    if (count < 1 || count > kMaxGroup) return LHIP_ERR_INVALID_SHAPE;
+    if (k <= 0 || k % 1024 != 0 || k > kMaxLdsK) return k > 0 && k % 32 == 0 ? LHIP_ERR_UNSUPPORTED : LHIP_ERR_INVALID_SHAPE;
+    int64_t total = 0;
+    for (int i = 0; i < count; ++i) total += n[i] > 0 ? n[i] : 0;
+    int r, sl, w, bpc;
+    choose_fused(total, static_cast<int>(k), epilogue, &r, &sl, &w, &bpc);
+    return lhip_q8_0_matvec_fused_f32_cfg(planar_dev, y_dev, n, count, x_dev, k, norm_weight_dev, eps, residual_dev,
+                                          epilogue, r, sl, w, bpc, stream);
 }
 
 }  // extern "C"

@@ -191,10 +191,10 @@ def llama_tensor_names(layers: int):
 
 def q8_load(path, cfg, device="cuda:0") -> dict:
     """Reads a Llama GGUF (linears Q8_0, norms and embedding F32) into the weight dict of luminal_amd.llama.LlamaQ8.
-    Q8_0 bytes are uploaded raw and re-arranged on the device; q|k|v and gate|up are row-concatenated."""
+    Q8_0 bytes are uploaded raw and re-arranged on the device; q|k|v are row-concatenated, gate and up rows interleaved."""
     import torch
 
-    from .llama import fuse_rows
+    from .llama import fuse_rows, interleave_rows
     from .quantized import Q8Weight
 
     hd = cfg.head_dim
@@ -227,7 +227,7 @@ def q8_load(path, cfg, device="cuda:0") -> dict:
                             raw(b + "attn_v.weight", cfg.kv_heads * hd, cfg.dim))
             w[f"{i}.qkv"] = Q8Weight.from_raw(qkv, cfg.qkv_rows, cfg.dim, device)
             w[f"{i}.o"] = Q8Weight.from_raw(raw(b + "attn_output.weight", cfg.dim, cfg.dim), cfg.dim, cfg.dim, device)
-            gu = fuse_rows(raw(b + "ffn_gate.weight", cfg.ffn, cfg.dim), raw(b + "ffn_up.weight", cfg.ffn, cfg.dim))
+            gu = interleave_rows(raw(b + "ffn_gate.weight", cfg.ffn, cfg.dim), raw(b + "ffn_up.weight", cfg.ffn, cfg.dim), cfg.dim)
             w[f"{i}.gate_up"] = Q8Weight.from_raw(gu, 2 * cfg.ffn, cfg.dim, device)
             w[f"{i}.down"] = Q8Weight.from_raw(raw(b + "ffn_down.weight", cfg.dim, cfg.ffn), cfg.dim, cfg.ffn, device)
     return w

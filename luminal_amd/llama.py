@@ -4,8 +4,11 @@ Host-side counterpart of examples/llama/src/{model.rs,main.rs}: the same layer
 stack and generation loop (prefill, then greedy decode with a KV cache), with
 every tensor op running in libluminal_hip.so.  torch holds the device buffers
 and, optionally, replays a captured HIP graph of one decode step.  Linear
-weights are Q8_0; q|k|v and gate|up are stored row-concatenated so each is one
-matvec (row-wise the same arithmetic as the reference's separate matmuls).
+weights are Q8_0; q|k|v are stored row-concatenated and gate/up row-interleaved
+(row 2j = gate_j, row 2j+1 = up_j) so each is one matvec (row-wise the same
+arithmetic as the reference's separate matmuls).  Batch-1 decode runs six
+launches per layer: RMS norm is folded into the qkv and gate/up matvecs, SwiGLU
+into the gate/up epilogue and the residual adds into the o and down epilogues.
 """
 from __future__ import annotations
 
@@ -15,7 +18,7 @@ import numpy as np
 import torch
 
 from . import capi
-from .quantized import Q8Weight
+from .quantized import FusedMatvec, Q8Weight
 
 
 @dataclass(frozen=True)
@@ -50,7 +53,7 @@ class LlamaQ8:
     def __init__(self, cfg: LlamaConfig, weights: dict, max_seq: int, device="cuda:0"):
         """weights: 'embed' f32 (vocab, dim); 'out_norm' f32 (dim); 'lm_head' Q8Weight (vocab, dim); and per
         layer i: f'{i}.attn_norm', f'{i}.ffn_norm' f32 (dim); f'{i}.qkv' Q8Weight (qkv_rows, dim);
-        f'{i}.o' (dim, dim); f'{i}.gate_up' (2*ffn, dim); f'{i}.down' (dim, ffn)."""
+        f'{i}.o' (dim, dim); f'{i}.gate_up' (2*ffn, dim), gate and up rows interleaved; f'{i}.down' (dim, ffn)."""
         self.cfg, self.w, self.max_seq, self.dev = cfg, weights, max_seq, torch.device(device)
         self.lib = capi.load_library()
         kv = (cfg.kv_heads, max_seq, cfg.head_dim)
@@ -61,6 +64,11 @@ class LlamaQ8:
         self.tok_i = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self._bufs = {}
         self._graph = None
+        # The fused matvec stages K activations in LDS in slices of 1024.
+        self.fused_decode = all(k % 1024 == 0 and k <= 16384 for k in (cfg.dim, cfg.ffn))
+        self._plans = None
+        ws = self.lib.lhip_attention_decode_workspace_nbytes(cfg.q_heads, cfg.kv_heads, cfg.head_dim)
+        self._attn_ws = torch.empty(ws, dtype=torch.uint8, device=self.dev) if ws else None
 
     # ---- buffers -----------------------------------------------------------
     def _buf(self, name, shape, dtype=torch.float32):
@@ -113,16 +121,19 @@ class LlamaQ8:
             else:  # residual of the previous layer's MLP, fused into this norm
                 self._norm(h, dn, h, w[f"{i}.attn_norm"], n, s)
             self._matmul(w[f"{i}.qkv"], n, qkv, s, bf16)
-            capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
-                                                   self.v_cache[i].data_ptr(), self.pos.data_ptr(), s, cfg.q_heads,
-                                                   cfg.kv_heads, hd, self.max_seq, cfg.theta, _s()), "rope")
-            capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
-                                              att.data_ptr(), self.pos.data_ptr(), s, cfg.q_heads, cfg.kv_heads, hd,
-                                              self.max_seq, _s()), "attention")
+            if s == 1:
+                self._attend_one(i, qkv, att)
+            else:
+                capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                       self.v_cache[i].data_ptr(), self.pos.data_ptr(), s, cfg.q_heads,
+                                                       cfg.kv_heads, hd, self.max_seq, cfg.theta, _s()), "rope")
+                capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                  self.v_cache[i].data_ptr(), att.data_ptr(), self.pos.data_ptr(), s,
+                                                  cfg.q_heads, cfg.kv_heads, hd, self.max_seq, _s()), "attention")
             self._matmul(w[f"{i}.o"], att, o, s, bf16)
             self._norm(h, o, h, w[f"{i}.ffn_norm"], n, s)          # h += attn out; n = norm(h)
             self._matmul(w[f"{i}.gate_up"], n, gu, s, bf16)
-            capi.check(lib.lhip_swiglu_f32(gu.data_ptr(), act.data_ptr(), s, cfg.ffn, _s()), "swiglu")
+            capi.check(lib.lhip_swiglu_f32(gu.data_ptr(), act.data_ptr(), s, cfg.ffn, 1, _s()), "swiglu")
             self._matmul(w[f"{i}.down"], act, dn, s, bf16)
         self._norm(h, dn, h, w["out_norm"], n, s)                    # last residual + final norm
         if all_logits:
@@ -133,6 +144,59 @@ class LlamaQ8:
         last = n[s - 1]
         self._matmul(w["lm_head"], last, logits, 1, False)  # only the last position is read (main.rs:58-61)
         return logits
+
+    def _build_plans(self):
+        cfg, w = self.cfg, self.w
+        h = self._buf("h", (1, cfg.dim)).view(-1)
+        qkv = self._buf("qkv", (1, cfg.qkv_rows)).view(-1)
+        att = self._buf("att", (1, cfg.dim)).view(-1)
+        act = self._buf("act", (1, cfg.ffn)).view(-1)
+        logits = self._buf("logits", (cfg.vocab,))
+        plans = []
+        for i in range(cfg.layers):
+            plans.append((
+                FusedMatvec([w[f"{i}.qkv"]], [qkv], norm_weight=w[f"{i}.attn_norm"], eps=cfg.eps),
+                FusedMatvec([w[f"{i}.o"]], [h], residual=h, epilogue=FusedMatvec.EPI_ADD),
+                FusedMatvec([w[f"{i}.gate_up"]], [act], norm_weight=w[f"{i}.ffn_norm"], eps=cfg.eps,
+                            epilogue=FusedMatvec.EPI_SWIGLU),
+                FusedMatvec([w[f"{i}.down"]], [h], residual=h, epilogue=FusedMatvec.EPI_ADD)))
+        head = FusedMatvec([w["lm_head"]], [logits], norm_weight=w["out_norm"], eps=cfg.eps)
+        self._plans = (plans, head, h, qkv, att, act, logits)
+
+    def forward_decode(self, token_f32: torch.Tensor):
+        """One token at position pos through the fused batch-1 path; returns the logits (vocab,)."""
+        cfg, lib = self.cfg, self.lib
+        if not self.fused_decode:
+            return self.forward(token_f32, 1)
+        if self._plans is None:
+            self._build_plans()
+        plans, head, h, qkv, att, act, logits = self._plans
+        capi.check(lib.lhip_gather_rows_f32(self.w["embed"].data_ptr(), token_f32.data_ptr(), h.data_ptr(), 1,
+                                            cfg.vocab, cfg.dim, _s()), "lhip_gather_rows_f32")
+        for i, (p_qkv, p_o, p_gu, p_down) in enumerate(plans):
+            p_qkv.run(h)                                   # qkv = Wqkv norm(h)
+            self._attend_one(i, qkv, att)
+            p_o.run(att)                                   # h += Wo att
+            p_gu.run(h)                                    # act = up * swish(gate) of Wgu norm(h)
+            p_down.run(act)                                # h += Wdown act
+        head.run(h)                                        # logits = Wout norm(h)
+        return logits
+
+    def _attend_one(self, i, qkv, att):
+        """Rotary, cache append and attention for one new token of layer i."""
+        cfg, lib = self.cfg, self.lib
+        if self._attn_ws is not None:
+            capi.check(lib.lhip_attention_decode_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                     self.v_cache[i].data_ptr(), att.data_ptr(), self.pos.data_ptr(),
+                                                     cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.max_seq, cfg.theta,
+                                                     self._attn_ws.data_ptr(), _s()), "lhip_attention_decode_f32")
+            return
+        capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                               self.pos.data_ptr(), 1, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
+                                               self.max_seq, cfg.theta, _s()), "rope")
+        capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                          att.data_ptr(), self.pos.data_ptr(), 1, cfg.q_heads, cfg.kv_heads,
+                                          cfg.head_dim, self.max_seq, _s()), "attention")
 
     def _pick(self, logits, advance):
         capi.check(self.lib.lhip_argmax_f32(logits.data_ptr(), self.cfg.vocab, self.tok.data_ptr(),
@@ -146,7 +210,7 @@ class LlamaQ8:
         return logits
 
     def decode_step(self):
-        logits = self.forward(self.tok, 1)
+        logits = self.forward_decode(self.tok)
         self._pick(logits, 1)
         return logits
 
@@ -183,6 +247,14 @@ class LlamaQ8:
 def fuse_rows(*raws: np.ndarray) -> np.ndarray:
     """Row-concatenate Q8_0 weights with the same K: their raw block streams simply follow each other."""
     return np.concatenate([np.ascontiguousarray(r, dtype=np.uint8).reshape(-1) for r in raws])
+
+
+def interleave_rows(a: np.ndarray, b: np.ndarray, k: int) -> np.ndarray:
+    """Raw Q8_0 block streams of two (n, k) weights -> the (2n, k) weight whose rows alternate a_0, b_0, a_1, ..."""
+    row = k // 32 * 34
+    a = np.ascontiguousarray(a, dtype=np.uint8).reshape(-1, row)
+    b = np.ascontiguousarray(b, dtype=np.uint8).reshape(-1, row)
+    return np.stack([a, b], axis=1).reshape(-1)
 
 
 def random_weights(cfg: LlamaConfig, seed: int, device="cuda:0", scale_sigma: float | None = None) -> dict:

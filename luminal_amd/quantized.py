@@ -146,3 +146,49 @@ class QuantizedGather:
             st = lib.lhip_q8_0_gather_f32(_ptr(w.planar), _ptr(idx), _ptr(out), idx.numel(), w.n, w.k, _stream())
         capi.check(st, "lhip_q8_0_gather_f32")
         return out
+
+
+class FusedMatvec:
+    """Batch-1 decode: up to four Q8_0 weights that read the same (K,) f32 activation in one launch, with an optional
+    RMS-norm prologue (norm_weight, eps) and epilogue (EPI_ADD: y = residual + W x; EPI_SWIGLU: rows are (gate, up)
+    pairs and y[j] = up_j * swish(gate_j)).  A plan object: the operand addresses are fixed at construction, `run`
+    only launches (lhip_q8_0_matvec_fused_f32)."""
+
+    EPI_NONE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+
+    def __init__(self, weights, outs, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
+                 residual: torch.Tensor | None = None, epilogue: int = 0, cfg: tuple | None = None):
+        import ctypes as C
+
+        if len(weights) != len(outs) or not 1 <= len(weights) <= 4:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "FusedMatvec", "1..4 weights, one output each")
+        k = weights[0].k
+        for w, y in zip(weights, outs):
+            want = w.n // 2 if epilogue == self.EPI_SWIGLU else w.n
+            if w.k != k or y.dtype != torch.float32 or y.numel() != want or not y.is_contiguous():
+                raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "FusedMatvec", "weights share K; outputs f32 (n,)")
+        if norm_weight is not None and (norm_weight.dtype != torch.float32 or norm_weight.numel() != k):
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "FusedMatvec", "norm weight is f32 (K,)")
+        if residual is not None and (residual.dtype != torch.float32 or residual.numel() != weights[0].n):
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "FusedMatvec", "residual is f32 (n,)")
+        self.k, self.count = k, len(weights)
+        self._keep = (list(weights), list(outs), norm_weight, residual)
+        self._w = (C.c_void_p * self.count)(*[w.planar.data_ptr() for w in weights])
+        self._y = (C.c_void_p * self.count)(*[y.data_ptr() for y in outs])
+        self._n = (C.c_int64 * self.count)(*[w.n for w in weights])
+        self._norm = norm_weight.data_ptr() if norm_weight is not None else None
+        self._res = residual.data_ptr() if residual is not None else None
+        self.eps, self.epilogue, self.cfg = float(eps), int(epilogue), cfg
+        self.lib = capi.load_library()
+
+    def run(self, x: torch.Tensor) -> None:
+        if x.dtype != torch.float32 or not x.is_cuda or x.numel() != self.k:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "FusedMatvec", f"activation must be f32 ({self.k},)")
+        if self.cfg:
+            st = self.lib.lhip_q8_0_matvec_fused_f32_cfg(self._w, self._y, self._n, self.count, _ptr(x), self.k,
+                                                         self._norm, self.eps, self._res, self.epilogue, *self.cfg,
+                                                         _stream())
+        else:
+            st = self.lib.lhip_q8_0_matvec_fused_f32(self._w, self._y, self._n, self.count, _ptr(x), self.k,
+                                                     self._norm, self.eps, self._res, self.epilogue, _stream())
+        capi.check(st, "lhip_q8_0_matvec_fused_f32")

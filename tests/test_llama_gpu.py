@@ -9,7 +9,7 @@ torch = pytest.importorskip("torch")
 
 from conftest import rel_err  # noqa: E402
 from luminal_amd import capi, synth  # noqa: E402
-from luminal_amd.llama import LlamaConfig, LlamaQ8, fuse_rows  # noqa: E402
+from luminal_amd.llama import LlamaConfig, LlamaQ8, fuse_rows, interleave_rows  # noqa: E402
 from luminal_amd.quantized import Q8Weight  # noqa: E402
 from oracle import llama_oracle as lo  # noqa: E402
 
@@ -52,7 +52,7 @@ def build_model(oracle, cfg, seed, max_seq=64):
         w[f"{i}.qkv"] = Q8Weight.from_raw(fuse_rows(raws[f"{i}.q"], raws[f"{i}.k"], raws[f"{i}.v"]), cfg.qkv_rows,
                                           cfg.dim, DEV)
         w[f"{i}.o"] = Q8Weight.from_raw(raws[f"{i}.o"], cfg.dim, cfg.dim, DEV)
-        w[f"{i}.gate_up"] = Q8Weight.from_raw(fuse_rows(raws[f"{i}.gate"], raws[f"{i}.up"]), 2 * cfg.ffn, cfg.dim, DEV)
+        w[f"{i}.gate_up"] = Q8Weight.from_raw(interleave_rows(raws[f"{i}.gate"], raws[f"{i}.up"], cfg.dim), 2 * cfg.ffn, cfg.dim, DEV)
         w[f"{i}.down"] = Q8Weight.from_raw(raws[f"{i}.down"], cfg.dim, cfg.ffn, DEV)
     return LlamaQ8(cfg, w, max_seq, DEV), wf
 
@@ -116,7 +116,7 @@ def test_rope_attention_swiglu_gather_argmax():
     # swiglu
     gu = rng.standard_normal((3, 2 * 96)).astype(np.float32)
     o = torch.empty((3, 96), dtype=torch.float32, device=DEV)
-    assert lib.lhip_swiglu_f32(torch.from_numpy(gu).to(DEV).data_ptr(), o.data_ptr(), 3, 96, s()) == 0
+    assert lib.lhip_swiglu_f32(torch.from_numpy(gu).to(DEV).data_ptr(), o.data_ptr(), 3, 96, 0, s()) == 0
     assert rel_err(o.cpu().numpy(), gu[:, 96:] * lo.swish(gu[:, :96].astype(np.float64))) < 1e-5
     # fp32 row gather with f32 ids, argmax with the reference's tie rule (last maximum wins)
     table = rng.standard_normal((50, 64)).astype(np.float32)
@@ -134,12 +134,79 @@ def test_rope_attention_swiglu_gather_argmax():
     assert int(idi.item()) == 4021 == lo.argmax_last(v) and idf.item() == 4021.0 and int(pos.item()) == pos0 + 3
 
 
+@pytest.mark.parametrize("hq,hkv,hd", [(8, 2, 128), (32, 8, 128), (4, 4, 64), (16, 2, 64), (4, 2, 128)])
+@pytest.mark.parametrize("pos0", [0, 1, 63, 64, 200, 1500])
+def test_decode_attention_equals_rope_append_attention(hq, hkv, hd, pos0):
+    """The one-launch decode attention against an f64 restatement of rotary + append + softmax(QK)V, at positions
+    that leave key ranges empty, ragged and many tiles long; three consecutive tokens share one workspace."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(hq * 1000 + pos0)
+    max_seq = 1600
+    kc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    vc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    kd, vd = torch.from_numpy(kc.copy()).to(DEV), torch.from_numpy(vc.copy()).to(DEV)
+    nws = lib.lhip_attention_decode_workspace_nbytes(hq, hkv, hd)
+    assert nws > 0
+    ws = torch.full((nws,), 0xFF, dtype=torch.uint8, device=DEV)  # contents on entry do not matter
+    out = torch.empty(hq * hd, device=DEV)
+    g = hq // hkv
+    for step in range(3):
+        p = pos0 + step
+        qkv = (2.0 * rng.standard_normal((hq + 2 * hkv, hd))).astype(np.float32)
+        pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+        qd = torch.from_numpy(qkv.copy()).to(DEV)
+        assert lib.lhip_attention_decode_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(),
+                                             pos.data_ptr(), hq, hkv, hd, max_seq, 500000.0, ws.data_ptr(), s()) == 0
+        assert np.array_equal(qd.cpu().numpy(), qkv)  # the input row is left alone
+        q_r = lo.rope(qkv[None, :hq].astype(np.float64), p, 500000.0)[0]
+        k_r = lo.rope(qkv[None, hq:hq + hkv].astype(np.float64), p, 500000.0)[0]
+        kc[:, p], vc[:, p] = k_r, qkv[hq + hkv:]
+        want = np.empty((hq, hd))
+        for h in range(hq):
+            sc = kc[h // g, :p + 1].astype(np.float64) @ q_r[h] / np.sqrt(hd)
+            w = np.exp(sc - sc.max())
+            want[h] = (w / w.sum()) @ vc[h // g, :p + 1].astype(np.float64)
+        # f32 rotary angles and softmax: judged against the scale of the output vector (elements that cancel to
+        # ~0 carry the same absolute rounding error as the rest)
+        err = np.max(np.abs(out.cpu().numpy() - want.reshape(-1))) / np.sqrt(np.mean(want * want))
+        # plus the f32 rotary angle: half an ulp of p turns q and k by p * 2^-24 rad, which moves a score by that
+        # times |q||k|/sqrt(hd) (~25 here)
+        assert err < 1e-4 + 25 * p * 2.0 ** -24, (step, p, err)
+        kgot, vgot = kd.cpu().numpy(), vd.cpu().numpy()
+        # the f32 angle p * inv_freq is off by up to half an ulp of p, which turns the pair by that much
+        k_tol = 2e-5 + p * 2.0 ** -23 * float(np.max(np.abs(qkv)))
+        assert np.max(np.abs(kgot[:, p] - k_r)) < k_tol and np.array_equal(vgot[:, p], qkv[hq + hkv:])
+        kc[:, p] = kgot[:, p]  # continue from the device's f32 rounding of the new key
+        assert np.array_equal(kgot, kc) and np.array_equal(vgot, vc)  # nothing else in the caches moved
+
+
+def test_decode_attention_argument_errors():
+    lib = capi.load_library()
+    a = torch.zeros(4096, device=DEV)
+    pos = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+
+    def call(hq=8, hkv=2, hd=128, qkv=a.data_ptr(), w=ws.data_ptr(), max_seq=4):
+        return lib.lhip_attention_decode_f32(qkv, a.data_ptr(), a.data_ptr(), a.data_ptr(), pos.data_ptr(), hq, hkv, hd,
+                                             max_seq, 1e4, w, s())
+
+    assert call() == capi.LHIP_OK
+    assert call(hq=6, hkv=2) == capi.LHIP_ERR_UNSUPPORTED and lib.lhip_attention_decode_workspace_nbytes(6, 2, 128) == 0
+    assert call(hd=256) == capi.LHIP_ERR_UNSUPPORTED
+    assert call(hq=7, hkv=2) == capi.LHIP_ERR_INVALID_SHAPE
+    assert call(max_seq=0) == capi.LHIP_ERR_INVALID_SHAPE
+    assert call(qkv=None) == capi.LHIP_ERR_NULL_PTR and call(w=None) == capi.LHIP_ERR_NULL_PTR
+    assert call(w=ws.data_ptr() + 16) == capi.LHIP_ERR_MISALIGNED
+    torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ end to end
 
 @pytest.mark.parametrize("cfg", [LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512),
                                  LlamaConfig(vocab=1000, dim=1024, layers=3, q_heads=8, kv_heads=2, ffn=2048)])
 def test_prefill_and_decode_logits_vs_oracle(oracle, cfg):
     eng, wf = build_model(oracle, cfg, seed=cfg.dim)
+    assert eng.fused_decode == (cfg.dim == 1024)  # the second configuration decodes through the fused matvecs
     rng = np.random.default_rng(3)
     prompt = [int(t) for t in rng.integers(0, cfg.vocab, 12)]
     kc, vc = empty_cache(cfg), empty_cache(cfg)
@@ -161,8 +228,9 @@ def test_prefill_and_decode_logits_vs_oracle(oracle, cfg):
         eng.tok_i.fill_(tok)
 
 
-def test_graph_replay_equals_eager_decode(oracle):
-    cfg = LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)
+@pytest.mark.parametrize("cfg", [LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512),
+                                 LlamaConfig(vocab=700, dim=1024, layers=2, q_heads=8, kv_heads=4, ffn=1024)])
+def test_graph_replay_equals_eager_decode(oracle, cfg):
     eng, _ = build_model(oracle, cfg, seed=7)
     prompt = [1, 2, 3, 4, 5]
     eng.prefill(prompt)
