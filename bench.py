@@ -7,6 +7,10 @@ token's worth of Q8_0 projections of Llama-3-8B at batch 1 — 32 layers x
 distinct weights (so every launch streams from HBM, not from cache), f32
 activations ~N(0,1), random weights: quants U{-127..127}, block scales
 |N(0,0.02)|/127 in f16.  Inputs are resident in HBM before timing starts.
+The sibling projections that read the same activations (q|k|v, gate|up) go
+out as one grouped launch each, from their separate weight buffers into their
+separate outputs, so a step is 129 launches; the 225-launch form is timed
+beside it.
 
 Prints ONE JSON line: whole-step GB/s of algorithmic bytes
 (N*K*34/32 + 4K + 4N per matvec), per-shape GB/s, the roofline fraction of the
@@ -29,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # Average HBM bytes per launch of the dominant kernel over one step, from the
 # committed rocprofv3 counter runs (FETCH_SIZE scaled by the copy-kernel factor
 # 2.0, plus WRITE_SIZE); None until measured.
-TRAFFIC_PER_LAUNCH = 28470579
+TRAFFIC_PER_LAUNCH = 138310222
 
 
 def parse():
@@ -374,13 +378,42 @@ def main():
         if st:
             capi.check(st, "lhip_q8_0_matmul_f32")
 
+    import ctypes as C
+
+    def group(names, wbufs):
+        """Argument block of one grouped launch: weights `names` (same K), each into its own output."""
+        cnt = len(names)
+        k = shapes[names[0]][1]
+        return ((C.c_void_p * cnt)(*[b.data_ptr() for b in wbufs]),
+                (C.c_void_p * cnt)(*[y[nm].data_ptr() for nm in names]),
+                (C.c_int64 * cnt)(*[shapes[nm][0] for nm in names]), cnt, x[k].data_ptr(), k)
+
+    def run_group(g):
+        st = lib.lhip_q8_0_matvec_fused_f32(g[0], g[1], g[2], g[3], g[4], g[5], None, 0.0, None, 0, stream)
+        if st:
+            capi.check(st, "lhip_q8_0_matvec_fused_f32")
+
+    plan = []  # per layer: (q|k|v), o, (gate|up), down
+    for l in range(layers):
+        plan.append((group(["q", "k", "v"], [weights["q"][l], weights["k"][l], weights["v"][l]]),
+                     group(["o"], [weights["o"][l]]),
+                     group(["gate", "up"], [weights["gate"][l], weights["up"][l]]),
+                     group(["down"], [weights["down"][l]])))
+    head = group(["lm_head"], [weights["lm_head"][0]])
+
     def step():
+        for groups in plan:
+            for g in groups:
+                run_group(g)
+        run_group(head)
+
+    def step_ungrouped():
         for l in range(layers):
             for nm in layer_names:
                 gemv(nm, weights[nm][l])
         gemv("lm_head", weights["lm_head"][0])
 
-    launches = layers * len(layer_names) + 1
+    launches = layers * 4 + 1
     step_bytes = layers * sum(synth.q8_0_gemv_bytes(*shapes[nm]) for nm in layer_names) \
         + synth.q8_0_gemv_bytes(*shapes["lm_head"])
 
@@ -398,6 +431,16 @@ def main():
     gpu_ms = ev0.elapsed_time(ev1)
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes / (wall / args.steps) / 1e9
+
+    # The same bytes as 225 separate matvec launches (one per weight).
+    step_ungrouped()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_ungrouped()
+    torch.cuda.synchronize()
+    ungrouped = {"launches_per_step": layers * len(layer_names) + 1,
+                 "gbs": round(step_bytes / ((time.perf_counter() - t0) / args.steps) / 1e9, 1)}
 
     # Per-shape rates: back-to-back launches rotating over that shape's distinct
     # weight buffers (lm_head alone is 558 MB, larger than the 256 MB last-level
@@ -421,6 +464,23 @@ def main():
         per_shape[nm] = {"n": shapes[nm][0], "k": shapes[nm][1], "us": round(us, 2),
                          "gbs": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
+    for label, idx, names in (("q|k|v grouped", 0, ["q", "k", "v"]), ("gate|up grouped", 2, ["gate", "up"])):
+        for groups in plan[:2]:
+            run_group(groups[idx])
+        torch.cuda.synchronize()
+        reps = max(1, 128 // layers)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for groups in plan:
+                run_group(groups[idx])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * layers)
+        nbytes = sum(synth.q8_0_gemv_bytes(*shapes[nm]) for nm in names)
+        per_shape[label] = {"n": [shapes[nm][0] for nm in names], "k": shapes[names[0]][1], "us": round(us, 2),
+                            "gbs": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
     # Calibration: plain copy and read-only kernels of known size (1 GiB), for
     # scaling hardware byte counters and as the streaming rate of this part.
     cal_n = 1 << 30
@@ -443,20 +503,19 @@ def main():
         calibration[label] = {"us": round(us, 1), "gbs": round(moved / us / 1e3, 1)}
     del cal_src, cal_dst
 
-    # Roofline of the dominant kernel.  All K = 4096 projections below lm_head's
-    # height run one kernel symbol, q8_gemv_f32_pipe_kernel<1, 2, 4> (1 row x 2
-    # slices per step, 4 waves per workgroup): q, k, v, o, gate, up = 192 of the
-    # step's 225 launches and about three quarters of its time.  Its launches
-    # are replayed alone, in step order over the same distinct weights, between
-    # two HIP events on the launch stream.
-    dom_names = ["q", "k", "v", "o", "gate", "up"]
-    dom_launches = layers * len(dom_names)
-    dom_bytes = layers * sum(synth.q8_0_gemv_bytes(*shapes[nm]) for nm in dom_names)
+    # Roofline of the dominant kernel.  The gate|up grouped launches and lm_head run one kernel symbol,
+    # q8_gemv_fused_kernel<2, 4, 4, false, 0> (2 rows x 4 slices of 1024 quants per step, 4 waves per workgroup,
+    # one workgroup per CU, no prologue or epilogue): 33 of the step's 129 launches, 4.55 of its 7.98 GB and
+    # about half of its time.  Its launches are replayed alone, in step order over the same distinct weights,
+    # between two HIP events on the launch stream.
+    dom_launches = layers + 1
+    dom_bytes = layers * sum(synth.q8_0_gemv_bytes(*shapes[nm]) for nm in ("gate", "up")) \
+        + synth.q8_0_gemv_bytes(*shapes["lm_head"])
 
     def dom_pass():
-        for l in range(layers):
-            for nm in dom_names:
-                gemv(nm, weights[nm][l])
+        for groups in plan:
+            run_group(groups[2])
+        run_group(head)
 
     dom_pass()
     torch.cuda.synchronize()
@@ -470,7 +529,7 @@ def main():
     achieved = (dom_bytes / dom_launches) / dom_us / 1e3  # GB/s
     roofline = {
         "bound": "hbm",
-        "kernel": "lhip::q8_gemv_f32_pipe_kernel<1, 2, 4>",
+        "kernel": "lhip::q8_gemv_fused_kernel<2, 4, 4, false, 0>",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -506,6 +565,7 @@ def main():
         },
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "per_shape": per_shape,
+        "one_launch_per_weight": ungrouped,
         "calibration": calibration,
         "roofline": roofline,
     }
