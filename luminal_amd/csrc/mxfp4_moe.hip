@@ -137,10 +137,14 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int *__restrict__ 
         for (int e = 0; e < E; ++e) {
             off[e] = o;
             p.offsets[e] = o;
-            for (int m0 = 0; m0 < cnt[e]; m0 += BM) {
+            // ceil(cnt / BM) tiles of equal height (a multiple of 16 rows): 140 rows with BM = 128 become
+            // 80 + 60 rather than 128 + 12, and the GEMM skips the row fragments a tile does not have.
+            const int tiles_e = (cnt[e] + BM - 1) / BM;
+            const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
+            for (int m0 = 0; m0 < cnt[e]; m0 += per) {
                 p.tile_expert[nt] = e;
                 p.tile_row0[nt] = o + m0;
-                p.tile_rows[nt] = min(BM, cnt[e] - m0);
+                p.tile_rows[nt] = min(per, cnt[e] - m0);
                 ++nt;
             }
             o += cnt[e];
@@ -244,11 +248,18 @@ struct BSet {
     bool valid;  // wave-uniform: false for a dead chunk past the padded K
 };
 
-template <int MT, int NT, bool GATED>
-__global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
+// WR = 1: 4 waves, each all MT row fragments x its NT column fragments.  WR = 2: 8 waves, the upper four
+// take the second half of the row fragments, so every SIMD holds two waves with half the accumulators each
+// and one wave's waits (LDS, barrier, weight stream) are covered by the other's matrix work.
+// D = weight prefetch distance in chunks (even).
+template <int MT, int NT, bool GATED, int WR, int D>
+__global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
     static_assert(!GATED || NT % 2 == 0, "gated tiles pair each gate fragment with its up fragment");
+    static_assert(MT % WR == 0 && D % 2 == 0, "tile shape");
     constexpr int BM = 16 * MT;
-    constexpr int D = 4;  // weight prefetch distance in chunks
+    constexpr int MTW = MT / WR;      // row fragments per wave
+    constexpr int THREADS = 256 * WR;
+    constexpr int STG = MT / WR;      // 16-byte pieces of the activation tile staged per thread and chunk
     constexpr int A_PLANE = BM * kARow;
     constexpr int A_BUF = 2 * A_PLANE + BM * 4;  // hi, lo, scales
 
@@ -262,11 +273,15 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave_id & 3;    // column group
+    const int wrow = wave_id >> 2;   // row half (WR = 2)
     const int r = lane & 15, grp = lane >> 4;
     const int Kp = g.Kp;
     const int chunks = Kp / kChunk;
     const int steps = (chunks + D - 1) / D * D;  // padded with dead chunks that add zero
+    const int frags = (rows + 15) >> 4;          // row fragments of this tile that hold rows
+    const int frag0 = wrow * MTW;                // first row fragment of this wave
 
     // ---- weight fragments: straight from global memory into MFMA registers.
     // The planar weights are tiled so that the 64 pieces a wave needs for one
@@ -297,17 +312,24 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         const int cc = min(c, chunks - 1);
 #pragma unroll
         for (int f = 0; f < NT; ++f) {
-            bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
-            bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+            // Short tiles (few routed rows per expert) read every weight once: keep them out of the caches.
+            // Tall tiles come several per expert, and the later ones find the weights in L2 / the last-level cache.
+            if (MT <= 2) {
+                bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
+                bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+            } else {
+                bs[set].q[f] = *reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024);
+                bs[set].s[f] = s_tile[f][cc * 64];
+            }
         }
     };
 
     // ---- activation tile: global -> registers -> LDS (double-buffered), shared by the 4 waves
-    const uint8_t *a_src[MT];
-    int a_dst[MT];
+    const uint8_t *a_src[STG];
+    int a_dst[STG];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int q = tid + i * 256;  // chunk of 16 bytes: plane, row, 16-byte column
+    for (int i = 0; i < STG; ++i) {
+        const int q = tid + i * THREADS;  // chunk of 16 bytes: plane, row, 16-byte column
         const int plane = q / (BM * 8), rem = q - plane * (BM * 8);
         const int row = rem >> 3, c16 = rem & 7;
         const int slot = row0 + min(row, rows - 1);  // rows past the tile re-read its last row (not stored)
@@ -321,27 +343,27 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
         as_src = g.a_sc + static_cast<size_t>(arow) * (Kp / 32);
     }
-    mu32x4 a_reg[MT];
+    mu32x4 a_reg[STG];
     uint32_t as_reg = 0;
     auto load_a = [&](int c) {
         const int cc = min(c, chunks - 1);  // dead chunks re-read the last one; their weights are zero
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a_reg[i] = *reinterpret_cast<const mu32x4 *>(a_src[i] + cc * kChunk);
+        for (int i = 0; i < STG; ++i) a_reg[i] = *reinterpret_cast<const mu32x4 *>(a_src[i] + cc * kChunk);
         if (tid < BM) as_reg = *reinterpret_cast<const uint32_t *>(as_src + cc * 4);
     };
     auto store_a = [&](int buf) {
         unsigned char *base = lds + buf * A_BUF;
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
+        for (int i = 0; i < STG; ++i) {
             asm volatile("" : "+v"(a_reg[i]));
             *reinterpret_cast<mu32x4 *>(base + a_dst[i]) = a_reg[i];
         }
         if (tid < BM) *reinterpret_cast<uint32_t *>(base + 2 * A_PLANE + tid * 4) = as_reg;
     };
 
-    v4f acc[MT][NT];
+    v4f acc[MTW][NT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < MTW; ++i)
 #pragma unroll
         for (int f = 0; f < NT; ++f) acc[i][f] = v4f{0.f, 0.f, 0.f, 0.f};
 
@@ -373,11 +395,12 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         }
         // The LDS reads of fragment i+1 are issued before the MFMAs of fragment i and
         // fenced there, so two fragments are live at a time instead of all MT.
-        AFrag cur = load_frag(base, 0);
+        AFrag cur = load_frag(base, frag0);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
+        for (int i = 0; i < MTW; ++i) {
+            if (frag0 + i >= frags) break;  // wave-uniform: this tile has no rows there
             AFrag nxt = cur;
-            if (i + 1 < MT) nxt = load_frag(base, i + 1);
+            if (i + 1 < MTW && frag0 + i + 1 < frags) nxt = load_frag(base, frag0 + i + 1);
             __builtin_amdgcn_sched_barrier(0);
             const int sa = static_cast<int>((cur.sw >> (8 * grp)) & 0xff);
             const v8i ah = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
@@ -421,10 +444,10 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_kernel(MoeGemmArgs g) {
 
     // ---- epilogue: acc[i][f][v] is row i*16 + 4*grp + v, column fragment f, column r
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < MTW; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int m = i * 16 + 4 * grp + v;
+            const int m = (frag0 + i) * 16 + 4 * grp + v;
             if (m >= rows) continue;
             const size_t orow = static_cast<size_t>(row0 + m) * g.N;
             if (GATED) {
@@ -657,15 +680,15 @@ static MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, int64_t E
     return w;
 }
 
-template <int MT, int NT, bool GATED>
+template <int MT, int NT, bool GATED, int WR = 1, int D = 4>
 static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
     constexpr int BM = 16 * MT;
     const size_t lds_bytes = 2 * (2 * static_cast<size_t>(BM) * kARow + BM * 4);
-    auto kern = mx_moe_gemm_kernel<MT, NT, GATED>;
+    auto kern = mx_moe_gemm_kernel<MT, NT, GATED, WR, D>;
     if (lds_bytes > 64 * 1024)
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256),
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256 * WR),
                        lds_bytes, s, a);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
@@ -776,7 +799,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
             break;
         case 2: st = launch_moe_gemm<2, 2, true>(a1, cb1, max_tiles, s); break;
         case 4: st = launch_moe_gemm<4, 4, true>(a1, cb1w, max_tiles, s); break;
-        default: st = launch_moe_gemm<8, 4, true>(a1, cb1w, max_tiles, s); break;
+        default: st = launch_moe_gemm<8, 4, true, 2, 4>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
     {
@@ -801,7 +824,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         switch (mt) {
             case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
             case 4: st = launch_moe_gemm<4, 4, false>(a2, cb2w, max_tiles, s); break;
-            default: st = launch_moe_gemm<8, 4, false>(a2, cb2w, max_tiles, s); break;
+            default: st = launch_moe_gemm<8, 4, false, 2, 4>(a2, cb2w, max_tiles, s); break;
         }
     }
     if (st) return st;
