@@ -249,7 +249,7 @@ struct BSet {
 };
 
 // WR = 1: 4 waves, each all MT row fragments x its NT column fragments.  WR = 2: 8 waves, the upper four
-// take the second half of the row fragments, so every SIMD holds two waves with half the accumulators each
+// take the odd row fragments, so every SIMD holds two waves with half the accumulators each
 // and one wave's waits (LDS, barrier, weight stream) are covered by the other's matrix work.
 // D = weight prefetch distance in chunks (even).
 template <int MT, int NT, bool GATED, int WR, int D>
@@ -281,7 +281,6 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
     const int chunks = Kp / kChunk;
     const int steps = (chunks + D - 1) / D * D;  // padded with dead chunks that add zero
     const int frags = (rows + 15) >> 4;          // row fragments of this tile that hold rows
-    const int frag0 = wrow * MTW;                // first row fragment of this wave
 
     // ---- weight fragments: straight from global memory into MFMA registers.
     // The planar weights are tiled so that the 64 pieces a wave needs for one
@@ -395,12 +394,13 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         }
         // The LDS reads of fragment i+1 are issued before the MFMAs of fragment i and
         // fenced there, so two fragments are live at a time instead of all MT.
-        AFrag cur = load_frag(base, frag0);
+        // Row fragments are dealt round-robin to the WR row groups, so a short tile still occupies all waves.
+        AFrag cur = load_frag(base, wrow);
 #pragma unroll
         for (int i = 0; i < MTW; ++i) {
-            if (frag0 + i >= frags) break;  // wave-uniform: this tile has no rows there
+            if (i * WR + wrow >= frags) break;  // wave-uniform: this tile has no rows there
             AFrag nxt = cur;
-            if (i + 1 < MTW && frag0 + i + 1 < frags) nxt = load_frag(base, frag0 + i + 1);
+            if (i + 1 < MTW && (i + 1) * WR + wrow < frags) nxt = load_frag(base, (i + 1) * WR + wrow);
             __builtin_amdgcn_sched_barrier(0);
             const int sa = static_cast<int>((cur.sw >> (8 * grp)) & 0xff);
             const v8i ah = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
     for (int i = 0; i < MTW; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int m = (frag0 + i) * 16 + 4 * grp + v;
+            const int m = (i * WR + wrow) * 16 + 4 * grp + v;
             if (m >= rows) continue;
             const size_t orow = static_cast<size_t>(row0 + m) * g.N;
             if (GATED) {
