@@ -289,15 +289,16 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     };
     const int n4 = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) ? n >> 2 : 0;  // vector part
     const float4 *x4 = reinterpret_cast<const float4 *>(x);
-    for (int j0 = threadIdx.x; j0 < n4; j0 += 4096) {  // four independent loads per trip
-        float4 c[4];
+    constexpr int U = 16;  // independent loads per trip: a 128k-entry row is two memory round trips
+    for (int j0 = threadIdx.x; j0 < n4; j0 += U * 1024) {
+        float4 c[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int j = j0 + u * 1024;
             c[u] = j < n4 ? x4[j] : make_float4(-3.4e38f, -3.4e38f, -3.4e38f, -3.4e38f);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int j = (j0 + u * 1024) * 4;
             if (j0 + u * 1024 < n4) {
                 take(c[u].x, j); take(c[u].y, j + 1); take(c[u].z, j + 2); take(c[u].w, j + 3);
