@@ -13,6 +13,10 @@
 
 namespace lhip {
 
+// attention_prefill.hip: matrix-core kernel for prompt-sized calls; false if the shape is not built.
+bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, float *out, const int *pos, int tokens,
+                              int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s);
+
 __device__ __forceinline__ float block_sum(float v, float *red) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -386,6 +390,13 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
     if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || head_dim % 64 != 0 ||
         max_seq <= 0 || q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 12000)
         return LHIP_ERR_INVALID_SHAPE;  // the score row of one query lives in LDS
+    if (tokens >= 8 && aligned(qkv_dev, 16) && aligned(k_cache_dev, 16) && aligned(v_cache_dev, 16) && aligned(out_dev, 16) &&
+        attention_prefill_launch(qkv_dev, k_cache_dev, v_cache_dev, out_dev, pos_dev, static_cast<int>(tokens),
+                                 static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
+                                 static_cast<int>(max_seq), as_stream(stream))) {
+        LHIP_CHECK_LAUNCH();
+        return LHIP_OK;
+    }
     hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)),
                        dim3(kAttnThreads),
                        static_cast<size_t>(max_seq) * sizeof(float), as_stream(stream), qkv_dev, k_cache_dev,

@@ -180,6 +180,34 @@ def test_decode_attention_equals_rope_append_attention(hq, hkv, hd, pos0):
         assert np.array_equal(kgot, kc) and np.array_equal(vgot, vc)  # nothing else in the caches moved
 
 
+@pytest.mark.parametrize("hq,hkv,hd", [(8, 2, 128), (32, 8, 128), (4, 4, 64), (16, 2, 64), (4, 2, 128), (8, 8, 128)])
+@pytest.mark.parametrize("S,pos0", [(8, 0), (33, 0), (70, 5), (64, 64), (129, 31)])
+def test_prompt_attention_on_matrix_cores(hq, hkv, hd, S, pos0):
+    """Calls of 8 or more tokens take the matrix-core kernel: against the f64 softmax(QK)V over the cache, for
+    query blocks and key tiles that are ragged, start mid-cache and span several tiles."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(hq * 100 + S + pos0)
+    max_seq = 200
+    kc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    vc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    qkv = rng.standard_normal((S, hq + 2 * hkv, hd)).astype(np.float32)
+    kd, vd, qd = (torch.from_numpy(a).to(DEV) for a in (kc, vc, qkv))
+    pos = torch.tensor([pos0], dtype=torch.int32, device=DEV)
+    out = torch.full((S, hq * hd), float("nan"), device=DEV)
+    assert lib.lhip_attention_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), pos.data_ptr(), S, hq,
+                                  hkv, hd, max_seq, s()) == 0
+    g = hq // hkv
+    want = np.empty((S, hq, hd))
+    for t in range(S):
+        n = pos0 + t + 1
+        for h in range(hq):
+            sc = kc[h // g, :n].astype(np.float64) @ qkv[t, h].astype(np.float64) / np.sqrt(hd)
+            w = np.exp(sc - sc.max())
+            want[t, h] = (w / w.sum()) @ vc[h // g, :n].astype(np.float64)
+    err = np.max(np.abs(out.cpu().numpy() - want.reshape(S, -1))) / np.sqrt(np.mean(want * want))
+    assert err < 1e-5, err
+
+
 def test_decode_attention_argument_errors():
     lib = capi.load_library()
     a = torch.zeros(4096, device=DEV)
