@@ -1,8 +1,9 @@
 """Build recipe of libluminal_hip.so (hipcc, gfx950 only).
 
 ``python -m luminal_amd.build`` compiles every HIP source under ``csrc/`` into
-one shared library beside this file, plus a code object (``.hsaco``) holding
-the same kernels for callers that load them with hipModuleLoad.
+one shared library beside this file.  The kernels are C++ templates launched by
+the library's own ``extern "C"`` entry points; callers bind those entry points,
+not the kernels.
 """
 from __future__ import annotations
 
@@ -15,7 +16,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libluminal_hip.so")
-HSACO = os.path.join(HERE, "luminal_hip_gfx950.hsaco")
 
 ARCH = "gfx950"
 # Packed-FP32 instructions are switched off for all device code.
