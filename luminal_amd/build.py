@@ -55,5 +55,24 @@ def build(verbose: bool = True) -> str:
     return LIB
 
 
+HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "host_mirror_test.cpp")
+HOST_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "_build", "host_mirror_test")
+
+
+def build_host_test(verbose: bool = True) -> str:
+    """Compile the test program of the C++ host mirror (host/luminal_hip.hpp) with the host compiler; it links
+    against libluminal_hip.so only."""
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("no host C++ compiler found (g++)")
+    os.makedirs(os.path.dirname(HOST_TEST_BIN), exist_ok=True)
+    if verbose:
+        print(f"[luminal_amd.build] {cxx} -> {HOST_TEST_BIN}", file=sys.stderr)
+    _run([cxx, "-std=c++17", "-O1", "-Wall", "-o", HOST_TEST_BIN, HOST_TEST_SRC, "-L" + HERE, "-lluminal_hip",
+          "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../../luminal_amd"])
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     build()
+    build_host_test()
