@@ -47,7 +47,7 @@ __device__ __forceinline__ uint2 dequant4_bf16(uint32_t q4, float d) {
 }
 
 // D = register prefetch depth in K tiles (D > 1 needs K % (64*D) == 0 and D even).
-template <int BM, int BN, int WM, int WN, int D>
+template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
                                                                    const __half *__restrict__ ds,
                                                                    const __bf16 *__restrict__ x,
@@ -120,13 +120,16 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
             d_reg[set][i] = d_src[i][k0 >> 6];
         }
     };
-    auto store_tile = [&](int set, int buf) {
+    // part p of P: the p-th share of the thread's chunks (P = 1: everything).
+    auto store_tile = [&](int set, int buf, int p = 0, int P = 1) {
         unsigned char *A = lds + buf * (A_BYTES + B_BYTES);
         unsigned char *B = A + A_BYTES;
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
+        for (int i = 0; i < A_CHUNKS; ++i)
+            if (i * P / A_CHUNKS == p) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
+            if (i * P / B_CHUNKS != p) continue;
             // Opaque to the optimiser: keeps the unpacking of this set here, at its use,
             // instead of next to its loads (where it would wait for data just requested).
             asm volatile("" : "+v"(b_reg[set][i]), "+v"(d_reg[set][i]));
@@ -167,6 +170,32 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         }
     };
 
+    // Pipelined form of compute_tile + store_tile: the operand fragments of step kk+1 are requested before the
+    // MFMAs of step kk, and the dequantise-and-store of the next tile is dealt out over the four steps so its VALU
+    // and LDS-write work sits between the MFMAs instead of after them (measured: +10 % on the large shapes).
+    auto compute_and_store = [&](int buf, int set, int next_buf) {
+        const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
+        const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
+        bf16x8 af[2][FM], bfr[2][FN];
+        auto load_frags = [&](int kk, int to) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[to][i] = *reinterpret_cast<const bf16x8 *>(A + i * 32 * kRowBytes + kk * 32);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) bfr[to][j] = *reinterpret_cast<const bf16x8 *>(B + j * 32 * kRowBytes + kk * 32);
+        };
+        load_frags(0, 0);
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+            if (kk + 1 < kBK / 16) load_frags(kk + 1, (kk + 1) & 1);
+            store_tile(set, next_buf, kk, kBK / 16);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
+        }
+    };
+
 #pragma unroll
     for (int j = 0; j < D; ++j) load_tile(j, j);
     store_tile(0, 0);
@@ -190,8 +219,12 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
                 // LDS stores below, the wait for the tile loaded D-1 steps ago also
                 // waits for them and the prefetch distance collapses.
                 __builtin_amdgcn_sched_barrier(0);
-                compute_tile(j & 1);
-                store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
+                if constexpr (PIPE) {
+                    compute_and_store(j & 1, (j + 1) % D, (j + 1) & 1);
+                } else {
+                    compute_tile(j & 1);
+                    store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
+                }
                 __syncthreads();
             }
         }
@@ -211,13 +244,13 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         }
 }
 
-template <int BM, int BN, int WM, int WN, int D>
+template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
 static lhip_status launch_gemm(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
                                hipStream_t s) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
-    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D>;
+    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, PIPE>;
     if (lds_bytes > 64 * 1024) {
         // Opting in to more than 64 KiB of dynamic LDS is a per-function attribute.
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -250,7 +283,7 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
     // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
     const bool deep = (k % (kBK * 4)) == 0;
 #define LHIP_TILE(BM, BN, WM, WN)                                                                  \
-    return deep ? launch_gemm<BM, BN, WM, WN, 4>(qs, ds, x_dev, y_dev, mi, ni, ki, s)              \
+    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(qs, ds, x_dev, y_dev, mi, ni, ki, s)        \
                 : launch_gemm<BM, BN, WM, WN, 1>(qs, ds, x_dev, y_dev, mi, ni, ki, s)
     switch (tile) {
         case 0: LHIP_TILE(256, 128, 4, 2);
