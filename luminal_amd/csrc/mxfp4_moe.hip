@@ -132,26 +132,31 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int *__restrict__ 
         if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    // Thread e lays out expert e: its first slot and first tile are prefix sums over the experts before it
+    // (E <= 1024 broadcast reads from LDS), then it writes its own tiles.
+    // ceil(cnt / BM) tiles of equal height (a multiple of 16 rows): 140 rows with BM = 128 become 80 + 60 rather
+    // than 128 + 12, and the GEMM skips the row fragments a tile does not have.
+    for (int e = threadIdx.x; e < E; e += 1024) {
         int o = 0, nt = 0;
-        for (int e = 0; e < E; ++e) {
-            off[e] = o;
-            p.offsets[e] = o;
-            // ceil(cnt / BM) tiles of equal height (a multiple of 16 rows): 140 rows with BM = 128 become
-            // 80 + 60 rather than 128 + 12, and the GEMM skips the row fragments a tile does not have.
-            const int tiles_e = (cnt[e] + BM - 1) / BM;
-            const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
-            for (int m0 = 0; m0 < cnt[e]; m0 += per) {
-                p.tile_expert[nt] = e;
-                p.tile_row0[nt] = o + m0;
-                p.tile_rows[nt] = min(per, cnt[e] - m0);
-                ++nt;
-            }
-            o += cnt[e];
+        for (int q = 0; q < e; ++q) {
+            o += cnt[q];
+            nt += (cnt[q] + BM - 1) / BM;  // equals the number of tiles written for q below
         }
-        off[E] = o;
-        p.offsets[E] = o;
-        *p.n_tiles = nt;
+        off[e] = o;
+        p.offsets[e] = o;
+        const int tiles_e = (cnt[e] + BM - 1) / BM;
+        const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
+        for (int m0 = 0; m0 < cnt[e]; m0 += per) {
+            p.tile_expert[nt] = e;
+            p.tile_row0[nt] = o + m0;
+            p.tile_rows[nt] = min(per, cnt[e] - m0);
+            ++nt;
+        }
+        if (e == E - 1) {
+            off[E] = o + cnt[e];
+            p.offsets[E] = o + cnt[e];
+            *p.n_tiles = nt;
+        }
     }
     __syncthreads();
     // Order inside an expert's range is arbitrary (atomic): every row is computed
