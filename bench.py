@@ -43,8 +43,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode_projection_set",
                     choices=["decode_projection_set", "prefill_gemm", "moe"],
-                    help="decode_projection_set (default, the headline metric), prefill_gemm (BASELINE config 2), "
-                         "moe (BASELINE config 3)")
+                    help="decode_projection_set (default, the headline metric), prefill_gemm (the Q8_0 prefill GEMM set), "
+                         "moe (the MXFP4 expert layer)")
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end Llama-3-8B decode section")
@@ -136,7 +136,7 @@ def _event_us(torch, fn, reps):
 
 
 def bench_prefill_gemm(args):
-    """BASELINE config 2: the seven Llama-3-8B weight shapes in Q8_0 against bf16 activations,
+    """Prefill GEMM set: the seven Llama-3-8B weight shapes in Q8_0 against bf16 activations,
     M in {128, 512, 2048}, f32 accumulation, bf16 output.  A step is one pass over all shapes at
     all three M; weights rotate over distinct buffers."""
     import torch
@@ -209,7 +209,7 @@ def bench_prefill_gemm(args):
 
 
 def bench_moe(args):
-    """BASELINE config 3: gpt-oss-style MXFP4 expert layer, H = I = 2880, 32 experts, top-4,
+    """MoE workload: gpt-oss-style MXFP4 expert layer, H = I = 2880, 32 experts, top-4,
     T in {1, 64, 1024}; a step is one layer pass at each T (routing rotates so T = 1 streams
     different experts from HBM every pass)."""
     import torch
@@ -293,7 +293,7 @@ def bench_moe(args):
 
 
 def llama_decode(torch):
-    """BASELINE config 4: random-weight Llama-3-8B, all linears Q8_0, norms and embeddings f32;
+    """End-to-end workload: random-weight Llama-3-8B, all linears Q8_0, norms and embeddings f32;
     512-token prefill (bf16 GEMM path), then 256 greedy batch-1 decode steps (f32 matvec path,
     one captured HIP graph per step, token and position stay on the device)."""
     import numpy as np

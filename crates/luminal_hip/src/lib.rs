@@ -6,7 +6,7 @@
 //! cx.compile((GenericCompiler::default(), HipQuantizedCompiler::<f32>::new(q_weights)), (&mut logits, &mut cache));
 //! ```
 //! This crate cannot be compiled where the backend was developed (no Rust toolchain); it is the
-//! maintainer-side half of the boundary documented in INTEGRATION.md.
+//! maintainer-side half of the boundary declared in include/luminal_hip.h.
 pub mod ffi;
 mod quantized;
 

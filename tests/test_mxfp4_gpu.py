@@ -132,7 +132,7 @@ def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
 
 @pytest.mark.parametrize("t", [1, 64, 1024])
 def test_moe_benchmark_layer(oracle, t):
-    """BASELINE config 3: H = I = 2880, 32 experts, top-4; the oracle runs on a sample of tokens."""
+    """The benchmark expert layer: H = I = 2880, 32 experts, top-4; the oracle runs on a sample of tokens."""
     e, h, i, topk = synth.MOE_EXPERTS, synth.MOE_HIDDEN, synth.MOE_INTER, synth.MOE_TOPK
     layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=2024)
     xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t, scale=1.0)

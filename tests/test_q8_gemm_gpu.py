@@ -97,7 +97,7 @@ def test_reference_metal_matmul_case(oracle):
 
 @pytest.mark.parametrize("name,m", [("q", 128), ("k", 512), ("down", 128), ("gate", 2048)])
 def test_full_size_prefill_shapes(oracle, name, m):
-    """BASELINE config 2 shapes; the oracle runs on a sample of weight rows."""
+    """The Llama-3-8B prefill shapes (M in {128, 512, 2048}); the oracle runs on a sample of weight rows."""
     n, k = synth.LLAMA3_8B_PROJ[name]
     qs, d = synth.q8_0_random(n, k, seed=300 + m)
     xf, bits = bf16_activations(oracle, m, k, seed=301)

@@ -84,7 +84,7 @@ def run_matmul(w, x, cfg=None):
 
 
 def test_config0_single_matvec_4096(oracle):
-    """BASELINE config 0: W 4096x4096, x 1x4096 N(0,1), y = x W^T in f32."""
+    """The single-matvec benchmark case: W 4096x4096, x 1x4096 N(0,1), y = x W^T in f32."""
     qs, d = synth.q8_0_random(4096, 4096, seed=0x5EED)
     x = synth.activations(1, 4096, seed=0x5EED + 1)
     w = upload(qs, d)
@@ -196,7 +196,7 @@ def test_zero_scale_blocks_and_extreme_quants(oracle):
 
 @pytest.mark.parametrize("name", ["q", "k", "gate", "down", "lm_head"])
 def test_full_size_projection_vs_oracle(oracle, name):
-    """BASELINE config 1 shapes at full size against the f64 truth."""
+    """The Llama-3-8B decode projection shapes at full size against the f64 truth."""
     n, k = synth.LLAMA3_8B_PROJ[name]
     qs, d = synth.q8_0_random(n, k, seed=100 + sorted(synth.LLAMA3_8B_PROJ).index(name))
     x = synth.activations(1, k, seed=77)
