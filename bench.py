@@ -191,7 +191,7 @@ def bench_prefill_gemm(args):
             per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
                                   "frac_mfma_bf16": round(fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                   "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
-    # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4, true> on the M = 2048 gate/up shape
+    # dominant kernel: q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true> on the M = 2048 gate/up shape
     n, k, m = 14336, 4096, 2048
     us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5) / len(bufs["gate/up"])
     ach = 2.0 * m * n * k / us / 1e6
@@ -203,7 +203,7 @@ def bench_prefill_gemm(args):
         "dtype": "int8 weights dequantised to bf16 x bf16 activations, f32 accumulate, bf16 out", "data": "synthetic",
         "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list)},
         "per_shape": per,
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4, true> (gate/up, M=2048)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true> (gate/up, M=2048)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_us": round(us, 1)}}))
 

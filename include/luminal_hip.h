@@ -144,7 +144,8 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
- * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each). */
+ * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
+ * K % 128 == 0, else LHIP_ERR_UNSUPPORTED). */
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream);
 

@@ -290,6 +290,10 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
         case 1: LHIP_TILE(128, 128, 2, 2);
         case 2: LHIP_TILE(128, 64, 2, 2);
         case 3: LHIP_TILE(64, 64, 2, 2);
+        case 4:  // 256x256 by eight 64x128 waves: 0.75 KiB of LDS operand reads per MFMA instead of 1; both
+                 // LDS buffers together are 144 KiB, which leaves registers for a prefetch depth of two K tiles
+            if (k % (kBK * 2) != 0) return LHIP_ERR_UNSUPPORTED;
+            return launch_gemm<256, 256, 4, 2, 2, true>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
         default: return LHIP_ERR_UNSUPPORTED;
     }
 #undef LHIP_TILE
@@ -298,11 +302,12 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream) {
     // Largest tile that still gives at least three quarters of the 256 CUs a
-    // workgroup (measured: 224 workgroups of 256x128 beat 448 of 128x128); a
-    // 256-row tile is skipped when it would be half padding.
+    // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
+    // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
     auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     int tile = 3;
-    if (m > 128 && blocks(256, 128) >= 192) tile = 0;
+    if (m > 128 && k % (kBK * 2) == 0 && blocks(256, 256) >= 192) tile = 4;
+    else if (m > 128 && blocks(256, 128) >= 192) tile = 0;
     else if (blocks(128, 128) >= 192) tile = 1;
     else if (blocks(128, 64) >= 192) tile = 2;
     return lhip_q8_0_matmul_bf16_cfg(planar_dev, x_dev, y_dev, m, n, k, tile, stream);

@@ -52,12 +52,17 @@ def truth_for(oracle, qs, d, xf):
     return oracle.matmul_f64(xf, wf)
 
 
-@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (16, 512, 1024), (33, 67, 128), (130, 200, 256), (257, 129, 4096),
-                                   (128, 1024, 4096), (300, 96, 14336)])
+                                   (128, 1024, 4096), (300, 96, 14336), (513, 600, 2048)])
 def test_gemm_vs_oracle_all_tiles_ragged(oracle, tile, m, n, k):
     qs, d = synth.q8_0_random(n, k, seed=m + n + k)
     xf, bits = bf16_activations(oracle, m, k, seed=m * n)
+    if tile == 4 and k % 128 != 0:  # the 256x256 tile prefetches two K tiles at a time
+        with pytest.raises(capi.LhipError) as e:
+            run(upload(qs, d), bits, tile)
+        assert e.value.status == capi.LHIP_ERR_UNSUPPORTED
+        return
     y = run(upload(qs, d), bits, tile)
     assert y.shape == (m, n)
     elem, norm = bf16_err(y, truth_for(oracle, qs, d, xf))
@@ -76,7 +81,7 @@ def test_gemm_integer_exact():
     want = x.astype(np.float64) @ (qs.astype(np.float64) * np.repeat(d.astype(np.float64), 32, axis=1)).T
     want_bf16 = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).float().numpy()
     w = upload(qs, d)
-    for tile in (None, 0, 1, 2, 3):
+    for tile in (None, 0, 1, 2, 3, 4):
         assert np.array_equal(run(w, bits, tile), want_bf16), tile
 
 
