@@ -143,6 +143,10 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
  * otherwise). */
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream);
+/* Same GEMM with the f32 accumulators stored as they are (y (m, N) f32, 4-byte aligned): what a caller
+ * whose surrounding operators are f32 wants instead of a bf16 round trip. */
+lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_dev, float *y_dev, int64_t m, int64_t n,
+                                         int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
  * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
  * K % 128 == 0, else LHIP_ERR_UNSUPPORTED). */
@@ -234,6 +238,18 @@ lhip_status lhip_attention_decode_f32(const float *qkv_dev, float *k_cache_dev, 
  * interleaved != 0, gate = gate_up[r][2j], up = gate_up[r][2j + 1] (the row order the fused matvec epilogue uses). */
 lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,
                             void *stream);
+/* The three operators that feed a bf16 GEMM, writing bf16 (round to nearest even) instead of f32, so a prompt pass
+ * needs no cast kernels: same arguments and arithmetic as their f32 forms, y / out are bf16 buffers (8-byte
+ * aligned).  lhip_attention_f32_bf16out runs the matrix-core kernel only (head_dim 64 or 128, q_heads / kv_heads in
+ * {1, 2, 4, 8}): LHIP_ERR_UNSUPPORTED otherwise. */
+lhip_status lhip_rms_norm_f32_bf16out(const float *x_dev, const float *residual_dev, float *x_out_dev,
+                                      const float *w_dev, void *y_bf16_dev, int64_t rows, int64_t dim, float eps,
+                                      void *stream);
+lhip_status lhip_swiglu_f32_bf16out(const float *gate_up_dev, void *out_bf16_dev, int64_t rows, int64_t f,
+                                    int interleaved, void *stream);
+lhip_status lhip_attention_f32_bf16out(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
+                                       void *out_bf16_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
+                                       int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
 /* Element-wise casts between f32 and bf16 (round to nearest even), for feeding f32
  * activations to the bf16 prefill GEMM. */
 lhip_status lhip_cast_f32_to_bf16(const float *x_dev, void *y_dev, int64_t n, void *stream);

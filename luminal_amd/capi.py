@@ -39,6 +39,7 @@ SIGNATURES = {
     "lhip_q8_0_matvec_fused_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _int, _int,
                                                    _int, _int, _vp]),
     "lhip_q8_0_matmul_bf16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_bf16_f32out": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_bf16_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_mxfp4_raw_nbytes": (_sz, [_i64, _i64]),
@@ -52,11 +53,14 @@ SIGNATURES = {
     "lhip_mxfp4_moe_bf16": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp, _vp]),
     "lhip_gather_rows_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_rms_norm_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
+    "lhip_rms_norm_f32_bf16out": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
     "lhip_rope_kv_append_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp]),
     "lhip_attention_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "lhip_attention_f32_bf16out": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lhip_attention_decode_workspace_nbytes": (C.c_size_t, [_i64, _i64, _i64]),
     "lhip_attention_decode_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp]),
     "lhip_swiglu_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "lhip_swiglu_f32_bf16out": (C.c_int32, [_vp, _vp, _i64, _i64, _int, _vp]),
     "lhip_cast_f32_to_bf16": (C.c_int32, [_vp, _vp, _i64, _vp]),
     "lhip_cast_bf16_to_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),
     "lhip_add_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),

@@ -30,11 +30,11 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kPfTileK = 32;  // keys per tile
 constexpr int kPfTileQ = 32;  // queries per workgroup
 
-template <int G, int HD>
+template <int G, int HD, typename OutT>
 __global__ __launch_bounds__(64 * G) void attention_prefill_kernel(const float *__restrict__ qkv,
                                                                   const float *__restrict__ k_cache,
                                                                   const float *__restrict__ v_cache,
-                                                                  float *__restrict__ out,
+                                                                  OutT *__restrict__ out,
                                                                   const int *__restrict__ pos_dev, int tokens, int hkv,
                                                                   int max_seq) {
     constexpr int THREADS = 64 * G;
@@ -197,30 +197,36 @@ __global__ __launch_bounds__(64 * G) void attention_prefill_kernel(const float *
     // ---- out[q][head*HD + VW*row + j] = O^T[j][row][q] / l
     if (my_q < tokens) {
         const float inv = 1.0f / l_run;
-        float *orow = out + (static_cast<size_t>(my_q) * hq + head) * HD;
+        OutT *orow = out + (static_cast<size_t>(my_q) * hq + head) * HD;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = 8 * (v >> 2) + 4 * h + (v & 3);
             if constexpr (VW == 4) {
-                *reinterpret_cast<float4 *>(orow + 4 * row) =
-                    make_float4(o_acc[0][v] * inv, o_acc[1][v] * inv, o_acc[2][v] * inv, o_acc[3][v] * inv);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) orow[4 * row + j] = static_cast<OutT>(o_acc[j][v] * inv);
             } else {
-                *reinterpret_cast<float2 *>(orow + 2 * row) = make_float2(o_acc[0][v] * inv, o_acc[1][v] * inv);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) orow[2 * row + j] = static_cast<OutT>(o_acc[j][v] * inv);
             }
         }
     }
 }
 
 // Launcher used by lhip_attention_f32 for prompt-sized calls; false if this shape is not built.
-bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, float *out, const int *pos, int tokens,
-                              int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s) {
+bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, void *out, bool out_bf16, const int *pos,
+                              int tokens, int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s) {
+    if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return false;
     const int g = q_heads / kv_heads;
     const dim3 grid(static_cast<unsigned>(kv_heads), static_cast<unsigned>((tokens + kPfTileQ - 1) / kPfTileQ));
     if (kv_heads > 65535 || grid.y > 65535) return false;
 #define LHIP_CASE(G, HD)                                                                                            \
     if (g == G && head_dim == HD) {                                                                                 \
-        hipLaunchKernelGGL((attention_prefill_kernel<G, HD>), grid, dim3(64 * G), 0, s, qkv, kc, vc, out, pos, tokens, \
-                           kv_heads, max_seq);                                                                      \
+        if (out_bf16)                                                                                               \
+            hipLaunchKernelGGL((attention_prefill_kernel<G, HD, __bf16>), grid, dim3(64 * G), 0, s, qkv, kc, vc,    \
+                               static_cast<__bf16 *>(out), pos, tokens, kv_heads, max_seq);                         \
+        else                                                                                                        \
+            hipLaunchKernelGGL((attention_prefill_kernel<G, HD, float>), grid, dim3(64 * G), 0, s, qkv, kc, vc,     \
+                               static_cast<float *>(out), pos, tokens, kv_heads, max_seq);                          \
         return true;                                                                                                \
     }
     LHIP_CASE(1, 64) LHIP_CASE(2, 64) LHIP_CASE(4, 64) LHIP_CASE(8, 64)

@@ -14,8 +14,8 @@
 namespace lhip {
 
 // attention_prefill.hip: matrix-core kernel for prompt-sized calls; false if the shape is not built.
-bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, float *out, const int *pos, int tokens,
-                              int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s);
+bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, void *out, bool out_bf16, const int *pos,
+                              int tokens, int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s);
 
 __device__ __forceinline__ float block_sum(float v, float *red) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -55,8 +55,22 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float4 *__restri
 // (LayerNorm with mean_norm = false: std_norm then weight, norm.rs:56-71, unary.rs:93-104).
 // One block of 1024 threads per row; each thread keeps up to 4 float4 of the row in
 // registers between the two passes (dim <= 16384, dim % 4 == 0); x_out may alias x.
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT *p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4<float>(float *p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4 *>(p) = make_float4(a, b, c, d);
+}
+template <>
+__device__ __forceinline__ void store4<__bf16>(__bf16 *p, float a, float b, float c, float d) {  // round to nearest even
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<bf16x4 *>(p) = bf16x4{static_cast<__bf16>(a), static_cast<__bf16>(b), static_cast<__bf16>(c),
+                                            static_cast<__bf16>(d)};
+}
+
+template <typename OutT>
 __global__ __launch_bounds__(1024) void rms_norm_kernel(const float *x, const float *res, float *x_out,
-                                                        const float *__restrict__ w, float *__restrict__ y, int dim,
+                                                        const float *__restrict__ w, OutT *__restrict__ y, int dim,
                                                         float eps) {
     __shared__ float red[16];
     const size_t base = static_cast<size_t>(blockIdx.x) * dim;
@@ -92,8 +106,8 @@ __global__ __launch_bounds__(1024) void rms_norm_kernel(const float *x, const fl
         const int j = threadIdx.x + i * 1024;
         if (j < dim4) {
             const float4 g = reinterpret_cast<const float4 *>(w)[j];
-            reinterpret_cast<float4 *>(y + base)[j] =
-                make_float4(v[i].x * scale * g.x, v[i].y * scale * g.y, v[i].z * scale * g.z, v[i].w * scale * g.w);
+            store4<OutT>(y + base + 4 * j, v[i].x * scale * g.x, v[i].y * scale * g.y, v[i].z * scale * g.z,
+                         v[i].w * scale * g.w);
         }
     }
 }
@@ -246,7 +260,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(const float *__
 }
 
 // out[s][j] = up * swish(gate), gate = gu[s][j], up = gu[s][f + j]   (model.rs:24-32)
-__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gu, float *__restrict__ out, int f,
+template <typename OutT>
+__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gu, OutT *__restrict__ out, int f,
                                                      size_t total, int interleaved) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= total) return;
@@ -254,7 +269,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
     const int j = static_cast<int>(i - s * f);
     const float g = gu[s * 2 * f + (interleaved ? 2 * j : j)];
     const float u = gu[s * 2 * f + (interleaved ? 2 * j + 1 : f + j)];
-    out[i] = u * (g * (1.0f / (1.0f + expf(-g))));
+    out[i] = static_cast<OutT>(u * (g * (1.0f / (1.0f + expf(-g)))));
 }
 
 __global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ y,
@@ -336,6 +351,32 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     }
 }
 
+template <typename OutT>
+static lhip_status rms_norm_any(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
+                                OutT *y_dev, int64_t rows, int64_t dim, float eps, void *stream) {
+    if (!x_dev || !w_dev || !y_dev || (residual_dev && !x_out_dev)) return LHIP_ERR_NULL_PTR;
+    if (rows <= 0 || dim <= 0 || rows > kMaxDim || dim > 16384 || dim % 4 != 0) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(x_dev, 16) || !aligned(w_dev, 16) || !aligned(y_dev, 4 * sizeof(OutT)) ||
+        (residual_dev && (!aligned(residual_dev, 16) || !aligned(x_out_dev, 16))))
+        return LHIP_ERR_MISALIGNED;
+    hipLaunchKernelGGL(rms_norm_kernel<OutT>, dim3(static_cast<unsigned>(rows)), dim3(1024), 0, as_stream(stream), x_dev,
+                       residual_dev, x_out_dev, w_dev, y_dev, static_cast<int>(dim), eps);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+template <typename OutT>
+static lhip_status swiglu_any(const float *gate_up_dev, OutT *out_dev, int64_t rows, int64_t f, int interleaved,
+                              void *stream) {
+    if (!gate_up_dev || !out_dev) return LHIP_ERR_NULL_PTR;
+    if (rows <= 0 || f <= 0 || rows > kMaxDim || f > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    const size_t total = static_cast<size_t>(rows) * static_cast<size_t>(f);
+    hipLaunchKernelGGL(swiglu_kernel<OutT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), gate_up_dev, out_dev, static_cast<int>(f), total, interleaved);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
 }  // namespace lhip
 
 using namespace lhip;
@@ -357,15 +398,14 @@ lhip_status lhip_gather_rows_f32(const float *table_dev, const float *idx_dev, f
 
 lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
                               float *y_dev, int64_t rows, int64_t dim, float eps, void *stream) {
-    if (!x_dev || !w_dev || !y_dev || (residual_dev && !x_out_dev)) return LHIP_ERR_NULL_PTR;
-    if (rows <= 0 || dim <= 0 || rows > kMaxDim || dim > 16384 || dim % 4 != 0) return LHIP_ERR_INVALID_SHAPE;
-    if (!aligned(x_dev, 16) || !aligned(w_dev, 16) || !aligned(y_dev, 16) ||
-        (residual_dev && (!aligned(residual_dev, 16) || !aligned(x_out_dev, 16))))
-        return LHIP_ERR_MISALIGNED;
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<unsigned>(rows)), dim3(1024), 0, as_stream(stream), x_dev,
-                       residual_dev, x_out_dev, w_dev, y_dev, static_cast<int>(dim), eps);
-    LHIP_CHECK_LAUNCH();
-    return LHIP_OK;
+    return rms_norm_any<float>(x_dev, residual_dev, x_out_dev, w_dev, y_dev, rows, dim, eps, stream);
+}
+
+lhip_status lhip_rms_norm_f32_bf16out(const float *x_dev, const float *residual_dev, float *x_out_dev,
+                                      const float *w_dev, void *y_bf16_dev, int64_t rows, int64_t dim, float eps,
+                                      void *stream) {
+    return rms_norm_any<__bf16>(x_dev, residual_dev, x_out_dev, w_dev, static_cast<__bf16 *>(y_bf16_dev), rows, dim, eps,
+                                stream);
 }
 
 lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v_cache_dev, const int32_t *pos_dev,
@@ -391,7 +431,7 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
         max_seq <= 0 || q_heads % kv_heads != 0 || tokens > kMaxDim || q_heads > 65535 || max_seq > 12000)
         return LHIP_ERR_INVALID_SHAPE;  // the score row of one query lives in LDS
     if (tokens >= 8 && aligned(qkv_dev, 16) && aligned(k_cache_dev, 16) && aligned(v_cache_dev, 16) && aligned(out_dev, 16) &&
-        attention_prefill_launch(qkv_dev, k_cache_dev, v_cache_dev, out_dev, pos_dev, static_cast<int>(tokens),
+        attention_prefill_launch(qkv_dev, k_cache_dev, v_cache_dev, out_dev, false, pos_dev, static_cast<int>(tokens),
                                  static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
                                  static_cast<int>(max_seq), as_stream(stream))) {
         LHIP_CHECK_LAUNCH();
@@ -406,15 +446,31 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
     return LHIP_OK;
 }
 
-lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,
-                            void *stream) {
-    if (!gate_up_dev || !out_dev) return LHIP_ERR_NULL_PTR;
-    if (rows <= 0 || f <= 0 || rows > kMaxDim || f > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
-    const size_t total = static_cast<size_t>(rows) * static_cast<size_t>(f);
-    hipLaunchKernelGGL(swiglu_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       gate_up_dev, out_dev, static_cast<int>(f), total, interleaved);
+lhip_status lhip_attention_f32_bf16out(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
+                                       void *out_bf16_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
+                                       int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream) {
+    if (!qkv_dev || !k_cache_dev || !v_cache_dev || !out_bf16_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
+    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_seq <= 0 || q_heads % kv_heads != 0 ||
+        tokens > kMaxDim || max_seq > kMaxDim)
+        return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(qkv_dev, 16) || !aligned(k_cache_dev, 16) || !aligned(v_cache_dev, 16) || !aligned(out_bf16_dev, 8))
+        return LHIP_ERR_MISALIGNED;
+    if (!attention_prefill_launch(qkv_dev, k_cache_dev, v_cache_dev, out_bf16_dev, true, pos_dev, static_cast<int>(tokens),
+                                  static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
+                                  static_cast<int>(max_seq), as_stream(stream)))
+        return LHIP_ERR_UNSUPPORTED;  // only the matrix-core kernel writes bf16
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
+}
+
+lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,
+                            void *stream) {
+    return swiglu_any<float>(gate_up_dev, out_dev, rows, f, interleaved, stream);
+}
+
+lhip_status lhip_swiglu_f32_bf16out(const float *gate_up_dev, void *out_bf16_dev, int64_t rows, int64_t f,
+                                    int interleaved, void *stream) {
+    return swiglu_any<__bf16>(gate_up_dev, static_cast<__bf16 *>(out_bf16_dev), rows, f, interleaved, stream);
 }
 
 lhip_status lhip_add_f32(float *x_dev, const float *y_dev, int64_t n, void *stream) {

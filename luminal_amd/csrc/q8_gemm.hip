@@ -47,11 +47,12 @@ __device__ __forceinline__ uint2 dequant4_bf16(uint32_t q4, float d) {
 }
 
 // D = register prefetch depth in K tiles (D > 1 needs K % (64*D) == 0 and D even).
-template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
+// OutT = __bf16 (rounded to nearest even) or float (the accumulators as they are).
+template <int BM, int BN, int WM, int WN, int D, bool PIPE = false, typename OutT = __bf16>
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
                                                                    const __half *__restrict__ ds,
                                                                    const __bf16 *__restrict__ x,
-                                                                   __bf16 *__restrict__ y, int M, int N, int K,
+                                                                   OutT *__restrict__ y, int M, int N, int K,
                                                                    int m_tiles, int n_tiles) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
@@ -239,27 +240,78 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = static_cast<__bf16>(acc[i][j][v]);
+                if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = static_cast<OutT>(acc[i][j][v]);
             }
         }
 }
 
-template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
-static lhip_status launch_gemm(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
-                               hipStream_t s) {
+template <int BM, int BN, int WM, int WN, int D, bool PIPE, typename OutT>
+static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
+                                 hipStream_t s) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
-    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, PIPE>;
+    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, PIPE, OutT>;
     if (lds_bytes > 64 * 1024) {
         // Opting in to more than 64 KiB of dynamic LDS is a per-function attribute.
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     }
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad)), dim3(WM * WN * 64), lds_bytes, s, qs,
-                       ds, static_cast<const __bf16 *>(x), static_cast<__bf16 *>(y), m, n, k, m_tiles, n_tiles);
+                       ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m, n, k, m_tiles, n_tiles);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
+}
+
+template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
+static lhip_status launch_gemm(bool f32_out, const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n,
+                               int k, hipStream_t s) {
+    return f32_out ? launch_gemm_t<BM, BN, WM, WN, D, PIPE, float>(qs, ds, x, y, m, n, k, s)
+                   : launch_gemm_t<BM, BN, WM, WN, D, PIPE, __bf16>(qs, ds, x, y, m, n, k, s);
+}
+
+static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
+                                 int tile, bool f32_out, void *stream) {
+    if (!planar_dev || !x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (k % kBK != 0) return LHIP_ERR_UNSUPPORTED;
+    if (!aligned(planar_dev, 256) || !aligned(x_dev, 16) || !aligned(y_dev, f32_out ? 4 : 2)) return LHIP_ERR_MISALIGNED;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    auto *qs = reinterpret_cast<const int8_t *>(base);
+    auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
+    const int mi = static_cast<int>(m), ni = static_cast<int>(n), ki = static_cast<int>(k);
+    hipStream_t s = as_stream(stream);
+    // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
+    const bool deep = (k % (kBK * 4)) == 0;
+#define LHIP_TILE(BM, BN, WM, WN)                                                                  \
+    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s) \
+                : launch_gemm<BM, BN, WM, WN, 1>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
+    switch (tile) {
+        case 0: LHIP_TILE(256, 128, 4, 2);
+        case 1: LHIP_TILE(128, 128, 2, 2);
+        case 2: LHIP_TILE(128, 64, 2, 2);
+        case 3: LHIP_TILE(64, 64, 2, 2);
+        case 4:  // 256x256 by eight 64x128 waves: 0.75 KiB of LDS operand reads per MFMA instead of 1; both
+                 // LDS buffers together are 144 KiB, which leaves registers for a prefetch depth of two K tiles
+            if (k % (kBK * 2) != 0) return LHIP_ERR_UNSUPPORTED;
+            return launch_gemm<256, 256, 4, 2, 2, true>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s);
+        default: return LHIP_ERR_UNSUPPORTED;
+    }
+#undef LHIP_TILE
+}
+
+static int gemm_auto_tile(int64_t m, int64_t n, int64_t k) {
+    // Largest tile that still gives at least three quarters of the 256 CUs a
+    // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
+    // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
+    auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    int tile = 3;
+    if (m > 128 && k % (kBK * 2) == 0 && blocks(256, 256) >= 192) tile = 4;
+    else if (m > 128 && blocks(256, 128) >= 192) tile = 0;
+    else if (blocks(128, 128) >= 192) tile = 1;
+    else if (blocks(128, 64) >= 192) tile = 2;
+    return tile;
 }
 
 }  // namespace lhip
@@ -270,47 +322,17 @@ extern "C" {
 
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream) {
-    if (!planar_dev || !x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
-    if (lhip_status s = check_q8_shape(n, k)) return s;
-    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
-    if (k % kBK != 0) return LHIP_ERR_UNSUPPORTED;
-    if (!aligned(planar_dev, 256) || !aligned(x_dev, 16) || !aligned(y_dev, 2)) return LHIP_ERR_MISALIGNED;
-    auto *base = static_cast<const uint8_t *>(planar_dev);
-    auto *qs = reinterpret_cast<const int8_t *>(base);
-    auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
-    const int mi = static_cast<int>(m), ni = static_cast<int>(n), ki = static_cast<int>(k);
-    hipStream_t s = as_stream(stream);
-    // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
-    const bool deep = (k % (kBK * 4)) == 0;
-#define LHIP_TILE(BM, BN, WM, WN)                                                                  \
-    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(qs, ds, x_dev, y_dev, mi, ni, ki, s)        \
-                : launch_gemm<BM, BN, WM, WN, 1>(qs, ds, x_dev, y_dev, mi, ni, ki, s)
-    switch (tile) {
-        case 0: LHIP_TILE(256, 128, 4, 2);
-        case 1: LHIP_TILE(128, 128, 2, 2);
-        case 2: LHIP_TILE(128, 64, 2, 2);
-        case 3: LHIP_TILE(64, 64, 2, 2);
-        case 4:  // 256x256 by eight 64x128 waves: 0.75 KiB of LDS operand reads per MFMA instead of 1; both
-                 // LDS buffers together are 144 KiB, which leaves registers for a prefetch depth of two K tiles
-            if (k % (kBK * 2) != 0) return LHIP_ERR_UNSUPPORTED;
-            return launch_gemm<256, 256, 4, 2, 2, true>(qs, ds, x_dev, y_dev, mi, ni, ki, s);
-        default: return LHIP_ERR_UNSUPPORTED;
-    }
-#undef LHIP_TILE
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, tile, false, stream);
 }
 
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream) {
-    // Largest tile that still gives at least three quarters of the 256 CUs a
-    // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
-    // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
-    auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    int tile = 3;
-    if (m > 128 && k % (kBK * 2) == 0 && blocks(256, 256) >= 192) tile = 4;
-    else if (m > 128 && blocks(256, 128) >= 192) tile = 0;
-    else if (blocks(128, 128) >= 192) tile = 1;
-    else if (blocks(128, 64) >= 192) tile = 2;
-    return lhip_q8_0_matmul_bf16_cfg(planar_dev, x_dev, y_dev, m, n, k, tile, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), false, stream);
+}
+
+lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_dev, float *y_dev, int64_t m, int64_t n,
+                                         int64_t k, void *stream) {
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), true, stream);
 }
 
 }  // extern "C"

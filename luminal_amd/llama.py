@@ -103,6 +103,8 @@ class LlamaQ8:
         """Runs s tokens (ids as f32 on the device) at positions pos .. pos+s-1, appends to the KV cache and
         returns the logits of the last position ((vocab,)), or of all positions ((s, vocab)).
         Does not advance the position."""
+        if bf16 and s > 1:
+            return self._forward_prompt_bf16(tokens_f32, s, all_logits)
         cfg, lib, w = self.cfg, self.lib, self.w
         d, hd = cfg.dim, cfg.head_dim
         h = self._buf("h", (s, d))
@@ -143,6 +145,66 @@ class LlamaQ8:
         logits = self._buf("logits", (cfg.vocab,))
         last = n[s - 1]
         self._matmul(w["lm_head"], last, logits, 1, False)  # only the last position is read (main.rs:58-61)
+        return logits
+
+    def _forward_prompt_bf16(self, tokens_f32: torch.Tensor, s: int, all_logits: bool):
+        """Prompt pass with the linears on the bf16 matrix-core GEMM.  The residual stream, rotary, attention and
+        softmax stay f32; the operators in front of a GEMM write bf16 and the GEMM stores its f32 accumulators, so
+        there is no cast kernel anywhere."""
+        cfg, lib, w = self.cfg, self.lib, self.w
+        d, hd = cfg.dim, cfg.head_dim
+        bf = torch.bfloat16
+        h = self._buf("h", (s, d))
+        nb = self._buf("nb", (s, d), bf)
+        qkv = self._buf("qkv", (s, cfg.qkv_rows))
+        attb = self._buf("attb", (s, d), bf)
+        att = self._buf("att", (s, d))
+        o = self._buf("o", (s, d))
+        gu = self._buf("gu", (s, 2 * cfg.ffn))
+        actb = self._buf("actb", (s, cfg.ffn), bf)
+        dn = self._buf("dn", (s, d))
+
+        def norm(res, wt):
+            capi.check(lib.lhip_rms_norm_f32_bf16out(h.data_ptr(), res.data_ptr() if res is not None else None,
+                                                     h.data_ptr() if res is not None else None, wt.data_ptr(),
+                                                     nb.data_ptr(), s, d, cfg.eps, _s()), "lhip_rms_norm_f32_bf16out")
+
+        def gemm(wq, x, y, m):
+            capi.check(lib.lhip_q8_0_matmul_bf16_f32out(wq.planar.data_ptr(), x.data_ptr(), y.data_ptr(), m, wq.n, wq.k,
+                                                        _s()), "lhip_q8_0_matmul_bf16_f32out")
+
+        capi.check(lib.lhip_gather_rows_f32(w["embed"].data_ptr(), tokens_f32.data_ptr(), h.data_ptr(), s, cfg.vocab,
+                                            d, _s()), "lhip_gather_rows_f32")
+        for i in range(cfg.layers):
+            norm(None if i == 0 else dn, w[f"{i}.attn_norm"])       # h += previous MLP out; nb = norm(h)
+            gemm(w[f"{i}.qkv"], nb, qkv, s)
+            capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                   self.v_cache[i].data_ptr(), self.pos.data_ptr(), s, cfg.q_heads,
+                                                   cfg.kv_heads, hd, self.max_seq, cfg.theta, _s()), "rope")
+            st = lib.lhip_attention_f32_bf16out(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                                attb.data_ptr(), self.pos.data_ptr(), s, cfg.q_heads, cfg.kv_heads, hd,
+                                                self.max_seq, _s())
+            if st == capi.LHIP_ERR_UNSUPPORTED:  # head shape without a matrix-core kernel: f32 attention, then cast
+                capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                  self.v_cache[i].data_ptr(), att.data_ptr(), self.pos.data_ptr(), s,
+                                                  cfg.q_heads, cfg.kv_heads, hd, self.max_seq, _s()), "attention")
+                capi.check(lib.lhip_cast_f32_to_bf16(att.data_ptr(), attb.data_ptr(), s * d, _s()), "cast")
+            else:
+                capi.check(st, "lhip_attention_f32_bf16out")
+            gemm(w[f"{i}.o"], attb, o, s)
+            norm(o, w[f"{i}.ffn_norm"])                              # h += attention out; nb = norm(h)
+            gemm(w[f"{i}.gate_up"], nb, gu, s)
+            capi.check(lib.lhip_swiglu_f32_bf16out(gu.data_ptr(), actb.data_ptr(), s, cfg.ffn, 1, _s()), "swiglu")
+            gemm(w[f"{i}.down"], actb, dn, s)
+        if all_logits:
+            norm(dn, w["out_norm"])
+            logits = self._buf("logits_all", (s, cfg.vocab))
+            gemm(w["lm_head"], nb, logits, s)
+            return logits
+        n = self._buf("n", (s, d))
+        self._norm(h, dn, h, w["out_norm"], n, s)                   # last residual + final norm, f32
+        logits = self._buf("logits", (cfg.vocab,))
+        self._matmul(w["lm_head"], n[s - 1], logits, 1, False)      # only the last position is read (main.rs:58-61)
         return logits
 
     def _build_plans(self):

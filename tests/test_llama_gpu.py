@@ -273,14 +273,77 @@ def test_graph_replay_equals_eager_decode(oracle, cfg):
     assert np.array_equal(eng.decode(10, use_graph=True).cpu().numpy(), eager)
 
 
-def test_bf16_prefill_then_f32_decode(oracle):
-    cfg = LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)
+@pytest.mark.parametrize("cfg", [LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512),
+                                 LlamaConfig(vocab=700, dim=1024, layers=2, q_heads=8, kv_heads=2, ffn=2048),
+                                 LlamaConfig(vocab=300, dim=768, layers=1, q_heads=12, kv_heads=4, ffn=256)])
+def test_bf16_prefill_then_f32_decode(oracle, cfg):
+    """The prompt pass on the bf16 GEMM (the third configuration has 3 query heads per KV head, for which there is
+    no matrix-core attention: it takes the f32 attention + cast branch)."""
     eng, wf = build_model(oracle, cfg, seed=9)
     prompt = [int(t) for t in np.random.default_rng(4).integers(0, cfg.vocab, 20)]
-    want = lo.forward(cfg, wf, prompt, empty_cache(cfg), empty_cache(cfg), 0)[-1]
+    kc, vc = empty_cache(cfg), empty_cache(cfg)
+    want = lo.forward(cfg, wf, prompt, kc, vc, 0)
+    t = np.asarray(want[-1])
     got = eng.prefill(prompt, bf16=True).cpu().numpy()
-    t = np.asarray(want)
     assert np.max(np.abs(got - t)) / np.sqrt(np.mean(t * t)) < 5e-2  # bf16 matmuls through the whole stack
+    eng.reset()
+    allpos = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True,
+                         all_logits=True).cpu().numpy()
+    assert np.max(np.abs(allpos - want)) / np.sqrt(np.mean(want * want)) < 5e-2
+    # the f32 decode step continues from the cache the bf16 pass wrote
+    eng.reset()
+    eng.prefill(prompt, bf16=True)
+    tok = lo.argmax_last(want[-1])
+    eng.tok.fill_(float(tok))
+    step = lo.forward(cfg, wf, [tok], kc, vc, len(prompt))[0]
+    got_step = eng.decode_step().cpu().numpy()
+    assert np.max(np.abs(got_step - step)) / np.sqrt(np.mean(step * step)) < 5e-2
+
+
+def test_bf16_output_forms_equal_the_rounded_f32_forms():
+    """rms norm, SwiGLU and prompt attention writing bf16 are the f32 operators followed by round-to-nearest-even."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(8)
+
+    def rounded(t):
+        return t.to(torch.bfloat16)
+
+    rows, dim = 5, 1024
+    x = torch.from_numpy(rng.standard_normal((rows, dim)).astype(np.float32)).to(DEV)
+    res = torch.from_numpy(rng.standard_normal((rows, dim)).astype(np.float32)).to(DEV)
+    g = torch.from_numpy((1 + 0.1 * rng.standard_normal(dim)).astype(np.float32)).to(DEV)
+    y32, xo32 = torch.empty_like(x), torch.empty_like(x)
+    y16 = torch.empty((rows, dim), dtype=torch.bfloat16, device=DEV)
+    xo16 = torch.empty_like(x)
+    assert lib.lhip_rms_norm_f32(x.data_ptr(), res.data_ptr(), xo32.data_ptr(), g.data_ptr(), y32.data_ptr(), rows, dim,
+                                 1e-5, s()) == 0
+    assert lib.lhip_rms_norm_f32_bf16out(x.data_ptr(), res.data_ptr(), xo16.data_ptr(), g.data_ptr(), y16.data_ptr(),
+                                         rows, dim, 1e-5, s()) == 0
+    assert torch.equal(y16, rounded(y32)) and torch.equal(xo16, xo32)
+
+    f = 96
+    gu = torch.from_numpy(rng.standard_normal((3, 2 * f)).astype(np.float32)).to(DEV)
+    for inter in (0, 1):
+        o32 = torch.empty((3, f), device=DEV)
+        o16 = torch.empty((3, f), dtype=torch.bfloat16, device=DEV)
+        assert lib.lhip_swiglu_f32(gu.data_ptr(), o32.data_ptr(), 3, f, inter, s()) == 0
+        assert lib.lhip_swiglu_f32_bf16out(gu.data_ptr(), o16.data_ptr(), 3, f, inter, s()) == 0
+        assert torch.equal(o16, rounded(o32))
+
+    hq, hkv, hd, S, max_seq = 8, 2, 128, 37, 64
+    qkv = torch.from_numpy(rng.standard_normal((S, (hq + 2 * hkv) * hd)).astype(np.float32)).to(DEV)
+    kc = torch.from_numpy(rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)).to(DEV)
+    vc = torch.from_numpy(rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)).to(DEV)
+    pos = torch.tensor([9], dtype=torch.int32, device=DEV)
+    a32 = torch.empty((S, hq * hd), device=DEV)
+    a16 = torch.empty((S, hq * hd), dtype=torch.bfloat16, device=DEV)
+    assert lib.lhip_attention_f32(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), a32.data_ptr(), pos.data_ptr(), S, hq,
+                                  hkv, hd, max_seq, s()) == 0
+    assert lib.lhip_attention_f32_bf16out(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), a16.data_ptr(), pos.data_ptr(),
+                                          S, hq, hkv, hd, max_seq, s()) == 0
+    assert torch.equal(a16, rounded(a32))
+    assert lib.lhip_attention_f32_bf16out(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), a16.data_ptr(), pos.data_ptr(),
+                                          S, 6, 2, hd, max_seq, s()) == capi.LHIP_ERR_UNSUPPORTED
 
 
 def test_gguf_loader_gives_the_same_model(oracle, tmp_path):

@@ -136,3 +136,24 @@ def test_gemm_argument_errors():
         capi.LHIP_ERR_INVALID_SHAPE
     assert lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 4, 64, 128, 9, s) == \
         capi.LHIP_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("m,n,k", [(70, 150, 512), (300, 700, 1024), (513, 600, 2048)])
+def test_f32_output_is_the_unrounded_accumulator(oracle, m, n, k):
+    """lhip_q8_0_matmul_bf16_f32out: same kernel, accumulators stored as f32 — rounding them gives the bf16 form bit
+    for bit, and they sit within the bf16-path bar of the f64 truth."""
+    lib = capi.load_library()
+    qs, d = synth.q8_0_random(n, k, seed=m + n)
+    xf, bits = bf16_activations(oracle, m, k, seed=3)
+    w = upload(qs, d)
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y16 = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    y32 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), x.data_ptr(), y16.data_ptr(), m, n, k, st) == 0
+    assert lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st) == 0
+    assert torch.equal(y32.to(torch.bfloat16), y16)
+    elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+    assert lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr() + 2, m, n, k,
+                                            st) == capi.LHIP_ERR_MISALIGNED
