@@ -25,6 +25,9 @@
 // bf16 MFMA over rounded weights would be.
 #include "common.h"
 
+#include <type_traits>
+#include <utility>
+
 namespace lhip {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -32,7 +35,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t mu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kChunk = 128;      // K elements per MFMA
-constexpr int kARow = 144;       // LDS bytes per activation row of a chunk: 128 fp8 + 16 padding
+constexpr int kARow = 160;       // LDS bytes per activation row of a chunk: 128 fp8 + 32 padding (with 16 the fragment reads,
+                                 // lane (r, g) at r * pitch + 16 g, take twice as long: measured 8.0 against 4.3 cycles per read)
 
 static inline int64_t pad128(int64_t k) { return (k + 127) / 128 * 128; }
 
@@ -246,6 +250,16 @@ struct MoeGemmArgs {
     void *out;                          // bf16 [R][N] (gated) or f32 [R][N]
 };
 
+// f(integral_constant<int, 1>) ... f(integral_constant<int, N-1>), expanded at compile time.
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_from1_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is + 1>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for_from1(F &&f) {
+    static_for_from1_impl(static_cast<F &&>(f), std::make_integer_sequence<int, (N > 1 ? N - 1 : 0)>{});
+}
+
 template <int MT, int NT>
 struct BSet {
     mu32x4 q[NT];
@@ -258,7 +272,8 @@ struct BSet {
 // and one wave's waits (LDS, barrier, weight stream) are covered by the other's matrix work.
 // D = weight prefetch distance in chunks (even).
 template <int MT, int NT, bool GATED, int WR, int D>
-__global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
+__global__ __launch_bounds__(256 * WR) __attribute__((amdgpu_waves_per_eu(1, (MT >= 8 && WR == 1) ? 1 : 8)))
+void mx_moe_gemm_kernel(MoeGemmArgs g) {
     static_assert(!GATED || NT % 2 == 0, "gated tiles pair each gate fragment with its up fragment");
     static_assert(MT % WR == 0 && D % 2 == 0, "tile shape");
     constexpr int BM = 16 * MT;
@@ -268,19 +283,22 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
     constexpr int A_PLANE = BM * kARow;
     constexpr int A_BUF = 2 * A_PLANE + BM * 4;  // hi, lo, scales
 
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x A_BUF
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 3 x A_BUF
 
+    // The tile's description is read together with the tile count (the plan arrays have an entry for
+    // every workgroup of the grid), so an unused workgroup costs one memory round trip, not two.
     const int tile = blockIdx.y;
-    if (tile >= *g.n_tiles) return;
+    const int n_tiles = *g.n_tiles;
     const int expert = g.tile_expert[tile];
     const int row0 = g.tile_row0[tile];
     const int rows = g.tile_rows[tile];
+    if (tile >= n_tiles) return;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave = wave_id & 3;    // column group
-    const int wrow = wave_id >> 2;   // row half (WR = 2)
+    const int wrow = WR == 1 ? 0 : wave_id >> 2;  // row group
     const int r = lane & 15, grp = lane >> 4;
     const int Kp = g.Kp;
     const int chunks = Kp / kChunk;
@@ -309,7 +327,7 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         s_tile[f] = g.w_sc + panel * chunks * 64 + lane;
     }
     BSet<MT, NT> bs[D];
-    auto load_b = [&](int set, int c) {
+    auto load_b = [&](int set, int c) __attribute__((always_inline)) {
         // Dead chunks (past the padded K) re-read the last chunk; compute() zeroes them.
         // (Masking here, next to the loads, would make the wave wait for data it has only just requested.)
         bs[set].valid = c < chunks;
@@ -328,7 +346,7 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         }
     };
 
-    // ---- activation tile: global -> registers -> LDS (double-buffered), shared by the 4 waves
+    // ---- activation tile: global -> registers -> LDS (three buffers), shared by all waves
     const uint8_t *a_src[STG];
     int a_dst[STG];
 #pragma unroll
@@ -347,22 +365,23 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         const int arow = g.a_index ? g.a_index[slot] / g.a_div : slot;
         as_src = g.a_sc + static_cast<size_t>(arow) * (Kp / 32);
     }
-    mu32x4 a_reg[STG];
-    uint32_t as_reg = 0;
-    auto load_a = [&](int c) {
-        const int cc = min(c, chunks - 1);  // dead chunks re-read the last one; their weights are zero
-#pragma unroll
-        for (int i = 0; i < STG; ++i) a_reg[i] = *reinterpret_cast<const mu32x4 *>(a_src[i] + cc * kChunk);
-        if (tid < BM) as_reg = *reinterpret_cast<const uint32_t *>(as_src + cc * 4);
+    struct AStage {
+        mu32x4 q[STG];
+        uint32_t s;
     };
-    auto store_a = [&](int buf) {
-        unsigned char *base = lds + buf * A_BUF;
+    auto load_a = [&](AStage &st, int c) __attribute__((always_inline)) {
+        const int cc = min(c, chunks - 1);  // dead chunks re-read the last one; they are not multiplied
+#pragma unroll
+        for (int i = 0; i < STG; ++i) st.q[i] = *reinterpret_cast<const mu32x4 *>(a_src[i] + cc * kChunk);
+        if (tid < BM) st.s = *reinterpret_cast<const uint32_t *>(as_src + cc * 4);
+    };
+    auto store_a = [&](AStage &st, unsigned char *base) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < STG; ++i) {
-            asm volatile("" : "+v"(a_reg[i]));
-            *reinterpret_cast<mu32x4 *>(base + a_dst[i]) = a_reg[i];
+            asm volatile("" : "+v"(st.q[i]));
+            *reinterpret_cast<mu32x4 *>(base + a_dst[i]) = st.q[i];
         }
-        if (tid < BM) *reinterpret_cast<uint32_t *>(base + 2 * A_PLANE + tid * 4) = as_reg;
+        if (tid < BM) *reinterpret_cast<uint32_t *>(base + 2 * A_PLANE + tid * 4) = st.s;
     };
 
     v4f acc[MTW][NT];
@@ -376,74 +395,107 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
         mu32x4 h0, h1, l0, l1;
         uint32_t sw;
     };
-    auto load_frag = [&](const unsigned char *base, int i) {
-        const unsigned char *p = base + (i * 16 + r) * kARow + grp * 16;
+    // Fragment `n` of this wave's row group (tile fragment n * WR + wrow): the lane's part of the address is
+    // fixed, so every read of a chunk is one base register plus an immediate offset.
+    const int frag_lane = (wrow * 16 + r) * kARow + grp * 16;
+    const int scale_lane = 2 * A_PLANE + (wrow * 16 + r) * 4;
+    auto load_frag = [&](const unsigned char *base, int n) __attribute__((always_inline)) {
+        const unsigned char *p = base + frag_lane + n * (WR * 16 * kARow);
         AFrag a;
         a.h0 = *reinterpret_cast<const mu32x4 *>(p);
         a.h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
         a.l0 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE);
         a.l1 = *reinterpret_cast<const mu32x4 *>(p + A_PLANE + 64);
-        a.sw = *reinterpret_cast<const uint32_t *>(base + 2 * A_PLANE + (i * 16 + r) * 4);
+        a.sw = *reinterpret_cast<const uint32_t *>(base + scale_lane + n * (WR * 16 * 4));
         return a;
     };
-    auto compute = [&](int set, int buf) {
-        const unsigned char *base = lds + buf * A_BUF;
-        mu32x4 bq[NT];
-        int bsc[NT];
+    // The MFMAs of row fragment i against the NT weight fragments of a set.
+    auto mfma_frag = [&](int set, const AFrag &cur, int i) __attribute__((always_inline)) {
+        const int sa = static_cast<int>((cur.sw >> (8 * grp)) & 0xff);
+        const v8i ah = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
+                        (int)cur.h1.x, (int)cur.h1.y, (int)cur.h1.z, (int)cur.h1.w};
+        const v8i al = {(int)cur.l0.x, (int)cur.l0.y, (int)cur.l0.z, (int)cur.l0.w,
+                        (int)cur.l1.x, (int)cur.l1.y, (int)cur.l1.z, (int)cur.l1.w};
 #pragma unroll
         for (int f = 0; f < NT; ++f) {
-            asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
-            const mu32x4 zero = {0, 0, 0, 0};
-            bq[f] = bs[set].valid ? bs[set].q[f] : zero;
-            bsc[f] = bs[set].valid ? static_cast<int>(bs[set].s[f]) : 127;
-        }
-        // The LDS reads of fragment i+1 are issued before the MFMAs of fragment i and
-        // fenced there, so two fragments are live at a time instead of all MT.
-        // Row fragments are dealt round-robin to the WR row groups, so a short tile still occupies all waves.
-        AFrag cur = load_frag(base, wrow);
-#pragma unroll
-        for (int i = 0; i < MTW; ++i) {
-            if (i * WR + wrow >= frags) break;  // wave-uniform: this tile has no rows there
-            AFrag nxt = cur;
-            if (i + 1 < MTW && (i + 1) * WR + wrow < frags) nxt = load_frag(base, (i + 1) * WR + wrow);
-            __builtin_amdgcn_sched_barrier(0);
-            const int sa = static_cast<int>((cur.sw >> (8 * grp)) & 0xff);
-            const v8i ah = {(int)cur.h0.x, (int)cur.h0.y, (int)cur.h0.z, (int)cur.h0.w,
-                            (int)cur.h1.x, (int)cur.h1.y, (int)cur.h1.z, (int)cur.h1.w};
-            const v8i al = {(int)cur.l0.x, (int)cur.l0.y, (int)cur.l0.z, (int)cur.l0.w,
-                            (int)cur.l1.x, (int)cur.l1.y, (int)cur.l1.z, (int)cur.l1.w};
-#pragma unroll
-            for (int f = 0; f < NT; ++f) {
-                const v8i b = {(int)bq[f].x, (int)bq[f].y, (int)bq[f].z, (int)bq[f].w, 0, 0, 0, 0};
-                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, bsc[f]);
-                acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, bsc[f]);
-                // Pin the accumulation here: nothing else reads acc until the epilogue, and
-                // without this the optimiser sinks every MFMA of the unrolled pipeline to its
-                // end, keeping the fragments of all its steps alive.
-                asm volatile("" : "+a"(acc[i][f]));
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            cur = nxt;
+            const mu32x4 &q = bs[set].q[f];
+            const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
+            const int sb = static_cast<int>(bs[set].s[f]);
+            acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+            acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+            // Pin the accumulation here: nothing else reads acc until the epilogue, and
+            // without this the optimiser sinks every MFMA of the unrolled pipeline to its
+            // end, keeping the fragments of all its steps alive.
+            asm volatile("" : "+a"(acc[i][f]));
         }
     };
 
-    // ---- pipeline
+    // ---- pipeline: three LDS buffers, one barrier per chunk, placed in the MIDDLE of the chunk's matrix work.
+    // Chunk c multiplies out of buffer c % 3.  After the MFMAs of its first row fragment every wave passes the
+    // barrier and then writes chunk c+2 (requested during chunk c-1) into buffer (c+2) % 3: that buffer was last
+    // read in chunk c-1, which every wave has left by then; and chunk c+2 is first read after the barrier of
+    // chunk c+1, by when every wave has written it.  So nothing waits at a chunk boundary (the first fragment of
+    // chunk c+1 is read right after the barrier of chunk c), a wave arriving at the barrier has its own and its
+    // SIMD neighbour's MFMAs in flight, and the staging traffic runs under matrix work.
+    // A dead chunk (past the padded K, there only to keep the unrolled shape) skips its MFMAs (wave-uniform).
+    // The prologue issues its loads in the loop's order (activation stage, then the youngest weight set):
+    // the compiler's wait counts inside the loop are the stricter of what the prologue and the previous
+    // trip leave outstanding, and with the stage requested last here the loop would wait for the weight
+    // set it has only just requested every time it stores a stage.
+    AStage stage, stage2;
 #pragma unroll
-    for (int j = 0; j < D; ++j) load_b(j, j);
-    load_a(0);
-    store_a(0);
+    for (int j = 0; j + 1 < D; ++j) load_b(j, j);
+    load_a(stage, 0);
+    load_a(stage2, 1);
+    store_a(stage, lds);
+    store_a(stage2, lds + A_BUF);
+    load_a(stage, 2);
+    load_b(D - 1, D - 1);
     __syncthreads();
+    unsigned char *cur = lds, *nxt = lds + A_BUF, *fill = lds + 2 * A_BUF;
+    AFrag first = load_frag(cur, 0);
     for (int c0 = 0; c0 < steps; c0 += D) {
 #pragma unroll
         for (int j = 0; j < D; ++j) {
             const int c = c0 + j;
-            load_a(c + 1);
+            const bool live = bs[j].valid;
+#pragma unroll
+            for (int f = 0; f < NT; ++f) asm volatile("" : "+v"(bs[j].q[f]), "+v"(bs[j].s[f]));
+            // Two fragment buffers used alternately besides `first` (compile-time parity, so no register
+            // copies); the LDS reads of fragment i+1 are issued before the MFMAs of fragment i and fenced
+            // there.  Reads ahead are unconditional (they stay inside the staged tile); the matrix work stops at
+            // the tile's last fragment.  Row fragments are dealt round-robin to the WR row groups, so a short
+            // tile still occupies all waves.
+            AFrag fr[2];
+            if (MTW > 1) fr[1] = load_frag(cur, 1);
             __builtin_amdgcn_sched_barrier(0);
-            compute(j, j & 1);
+            if (live && wrow < frags) mfma_frag(j, first, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            if (MTW > 2) fr[0] = load_frag(cur, 2);
+            store_a(stage, fill);
+            load_a(stage, c + 3);
+            first = load_frag(nxt, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (live) {
+                // Unrolled by template expansion (a pragma gives up on ten fragments with an exit test each, and
+                // the accumulators, then indexed at run time, land in scratch memory).
+                static_for_from1<MTW>([&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    if (i * WR + wrow < frags) {  // wave-uniform: the tile has rows there
+                        if (i >= 2 && i + 1 < MTW) fr[(i + 1) & 1] = load_frag(cur, i + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mfma_frag(j, fr[i & 1], i);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);
             load_b(j, c + D);  // refill the set just consumed
-            store_a((j + 1) & 1);
-            __syncthreads();
+            unsigned char *t = cur;
+            cur = nxt;
+            nxt = fill;
+            fill = t;
         }
     }
 
@@ -460,7 +512,9 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_kernel(MoeGemmArgs g) {
                 for (int p = 0; p < NT / 2; ++p)
                     if (col[2 * p] < g.N) {
                         const float gate = acc[i][2 * p][v], up = acc[i][2 * p + 1][v];
-                        const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                        // Hardware exp2 and reciprocal (1 ulp each): the result is rounded to bf16 right away,
+                        // and the library forms cost more than the tile's matrix work is worth.
+                        const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
                         static_cast<__bf16 *>(g.out)[orow + col[2 * p]] = static_cast<__bf16>(act);
                     }
             } else {
@@ -606,7 +660,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
             for (int p = 0; p < NT / 2; ++p)
                 if (col[2 * p] < g.N) {
                     const float gate = acc[2 * p][v], up = acc[2 * p + 1][v];
-                    const float act = up * (gate * (1.0f / (1.0f + expf(-gate))));
+                    const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
                     static_cast<__bf16 *>(g.out)[orow + col[2 * p]] = static_cast<__bf16>(act);
                 }
         } else {
@@ -688,7 +742,7 @@ static MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, int64_t E
 template <int MT, int NT, bool GATED, int WR = 1, int D = 4>
 static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
     constexpr int BM = 16 * MT;
-    const size_t lds_bytes = 2 * (2 * static_cast<size_t>(BM) * kARow + BM * 4);
+    const size_t lds_bytes = 3 * (2 * static_cast<size_t>(BM) * kARow + BM * 4);
     auto kern = mx_moe_gemm_kernel<MT, NT, GATED, WR, D>;
     if (lds_bytes > 64 * 1024)
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -766,7 +820,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
 
     // Row tile: as many routed rows per expert as there are on average, 16..128.
     const int avg = (R + E - 1) / E;
-    const int mt = avg > 64 ? 8 : (avg > 32 ? 4 : (avg > 16 ? 2 : 1));
+    const int mt = avg > 96 ? 10 : avg > 64 ? 8 : (avg > 32 ? 4 : (avg > 16 ? 2 : 1));
     const int BM = 16 * mt;
     const int max_tiles = R / BM + E;
     // A handful of routed rows in total (batch-1 decode and the like): stage each tile's
@@ -804,7 +858,8 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
             break;
         case 2: st = launch_moe_gemm<2, 2, true>(a1, cb1, max_tiles, s); break;
         case 4: st = launch_moe_gemm<4, 4, true>(a1, cb1w, max_tiles, s); break;
-        default: st = launch_moe_gemm<8, 4, true, 2, 4>(a1, cb1w, max_tiles, s); break;
+        case 8: st = launch_moe_gemm<8, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
+        default: st = launch_moe_gemm<10, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
     {
@@ -829,7 +884,8 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         switch (mt) {
             case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
             case 4: st = launch_moe_gemm<4, 4, false>(a2, cb2w, max_tiles, s); break;
-            default: st = launch_moe_gemm<8, 4, false, 2, 4>(a2, cb2w, max_tiles, s); break;
+            case 8: st = launch_moe_gemm<8, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
+            default: st = launch_moe_gemm<10, 3, false, 2, 2>(a2, (H + 191) / 192, max_tiles, s); break;
         }
     }
     if (st) return st;
