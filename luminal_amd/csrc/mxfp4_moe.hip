@@ -39,6 +39,9 @@ constexpr int kARow = 160;       // LDS bytes per activation row of a chunk: 128
                                  // lane (r, g) at r * pitch + 16 g, take twice as long: measured 8.0 against 4.3 cycles per read)
 
 static inline int64_t pad128(int64_t k) { return (k + 127) / 128 * 128; }
+// Row pitch of a whole quantised activation row in LDS (Kp a multiple of 128): the row plus padding that makes the
+// pitch 160 mod 256, the residue measured free of bank conflicts for the fragment reads.
+__host__ __device__ static inline int moe_small_pitch(int Kp) { return Kp + ((Kp & 255) ? 32 : 160); }
 
 // ---------------------------------------------------------------------------
 // Router: top-k of the logits (ties to the lower index), softmax over the k.
@@ -123,8 +126,7 @@ struct MoePlan {
     int *n_tiles;      // [1]
 };
 
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const int *__restrict__ sel, int R, int E, int BM,
-                                                        MoePlan p) {
+__device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int R, int E, int BM, const MoePlan &p) {
     __shared__ int cnt[1024], off[1025], cur[1024];
     for (int e = threadIdx.x; e < E; e += 1024) {
         cnt[e] = 0;
@@ -183,11 +185,10 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int *__restrict__ 
 // Planes have row stride Kp = K rounded up to 128, zero-filled past K; the scale
 // plane has row stride Kp/32, filled with 127 (2^0) past K.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
-                                                              uint8_t *__restrict__ lo, uint8_t *__restrict__ sc,
-                                                              int rows, int K, int Kp) {
+__device__ __forceinline__ void mx_quantize_act_item(size_t idx, const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
+                                                     uint8_t *__restrict__ lo, uint8_t *__restrict__ sc, int rows, int K,
+                                                     int Kp) {
     const int per_row = Kp / 8;
-    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     const size_t row = idx / per_row;
     const int c8 = static_cast<int>(idx - row * per_row);
     const bool live = row < static_cast<size_t>(rows);
@@ -230,6 +231,24 @@ __global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__re
     *reinterpret_cast<uint2 *>(hi + row * Kp + k) = make_uint2(ph[0], ph[1]);
     *reinterpret_cast<uint2 *>(lo + row * Kp + k) = make_uint2(pl[0], pl[1]);
     if ((c8 & 3) == 0) sc[row * (Kp / 32) + (c8 >> 2)] = static_cast<uint8_t>(k < K ? e : 127);
+}
+
+__global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
+                                                              uint8_t *__restrict__ lo, uint8_t *__restrict__ sc,
+                                                              int rows, int K, int Kp) {
+    mx_quantize_act_item(static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x, x, hi, lo, sc, rows, K, Kp);
+}
+
+// The two independent first steps of a layer pass in one launch: workgroup 0 makes the plan, the others
+// quantise the layer input (1024 items each).
+__global__ __launch_bounds__(1024) void moe_prepare_kernel(const int *__restrict__ sel, int R, int E, int BM, MoePlan p,
+                                                           const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
+                                                           uint8_t *__restrict__ lo, uint8_t *__restrict__ sc, int rows,
+                                                           int K, int Kp) {
+    if (blockIdx.x == 0)
+        moe_plan_block(sel, R, E, BM, p);
+    else
+        mx_quantize_act_item(static_cast<size_t>(blockIdx.x - 1) * 1024 + threadIdx.x, x, hi, lo, sc, rows, K, Kp);
 }
 
 // ---------------------------------------------------------------------------
@@ -530,7 +549,7 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
 // The tile's whole quantised activation rows (all of K) are staged in LDS once,
 // so the K loop is nothing but the weight stream — no activation loads, no
 // barriers — with D = 8 chunks of weights in flight per wave.  Needs
-// 2 * 16 * (Kp + 16) + 16 * Kp/32 bytes of LDS (K up to ~4.6k).
+// 2 * 16 * pitch + 16 * Kp/32 bytes of LDS (K up to ~4.6k).
 // ---------------------------------------------------------------------------
 template <int NT, bool GATED>
 __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
@@ -551,7 +570,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
     const int Kp = g.Kp;
     const int chunks = Kp / kChunk;
     const int steps = (chunks + D - 1) / D * D;
-    const int a_row = Kp + 16;             // LDS bytes per activation row (padded against bank conflicts)
+    const int a_row = moe_small_pitch(Kp);  // LDS bytes per activation row
     const int a_plane = 16 * a_row;
     const int sc_row = Kp / 32;            // scale bytes per row
     unsigned char *lds_sc = lds + 2 * a_plane;
@@ -753,7 +772,7 @@ static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max
     return LHIP_OK;
 }
 
-static inline size_t moe_small_lds_bytes(int Kp) { return 2 * 16 * static_cast<size_t>(Kp + 16) + 16 * (Kp / 32); }
+static inline size_t moe_small_lds_bytes(int Kp) { return 2 * 16 * static_cast<size_t>(moe_small_pitch(Kp)) + 16 * (Kp / 32); }
 
 template <int NT, bool GATED>
 static lhip_status launch_moe_gemm_small(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
@@ -828,12 +847,10 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     // that staging costs more than it saves (measured at T = 64: 168 us against 108 us).
     const bool decode_sized = R <= 4 * E / 2;
 
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel_dev, R, E, BM, w.plan);
-    LHIP_CHECK_LAUNCH();
     {
-        const size_t threads = static_cast<size_t>(T) * (Hp / 8);
-        hipLaunchKernelGGL(mx_quantize_act_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s,
-                           static_cast<const __bf16 *>(x_dev), w.x_hi, w.x_lo, w.x_sc, T, H, Hp);
+        const size_t items = static_cast<size_t>(T) * (Hp / 8);
+        hipLaunchKernelGGL(moe_prepare_kernel, dim3(static_cast<unsigned>(1 + (items + 1023) / 1024)), dim3(1024), 0, s,
+                           sel_dev, R, E, BM, w.plan, static_cast<const __bf16 *>(x_dev), w.x_hi, w.x_lo, w.x_sc, T, H, Hp);
         LHIP_CHECK_LAUNCH();
     }
     auto *gu = static_cast<const uint8_t *>(w_gate_up_planar);
