@@ -31,7 +31,11 @@ constexpr int kPfTileK = 32;  // keys per tile
 constexpr int kPfTileQ = 32;  // queries per workgroup
 
 template <int G, int HD, typename OutT>
-__global__ __launch_bounds__(64 * G) void attention_prefill_kernel(const float *__restrict__ qkv,
+// Register budget: with the default (as many waves per SIMD as the LDS allows) the compiler spills the prefetched
+// tile to scratch right after requesting it, i.e. waits for the loads it was meant to overlap.  One wave per SIMD
+// at head_dim 128 (Q 64 + O 64 + staging 32 registers and the sweep's temporaries), two otherwise.
+__global__ __launch_bounds__(64 * G) __attribute__((amdgpu_waves_per_eu(1, (HD == 128 && G <= 4) ? 1 : 2)))
+void attention_prefill_kernel(const float *__restrict__ qkv,
                                                                   const float *__restrict__ k_cache,
                                                                   const float *__restrict__ v_cache,
                                                                   OutT *__restrict__ out,
@@ -78,25 +82,27 @@ __global__ __launch_bounds__(64 * G) void attention_prefill_kernel(const float *
     const float4 *kc4 = reinterpret_cast<const float4 *>(k_cache) + static_cast<size_t>(kvh) * max_seq * (HD / 4);
     const float4 *vc4 = reinterpret_cast<const float4 *>(v_cache) + static_cast<size_t>(kvh) * max_seq * (HD / 4);
     constexpr int NST = PREFETCH ? LD : 1;
+    constexpr bool EXACT = TILE_F4 % THREADS == 0;  // every thread has a piece in every round: no test, so the
+                                                    // staging registers are plain registers, not a private array
     float4 kst[NST], vst[NST];
-    auto load_tile = [&](int t) {
+    auto load_tile = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NST; ++i) {
             const int f = tid + i * THREADS;  // float4 index inside the tile: row = f / (HD/4)
             const int row = f / (HD / 4), col = f - row * (HD / 4);
             const int key = min(t * kPfTileK + row, n_keys - 1);  // rows past the end repeat the last key (masked)
-            if (f < TILE_F4) {
+            if (EXACT || f < TILE_F4) {
                 kst[i] = kc4[static_cast<size_t>(key) * (HD / 4) + col];
                 vst[i] = vc4[static_cast<size_t>(key) * (HD / 4) + col];
             }
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NST; ++i) {
             const int f = tid + i * THREADS;
             const int row = f / (HD / 4), col = f - row * (HD / 4);
-            if (f < TILE_F4) {
+            if (EXACT || f < TILE_F4) {
                 *reinterpret_cast<float4 *>(&k_s[row * KP + col * 4]) = kst[i];
                 *reinterpret_cast<float4 *>(&v_s[row * HD + col * 4]) = vst[i];
             }
