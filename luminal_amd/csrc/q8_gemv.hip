@@ -525,7 +525,8 @@ static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, 
     if (rows_per_wave == R && k_unroll == S) {                                                                   \
         if (waves_per_block == 4) return launch_pipe<R, S, 4>(qs, ds, x, y, m, n, k, blocks_per_cu, s);          \
         if (waves_per_block == 8) return launch_pipe<R, S, 8>(qs, ds, x, y, m, n, k, blocks_per_cu, s);          \
-        if (waves_per_block == 16 && R * S <= 8) return launch_pipe<R, S, 16>(qs, ds, x, y, m, n, k, blocks_per_cu, s); \
+        if constexpr (R * S <= 8)                                                                                \
+            if (waves_per_block == 16) return launch_pipe<R, S, 16>(qs, ds, x, y, m, n, k, blocks_per_cu, s);    \
         return LHIP_ERR_UNSUPPORTED;                                                                             \
     }
     LHIP_CASE(1, 1) LHIP_CASE(1, 2) LHIP_CASE(1, 4)
