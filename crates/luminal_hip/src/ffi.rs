@@ -19,6 +19,9 @@ extern "C" {
     pub fn lhip_q8_0_repack(raw: *const c_void, planar: *mut c_void, n: i64, k: i64, s: Stream) -> Status;
     pub fn lhip_q8_0_matmul_f32(w: *const c_void, x: *const f32, y: *mut f32, m: i64, n: i64, k: i64, s: Stream) -> Status;
     pub fn lhip_q8_0_gather_f32(w: *const c_void, idx: *const f32, out: *mut f32, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;
+    // T = f16: x / y / out are IEEE binary16 buffers, sums stay f32
+    pub fn lhip_q8_0_matmul_f16(w: *const c_void, x: *const c_void, y: *mut c_void, m: i64, n: i64, k: i64, s: Stream) -> Status;
+    pub fn lhip_q8_0_gather_f16(w: *const c_void, idx: *const f32, out: *mut c_void, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;
 }
 
 #[track_caller]

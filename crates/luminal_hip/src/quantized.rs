@@ -6,6 +6,8 @@
 //! C entry point reads them from device memory.
 use std::{any::Any, ffi::c_void, marker::PhantomData, ptr::null_mut};
 
+use half::f16;
+
 use luminal::{
     op::{InputTensor, Operator},
     prelude::*,
@@ -110,6 +112,25 @@ impl Operator for QuantizedMatmul<f32> {
     }
 }
 
+/// T = f16 (the type luminal's llama example runs in on CUDA): the activation is a device buffer of f16 — there is
+/// no host f16 producer in this pipeline — and the output is f16; sums are f32 inside the kernel.
+impl Operator for QuantizedMatmul<f16> {
+    fn process(&mut self, inp: Vec<(InputTensor, ShapeTracker)>) -> Vec<Tensor> {
+        assert!(!inp[1].1.is_contiguous(), "Weight matrix must be column-major");
+        let (a, b) = (usize_dims(&inp[0].1), usize_dims(&inp[1].1));
+        let rows: usize = a[..a.len() - 1].iter().product::<usize>().max(1);
+        let (k, n) = (b[b.len() - 2], b[b.len() - 1]);
+        let out = HipData::alloc(rows * n * 2);
+        check(
+            unsafe {
+                ffi::lhip_q8_0_matmul_f16(device_ptr(&inp[1].0), device_ptr(&inp[0].0), out.ptr, rows as i64, n as i64, k as i64, null_mut())
+            },
+            "lhip_q8_0_matmul_f16",
+        );
+        vec![Tensor::new(out)]
+    }
+}
+
 /// Row gather from a Q8_0 embedding table; indices arrive as host f32 like in the other backends.
 #[derive(Clone, Debug)]
 pub struct QuantizedGather<T> {
@@ -129,6 +150,24 @@ impl Operator for QuantizedGather<f32> {
                                           vocab as i64, self.embed_dim as i64, null_mut())
             },
             "lhip_q8_0_gather_f32",
+        );
+        check(unsafe { ffi::lhip_stream_sync(null_mut()) }, "lhip_stream_sync"); // idx_dev is freed on return
+        vec![Tensor::new(out)]
+    }
+}
+
+impl Operator for QuantizedGather<f16> {
+    fn process(&mut self, inp: Vec<(InputTensor, ShapeTracker)>) -> Vec<Tensor> {
+        let idx = inp[0].0.borrowed().downcast_ref::<Vec<f32>>().expect("gather indices are host f32");
+        let vocab = inp[1].1.dims().into_iter().map(|d| d.to_usize().unwrap()).product::<usize>() / self.embed_dim;
+        let idx_dev = HipData::from_host(idx);
+        let out = HipData::alloc(idx.len() * self.embed_dim * 2);
+        check(
+            unsafe {
+                ffi::lhip_q8_0_gather_f16(device_ptr(&inp[1].0), idx_dev.ptr as _, out.ptr, idx.len() as i64,
+                                          vocab as i64, self.embed_dim as i64, null_mut())
+            },
+            "lhip_q8_0_gather_f16",
         );
         check(unsafe { ffi::lhip_stream_sync(null_mut()) }, "lhip_stream_sync"); // idx_dev is freed on return
         vec![Tensor::new(out)]
@@ -155,7 +194,21 @@ impl<T> HipQuantizedCompiler<T> {
     }
 }
 
-impl Compiler for HipQuantizedCompiler<f32> {
+/// The activation types the pass can emit operators for.
+pub trait HipActivation: 'static + Sized {
+    fn matmul() -> Box<dyn Operator>;
+    fn gather(embed_dim: usize) -> Box<dyn Operator>;
+}
+impl HipActivation for f32 {
+    fn matmul() -> Box<dyn Operator> { Box::new(QuantizedMatmul::<f32>::default()) }
+    fn gather(embed_dim: usize) -> Box<dyn Operator> { Box::new(QuantizedGather::<f32> { embed_dim, _t: PhantomData }) }
+}
+impl HipActivation for f16 {
+    fn matmul() -> Box<dyn Operator> { Box::new(QuantizedMatmul::<f16>::default()) }
+    fn gather(embed_dim: usize) -> Box<dyn Operator> { Box::new(QuantizedGather::<f16> { embed_dim, _t: PhantomData }) }
+}
+
+impl<T: HipActivation> Compiler for HipQuantizedCompiler<T> {
     type Output = ();
     fn compile<To: ToIdsMut>(&self, graph: &mut Graph, _ids: To) {
         check(unsafe { ffi::lhip_init(0) }, "lhip_init");
@@ -168,9 +221,9 @@ impl Compiler for HipQuantizedCompiler<f32> {
                 assert_eq!(slot, 1, "Quantized weight {consumer:?} is the wrong input!");
                 let op = graph.node_weight_mut(consumer).unwrap();
                 if let Some(g) = op.as_any().downcast_ref::<luminal_cpu::Gather>() {
-                    *op = Box::new(QuantizedGather::<f32> { embed_dim: g.embed_dim, _t: PhantomData });
+                    *op = T::gather(g.embed_dim);
                 } else if op.as_any().is::<luminal_cpu::MatMul2D>() || op.as_any().is::<luminal_cpu::BatchedMatMul2D>() {
-                    *op = Box::new(QuantizedMatmul::<f32>::default());
+                    *op = T::matmul();
                 } else {
                     panic!("Quantized weight {consumer:?} is an input to a node that isn't a matmul or gather ({op:?})");
                 }

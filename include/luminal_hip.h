@@ -159,6 +159,16 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
 lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, float *out_dev, int64_t n_idx,
                                  int64_t n, int64_t k, void *stream);
 
+/* The reference's second activation type, T = f16 (QuantizedMatmul<f16> / QuantizedGather<f16>,
+ * crates/luminal_cuda/src/quantized.rs:42-109,170-233; its llama example runs in f16): x and y are IEEE binary16
+ * (x 8-byte aligned), every product and sum is f32 as in the kernel there (:72,94-96) and the result is rounded to
+ * f16 once at the store (:106); the gather rounds q*d to f16 once, which equals the product taken in half
+ * precision.  Same shapes, launch choice and errors as the f32 forms. */
+lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, void *y_f16_dev, int64_t m, int64_t n,
+                                 int64_t k, void *stream);
+lhip_status lhip_q8_0_gather_f16(const void *planar_dev, const float *idx_dev, void *out_f16_dev, int64_t n_idx,
+                                 int64_t n, int64_t k, void *stream);
+
 /* ---- MXFP4 weights and the mixture-of-experts layer -------------------------
  * No counterpart in the reference (it has no MXFP4 and no MoE op); built to its
  * conventions: exact dequantisation, then f32-accumulated matmul

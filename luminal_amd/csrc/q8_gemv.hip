@@ -67,12 +67,24 @@ __device__ __forceinline__ float dot16(const u32x4 &q, const float4 (&x)[4]) {
     return s;
 }
 
+// Activation / output element type T (the reference's QuantizedMatmul<T>): float, or __half with every product and
+// sum still in f32 (crates/luminal_cuda/src/quantized.rs:72,94-96 accumulate in float and store (T)sum, :106).
+// Four consecutive activations as f32.
+__device__ __forceinline__ float4 load_x4(const float *x, int i4) { return reinterpret_cast<const float4 *>(x)[i4]; }
+__device__ __forceinline__ float4 load_x4(const __half *x, int i4) {
+    const uint2 raw = reinterpret_cast<const uint2 *>(x)[i4];
+    const __half2 lo = *reinterpret_cast<const __half2 *>(&raw.x), hi = *reinterpret_cast<const __half2 *>(&raw.y);
+    return make_float4(__low2float(lo), __high2float(lo), __low2float(hi), __high2float(hi));
+}
+__device__ __forceinline__ void store_y(float *y, int i, float v) { y[i] = v; }
+__device__ __forceinline__ void store_y(__half *y, int i, float v) { y[i] = __float2half(v); }  // round to nearest even
+
 // R rows per wave, W waves per workgroup, U slices of 1024 quants per step.
 // grid.x covers ceil(n / (R*W)) row tiles, grid.y the rows of x (m).
-template <int R, int W, int U>
+template <int R, int W, int U, typename T = float>
 __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__restrict__ qs,
                                                               const __half *__restrict__ ds,
-                                                              const float *__restrict__ x, float *__restrict__ y,
+                                                              const T *__restrict__ x, T *__restrict__ y,
                                                               int n, int k) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -111,9 +123,8 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__res
                 q[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow[r] + ko));
                 d[u][r] = drow[r][ko >> 5];
             }
-            const float4 *xp = reinterpret_cast<const float4 *>(x + ko);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) xv[u][j] = xp[j];
+            for (int j = 0; j < 4; ++j) xv[u][j] = load_x4(x, (ko >> 2) + j);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -123,9 +134,8 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__res
     // Tail: remaining slices one at a time (lanes past K idle).
     for (; kofs < k; kofs += 1024) {
         float4 xv[4];
-        const float4 *xp = reinterpret_cast<const float4 *>(x + kofs);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xv[j] = xp[j];
+        for (int j = 0; j < 4; ++j) xv[j] = load_x4(x, (kofs >> 2) + j);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const u32x4 q = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow[r] + kofs));
@@ -139,7 +149,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_kernel(const int8_t *__res
         const float s = wave_sum(acc[r]);
         if (lane == r) out = s;
     }
-    if (lane < R && row0 + lane < n) y[row0 + lane] = out;
+    if (lane < R && row0 + lane < n) store_y(y, row0 + lane, out);
 }
 
 // ---------------------------------------------------------------------------
@@ -213,10 +223,10 @@ __device__ __forceinline__ void compute_step(StepBuf<R, S> &b, const float4 *xs4
     }
 }
 
-template <int R, int S, int W>
+template <int R, int S, int W, typename XT = float>
 __global__ __launch_bounds__(W * 64) void q8_gemv_f32_pipe_kernel(const int8_t *__restrict__ qs,
                                                                 const unsigned short *__restrict__ ds,
-                                                                const float *__restrict__ x, float *__restrict__ y,
+                                                                const XT *__restrict__ x, XT *__restrict__ y,
                                                                 int n, int k) {
     extern __shared__ float4 xs4[];
     const unsigned lane = threadIdx.x & 63u;
@@ -237,13 +247,12 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_pipe_kernel(const int8_t *
     load_step(a, qs, ds, wave_global * R, n, k, 0, lane, T > 0);
 
     {
-        const float4 *x4 = reinterpret_cast<const float4 *>(x);
         const int k4 = k >> 2;
 #pragma unroll 4
         for (int i = threadIdx.x; i < k4; i += W * 64) {
             // destination index i = slice*256 + j*64 + l  <-  source slice*256 + l*4 + j
             const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
-            xs4[i] = x4[src];
+            xs4[i] = load_x4(x, src);
         }
     }
     __syncthreads();
@@ -272,7 +281,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_f32_pipe_kernel(const int8_t *
             acc[r] = 0.f;
         }
         const int row0 = gg * R;
-        if (lane < static_cast<unsigned>(R) && row0 + static_cast<int>(lane) < n) y[row0 + lane] = out;
+        if (lane < static_cast<unsigned>(R) && row0 + static_cast<int>(lane) < n) store_y(y, row0 + lane, out);
     };
 
     while (true) {
@@ -479,25 +488,25 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
 constexpr int kNumCUs = 256;
 constexpr int kMaxLdsK = 16384;  // 64 KiB of staged activations
 
-template <int R, int W, int U>
-static lhip_status launch_oneshot(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
+template <int R, int W, int U, typename T>
+static lhip_status launch_oneshot(const int8_t *qs, const __half *ds, const T *x, T *y, int m, int n, int k,
                                   hipStream_t s) {
     const unsigned tiles = static_cast<unsigned>((n + R * W - 1) / (R * W));
-    hipLaunchKernelGGL((q8_gemv_f32_kernel<R, W, U>), dim3(tiles, static_cast<unsigned>(m)), dim3(W * 64), 0, s, qs,
+    hipLaunchKernelGGL((q8_gemv_f32_kernel<R, W, U, T>), dim3(tiles, static_cast<unsigned>(m)), dim3(W * 64), 0, s, qs,
                        ds, x, y, n, k);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
-template <int R, int S, int W>
-static lhip_status launch_pipe(const int8_t *qs, const __half *ds, const float *x, float *y, int m, int n, int k,
+template <int R, int S, int W, typename T>
+static lhip_status launch_pipe(const int8_t *qs, const __half *ds, const T *x, T *y, int m, int n, int k,
                                int blocks_per_cu, hipStream_t s) {
     if (k % (S * 1024) != 0 || k > kMaxLdsK) return LHIP_ERR_UNSUPPORTED;
     const int n_groups = (n + R - 1) / R;
     int grid = (n_groups + W - 1) / W;
     const int cap = kNumCUs * blocks_per_cu;
     if (grid > cap) grid = cap;
-    hipLaunchKernelGGL((q8_gemv_f32_pipe_kernel<R, S, W>), dim3(static_cast<unsigned>(grid), static_cast<unsigned>(m)),
+    hipLaunchKernelGGL((q8_gemv_f32_pipe_kernel<R, S, W, T>), dim3(static_cast<unsigned>(grid), static_cast<unsigned>(m)),
                        dim3(W * 64), static_cast<size_t>(k) * sizeof(float), s, qs,
                        reinterpret_cast<const unsigned short *>(ds), x, y, n, k);
     LHIP_CHECK_LAUNCH();
@@ -534,6 +543,22 @@ static lhip_status dispatch(int rows_per_wave, int k_unroll, int blocks_per_cu, 
     LHIP_CASE(4, 1) LHIP_CASE(4, 2) LHIP_CASE(4, 4)
 #undef LHIP_CASE
     return LHIP_ERR_UNSUPPORTED;
+}
+
+// The f16 activation type runs the launch shapes choose() picks, nothing else.
+static lhip_status dispatch_f16(int rows_per_wave, int k_unroll, int blocks_per_cu, int waves_per_block, const int8_t *qs,
+                                const __half *ds, const __half *x, __half *y, int m, int n, int k, hipStream_t s) {
+    if (blocks_per_cu == 0) {
+        if (rows_per_wave == 1) return launch_oneshot<1, 4, 1>(qs, ds, x, y, m, n, k, s);
+        if (rows_per_wave == 2) return launch_oneshot<2, 4, 1>(qs, ds, x, y, m, n, k, s);
+        return launch_oneshot<4, 4, 1>(qs, ds, x, y, m, n, k, s);
+    }
+    if (rows_per_wave == 2) return launch_pipe<2, 4, 4>(qs, ds, x, y, m, n, k, blocks_per_cu, s);
+    if (waves_per_block == 16)
+        return k_unroll == 2 ? launch_pipe<1, 2, 16>(qs, ds, x, y, m, n, k, blocks_per_cu, s)
+                             : launch_pipe<1, 1, 16>(qs, ds, x, y, m, n, k, blocks_per_cu, s);
+    return k_unroll == 2 ? launch_pipe<1, 2, 4>(qs, ds, x, y, m, n, k, blocks_per_cu, s)
+                         : launch_pipe<1, 1, 4>(qs, ds, x, y, m, n, k, blocks_per_cu, s);
 }
 
 // Default launch shape per problem size.
@@ -661,6 +686,22 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
     int r, u, b, w;
     choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
     return lhip_q8_0_matmul_f32_cfg(planar_dev, x_dev, y_dev, m, n, k, r, u, b, w, stream);
+}
+
+lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, void *y_f16_dev, int64_t m, int64_t n,
+                                 int64_t k, void *stream) {
+    if (!planar_dev || !x_f16_dev || !y_f16_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (m <= 0 || m > 65535) return LHIP_ERR_INVALID_SHAPE;
+    // Rows of x start at multiples of K halves; K % 32 == 0 keeps them 8-byte aligned.
+    if (!aligned(planar_dev, 256) || !aligned(x_f16_dev, 8) || !aligned(y_f16_dev, 2)) return LHIP_ERR_MISALIGNED;
+    int r, u, b, w;
+    choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    return dispatch_f16(r, u, b, w, reinterpret_cast<const int8_t *>(base),
+                        reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)),
+                        static_cast<const __half *>(x_f16_dev), static_cast<__half *>(y_f16_dev), static_cast<int>(m),
+                        static_cast<int>(n), static_cast<int>(k), as_stream(stream));
 }
 
 lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float *const *y_dev, const int64_t *n,

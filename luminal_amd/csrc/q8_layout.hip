@@ -60,24 +60,35 @@ __global__ __launch_bounds__(kThreads) void q8_dequant_kernel(const uint32_t *__
     for (; i < n_quads; i += stride) out[i] = dequant4(qs[i], __half2float(ds[i >> 3]));
 }
 
+// Four dequantised weights in the output type: f32 as they are (the product is exact), or rounded once to f16
+// (what `(half)q * (half)d` gives: crates/luminal_cuda/src/quantized.rs:196-199 multiplies in T).
+struct Half4 {
+    __half2 lo, hi;
+};
+__device__ __forceinline__ void store_quad(float4 *o, int j, float4 v) { o[j] = v; }
+__device__ __forceinline__ void store_quad(Half4 *o, int j, float4 v) {
+    o[j] = Half4{__floats2half2_rn(v.x, v.y), __floats2half2_rn(v.z, v.w)};
+}
+
 // grid.x = index row, threads stride over the K/4 quads of that row.
+template <typename Quad>
 __global__ __launch_bounds__(kThreads) void q8_gather_kernel(const uint32_t *__restrict__ qs,
                                                               const __half *__restrict__ ds,
                                                               const float *__restrict__ idx,
-                                                              float4 *__restrict__ out, int n, int k) {
+                                                              Quad *__restrict__ out, int n, int k) {
     const int t = blockIdx.x;
     const float fi = idx[t];
     // `as usize` in the reference's CPU gather truncates toward zero.
     const long row = (fi >= 0.0f && fi < 2147483648.0f) ? static_cast<long>(fi) : -1;
     const int quads = k >> 2;
-    float4 *o = out + static_cast<size_t>(t) * quads;
+    Quad *o = out + static_cast<size_t>(t) * quads;
     if (row < 0 || row >= n) {
-        for (int j = threadIdx.x; j < quads; j += kThreads) o[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int j = threadIdx.x; j < quads; j += kThreads) store_quad(o, j, make_float4(0.f, 0.f, 0.f, 0.f));
         return;
     }
     const uint32_t *q = qs + static_cast<size_t>(row) * quads;
     const __half *d = ds + static_cast<size_t>(row) * (k >> 5);
-    for (int j = threadIdx.x; j < quads; j += kThreads) o[j] = dequant4(q[j], __half2float(d[j >> 3]));
+    for (int j = threadIdx.x; j < quads; j += kThreads) store_quad(o, j, dequant4(q[j], __half2float(d[j >> 3])));
 }
 
 static inline unsigned grid_for(size_t items) {
@@ -157,10 +168,25 @@ lhip_status lhip_q8_0_gather_f32(const void *planar_dev, const float *idx_dev, f
     if (n_idx <= 0 || n_idx > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     if (!aligned(planar_dev, 256) || !aligned(out_dev, 16) || !aligned(idx_dev, 4)) return LHIP_ERR_MISALIGNED;
     auto *base = static_cast<const uint8_t *>(planar_dev);
-    hipLaunchKernelGGL(q8_gather_kernel, dim3(static_cast<unsigned>(n_idx)), dim3(kThreads), 0, as_stream(stream),
+    hipLaunchKernelGGL(q8_gather_kernel<float4>, dim3(static_cast<unsigned>(n_idx)), dim3(kThreads), 0, as_stream(stream),
                        reinterpret_cast<const uint32_t *>(base),
                        reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), idx_dev,
                        reinterpret_cast<float4 *>(out_dev), static_cast<int>(n), static_cast<int>(k));
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_q8_0_gather_f16(const void *planar_dev, const float *idx_dev, void *out_f16_dev, int64_t n_idx,
+                                 int64_t n, int64_t k, void *stream) {
+    if (!planar_dev || !idx_dev || !out_f16_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (n_idx <= 0 || n_idx > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(planar_dev, 256) || !aligned(out_f16_dev, 8) || !aligned(idx_dev, 4)) return LHIP_ERR_MISALIGNED;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    hipLaunchKernelGGL(q8_gather_kernel<Half4>, dim3(static_cast<unsigned>(n_idx)), dim3(kThreads), 0, as_stream(stream),
+                       reinterpret_cast<const uint32_t *>(base),
+                       reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), idx_dev,
+                       reinterpret_cast<Half4 *>(out_f16_dev), static_cast<int>(n), static_cast<int>(k));
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }

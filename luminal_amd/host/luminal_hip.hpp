@@ -4,7 +4,7 @@
 // Names, argument meaning and failure behaviour follow the reference:
 //   HipData                 <- CudaData<T>                         crates/luminal_cuda/src/lib.rs:83-100
 //   Operator::process       <- trait Operator                      src/op.rs:82-90
-//   QuantizedMatmul         <- QuantizedMatmul<T>                  crates/luminal_cuda/src/quantized.rs:111-168
+//   QuantizedMatmul         <- QuantizedMatmul<T>, T = f32 | f16   crates/luminal_cuda/src/quantized.rs:111-168
 //   QuantizedGather         <- QuantizedGather<T>                  crates/luminal_cuda/src/quantized.rs:170-233
 //   HipQuantizedCompiler    <- CudaQuantizedCompiler<T>            crates/luminal_cuda/src/quantized.rs:235-272
 //   downstream              <- luminal::module::downstream         src/module.rs:84-113
@@ -58,6 +58,11 @@ class HipData {
         check(lhip_memcpy_d2h(v.data(), ptr_, bytes_, nullptr), "lhip_memcpy_d2h");
         return v;
     }
+    std::vector<uint16_t> to_host_f16_codes() const {
+        std::vector<uint16_t> v(bytes_ / sizeof(uint16_t));
+        check(lhip_memcpy_d2h(v.data(), ptr_, bytes_, nullptr), "lhip_memcpy_d2h");
+        return v;
+    }
     // Raw GGUF Q8_0 blocks of an (n, k) weight -> planar device buffer (what the HIP loader keeps per tensor).
     static std::shared_ptr<HipData> q8_0_from_raw(const std::vector<uint8_t> &raw_blocks, int64_t n, int64_t k) {
         if (raw_blocks.size() != lhip_q8_0_raw_nbytes(n, k) || raw_blocks.empty())
@@ -108,10 +113,17 @@ inline const HipData &device_operand(const Tensor &t, const char *what) {
     return **p;
 }
 
-// (batch.., m, K) f32 x Q8_0 (N, K) -> (batch.., m, N) f32.  inp[0] = activations (device f32, or host f32 which is
-// uploaded for the call), inp[1] = weight with dims [.., K, N], necessarily a permuted (non-contiguous) view.
+// The reference's operators are generic over the activation type T (f32 or f16); here it is a run-time tag.
+enum class DType { F32, F16 };
+inline size_t dtype_size(DType t) { return t == DType::F32 ? 4 : 2; }
+
+// (batch.., m, K) T x Q8_0 (N, K) -> (batch.., m, N) T.  inp[0] = activations (a device buffer of T, or, for f32,
+// host f32 which is uploaded for the call), inp[1] = weight with dims [.., K, N], necessarily a permuted
+// (non-contiguous) view.
 class QuantizedMatmul : public Operator {
   public:
+    explicit QuantizedMatmul(DType dtype = DType::F32) : dtype(dtype) {}
+    DType dtype;
     std::vector<Tensor> process(const std::vector<Input> &inp) override {
         const ShapeTracker &a = inp.at(0).second, &b = inp.at(1).second;
         if (b.contiguous) throw Panic("Weight matrix must be column-major");
@@ -122,15 +134,20 @@ class QuantizedMatmul : public Operator {
         std::shared_ptr<HipData> staged;
         const void *x;
         if (auto host = std::get_if<std::shared_ptr<std::vector<float>>>(&inp[0].first->data)) {
+            if (dtype != DType::F32) throw Panic("QuantizedMatmul<f16>: host activations are f32");
             staged = HipData::from_host(**host);
             x = staged->ptr();
         } else {
             x = device_operand(*inp[0].first, "activation").ptr();
         }
-        auto out = std::make_shared<HipData>(static_cast<size_t>(rows * n) * sizeof(float));
-        check(lhip_q8_0_matmul_f32(device_operand(*inp[1].first, "weight").ptr(), static_cast<const float *>(x),
-                                   static_cast<float *>(out->ptr()), rows, n, k, nullptr),
-              "lhip_q8_0_matmul_f32");
+        auto out = std::make_shared<HipData>(static_cast<size_t>(rows * n) * dtype_size(dtype));
+        const void *w = device_operand(*inp[1].first, "weight").ptr();
+        if (dtype == DType::F32)
+            check(lhip_q8_0_matmul_f32(w, static_cast<const float *>(x), static_cast<float *>(out->ptr()), rows, n, k,
+                                       nullptr),
+                  "lhip_q8_0_matmul_f32");
+        else
+            check(lhip_q8_0_matmul_f16(w, x, out->ptr(), rows, n, k, nullptr), "lhip_q8_0_matmul_f16");
         check(lhip_stream_sync(nullptr), "lhip_stream_sync");  // a staged activation is released on return
         return {Tensor{out}};
     }
@@ -140,22 +157,27 @@ class QuantizedMatmul : public Operator {
 // Row gather from a Q8_0 embedding table; indices arrive as host f32, as in every luminal backend.
 class QuantizedGather : public Operator {
   public:
-    explicit QuantizedGather(int64_t embed_dim) : embed_dim(embed_dim) {}
+    explicit QuantizedGather(int64_t embed_dim, DType dtype = DType::F32) : embed_dim(embed_dim), dtype(dtype) {}
     std::vector<Tensor> process(const std::vector<Input> &inp) override {
         auto idx = std::get_if<std::shared_ptr<std::vector<float>>>(&inp.at(0).first->data);
         if (!idx) throw Panic("gather indices are host f32");
         const int64_t vocab = inp.at(1).second.n_elements() / embed_dim;
         auto idx_dev = HipData::from_host(**idx);
-        auto out = std::make_shared<HipData>((*idx)->size() * embed_dim * sizeof(float));
-        check(lhip_q8_0_gather_f32(device_operand(*inp[1].first, "table").ptr(), static_cast<const float *>(idx_dev->ptr()),
-                                   static_cast<float *>(out->ptr()), static_cast<int64_t>((*idx)->size()), vocab, embed_dim,
-                                   nullptr),
-              "lhip_q8_0_gather_f32");
+        auto out = std::make_shared<HipData>((*idx)->size() * embed_dim * dtype_size(dtype));
+        const void *table = device_operand(*inp[1].first, "table").ptr();
+        const auto *ids = static_cast<const float *>(idx_dev->ptr());
+        const auto count = static_cast<int64_t>((*idx)->size());
+        if (dtype == DType::F32)
+            check(lhip_q8_0_gather_f32(table, ids, static_cast<float *>(out->ptr()), count, vocab, embed_dim, nullptr),
+                  "lhip_q8_0_gather_f32");
+        else
+            check(lhip_q8_0_gather_f16(table, ids, out->ptr(), count, vocab, embed_dim, nullptr), "lhip_q8_0_gather_f16");
         check(lhip_stream_sync(nullptr), "lhip_stream_sync");
         return {Tensor{out}};
     }
     std::string name() const override { return "QuantizedGather"; }
     int64_t embed_dim;
+    DType dtype;
 };
 
 // ---- the operators a graph holds before the pass runs (markers; a CPU backend would execute them) -------------
@@ -251,7 +273,8 @@ inline std::vector<NodeIndex> downstream(const std::vector<NodeIndex> &nodes, co
 // Rewrites the consumers of the given Q8_0 weight nodes into the HIP quantized operators.
 class HipQuantizedCompiler {
   public:
-    explicit HipQuantizedCompiler(std::vector<NodeIndex> weights) : weights_(std::move(weights)) {}
+    explicit HipQuantizedCompiler(std::vector<NodeIndex> weights, DType dtype = DType::F32)
+        : weights_(std::move(weights)), dtype_(dtype) {}
     // init_device = false leaves device selection to the caller (and lets the rewrite be exercised without a GPU).
     void compile(Graph &graph, bool init_device = true) const {
         if (init_device) check(lhip_init(0), "lhip_init");
@@ -261,9 +284,9 @@ class HipQuantizedCompiler {
                 if (e->input_order != 1) throw Panic("Quantized weight " + target + " is the wrong input!");
                 auto &op = graph.nodes[e->dst];
                 if (auto gather = dynamic_cast<Gather *>(op.get())) {
-                    op = std::make_unique<QuantizedGather>(gather->embed_dim);
+                    op = std::make_unique<QuantizedGather>(gather->embed_dim, dtype_);
                 } else if (dynamic_cast<MatMul2D *>(op.get())) {
-                    op = std::make_unique<QuantizedMatmul>();
+                    op = std::make_unique<QuantizedMatmul>(dtype_);
                 } else {
                     throw Panic("Quantized weight " + target + " is an input to a node that isn't a matmul or gather (" +
                                 op->name() + ")");
@@ -274,6 +297,7 @@ class HipQuantizedCompiler {
 
   private:
     std::vector<NodeIndex> weights_;
+    DType dtype_;
 };
 
 }  // namespace luminal_hip

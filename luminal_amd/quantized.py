@@ -72,8 +72,9 @@ class Q8Weight:
 
 
 class QuantizedMatmul:
-    """(.., M, K) x Q8_0 (N, K) -> (.., M, N), f32
-    (QuantizedMatmul<f32>::process, crates/luminal_cuda/src/quantized.rs:116-168)."""
+    """(.., M, K) x Q8_0 (N, K) -> (.., M, N) in the activation type T = f32 or f16, f32 accumulation either way
+    (QuantizedMatmul<T>::process, crates/luminal_cuda/src/quantized.rs:116-168).  The launch shape can be chosen
+    for f32 only."""
 
     def __init__(self, rows_per_wave: int | None = None, k_unroll: int | None = None, blocks_per_cu: int = 0,
                  waves_per_block: int = 4):
@@ -81,15 +82,21 @@ class QuantizedMatmul:
 
     def process(self, x: torch.Tensor, w: Q8Weight) -> torch.Tensor:
         lib = capi.load_library()
-        if x.dtype != torch.float32 or not x.is_cuda:
-            raise TypeError("QuantizedMatmul expects f32 activations on the GPU")
+        if x.dtype not in (torch.float32, torch.float16) or not x.is_cuda:
+            raise TypeError("QuantizedMatmul expects f32 or f16 activations on the GPU")
         if x.shape[-1] != w.k:
             raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "QuantizedMatmul",
                                  f"activation K {x.shape[-1]} != weight K {w.k}")
         x = x.contiguous()
         m = x.numel() // w.k
-        out = torch.empty(x.shape[:-1] + (w.n,), dtype=torch.float32, device=x.device)
+        out = torch.empty(x.shape[:-1] + (w.n,), dtype=x.dtype, device=x.device)
         with torch.cuda.device(x.device):
+            if x.dtype == torch.float16:
+                if self.cfg:
+                    raise TypeError("QuantizedMatmul: a launch shape can be chosen for f32 activations only")
+                st = lib.lhip_q8_0_matmul_f16(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, _stream())
+                capi.check(st, "lhip_q8_0_matmul_f16")
+                return out
             if self.cfg:
                 st = lib.lhip_q8_0_matmul_f32_cfg(_ptr(w.planar), _ptr(x), _ptr(out), m, w.n, w.k, self.cfg[0],
                                                   self.cfg[1], self.cfg[2], self.cfg[3], _stream())
@@ -129,11 +136,14 @@ class QuantizedMatmulBf16:
 
 
 class QuantizedGather:
-    """Row gather from a Q8_0 table; indices are f32 as in the reference
-    (QuantizedGather<f32>::process, crates/luminal_cuda/src/quantized.rs:202-233)."""
+    """Row gather from a Q8_0 table into T = f32 (default) or f16; indices are f32 as in the reference
+    (QuantizedGather<T>::process, crates/luminal_cuda/src/quantized.rs:202-233)."""
 
-    def __init__(self, embed_dim: int):
+    def __init__(self, embed_dim: int, dtype: torch.dtype = torch.float32):
+        if dtype not in (torch.float32, torch.float16):
+            raise TypeError("QuantizedGather gathers into f32 or f16")
         self.embed_dim = embed_dim
+        self.dtype = dtype
 
     def process(self, indexes: torch.Tensor, w: Q8Weight) -> torch.Tensor:
         lib = capi.load_library()
@@ -141,10 +151,11 @@ class QuantizedGather:
             raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "QuantizedGather",
                                  f"embed_dim {self.embed_dim} != weight K {w.k}")
         idx = indexes.to(device=w.planar.device, dtype=torch.float32).contiguous().reshape(-1)
-        out = torch.empty((idx.numel(), w.k), dtype=torch.float32, device=idx.device)
+        out = torch.empty((idx.numel(), w.k), dtype=self.dtype, device=idx.device)
+        gather = lib.lhip_q8_0_gather_f32 if self.dtype == torch.float32 else lib.lhip_q8_0_gather_f16
         with torch.cuda.device(idx.device):
-            st = lib.lhip_q8_0_gather_f32(_ptr(w.planar), _ptr(idx), _ptr(out), idx.numel(), w.n, w.k, _stream())
-        capi.check(st, "lhip_q8_0_gather_f32")
+            st = gather(_ptr(w.planar), _ptr(idx), _ptr(out), idx.numel(), w.n, w.k, _stream())
+        capi.check(st, "lhip_q8_0_gather")
         return out
 
 

@@ -212,6 +212,62 @@ static void test_quantized_matmul_and_graph_execution() {
     EXPECT(msg.find("lhip_q8_0_matmul_f32") != std::string::npos && msg.find("INVALID_SHAPE") != std::string::npos);
 }
 
+static void test_f16_graph() {
+    // The same two-node graph compiled for T = f16 (the type the reference's llama example runs in):
+    // gather -> f16 rows (exact rows rounded once), matmul -> f32 sums rounded once to f16.
+    std::mt19937 rng(3);
+    const int vocab = 50, dim = 64, n = 40, m = 5;
+    std::normal_distribution<float> gauss(0.f, 0.02f);
+    auto make = [&](int rows, int cols, std::vector<int8_t> &q, std::vector<float> &d) {
+        q.resize(static_cast<size_t>(rows) * cols);
+        d.resize(q.size() / 32);
+        for (auto &v : q) v = static_cast<int8_t>(static_cast<int>(rng() % 255) - 127);
+        for (auto &v : d) v = f16_value(f16_code(std::fabs(gauss(rng)) / 127.f + 1e-3f));
+        return q8_0_blocks(q, d);
+    };
+    std::vector<int8_t> eq, wq;
+    std::vector<float> ed, wd;
+    auto e_raw = make(vocab, dim, eq, ed), w_raw = make(n, dim, wq, wd);
+    std::vector<float> ids(m);
+    for (auto &v : ids) v = static_cast<float>(rng() % vocab);
+    Graph g;
+    auto tok = g.add(std::make_unique<Function>());
+    auto embed = g.add(std::make_unique<Function>());
+    auto w = g.add(std::make_unique<Function>());
+    auto gather = g.add(std::make_unique<Gather>(dim));
+    auto mm = g.add(std::make_unique<MatMul2D>());
+    g.connect(tok, gather, 0, {{m}, true});
+    g.connect(embed, gather, 1, {{vocab, dim}, true});
+    g.connect(gather, mm, 0, {{m, dim}, true});
+    g.connect(w, mm, 1, {{dim, n}, false});
+    HipQuantizedCompiler({embed, w}, DType::F16).compile(g);
+    EXPECT(dynamic_cast<QuantizedMatmul *>(g.nodes[mm].get())->dtype == DType::F16);
+    dynamic_cast<Function *>(g.nodes[tok].get())->value = Tensor{std::make_shared<std::vector<float>>(ids)};
+    dynamic_cast<Function *>(g.nodes[embed].get())->value = Tensor{HipData::q8_0_from_raw(e_raw, vocab, dim)};
+    dynamic_cast<Function *>(g.nodes[w].get())->value = Tensor{HipData::q8_0_from_raw(w_raw, n, dim)};
+    g.execute();
+    auto rows = device_operand(g.results.at(gather), "gather").to_host_f16_codes();
+    bool exact = rows.size() == static_cast<size_t>(m) * dim;
+    for (int t = 0; exact && t < m; ++t)
+        for (int c = 0; c < dim; ++c) {
+            const size_t i = static_cast<size_t>(ids[t]) * dim + c;
+            exact &= rows[static_cast<size_t>(t) * dim + c] == f16_code(static_cast<float>(eq[i]) * ed[i / 32]);
+        }
+    EXPECT(exact);
+    auto out = device_operand(g.results.at(mm), "matmul").to_host_f16_codes();
+    double worst = 0, rms = 0;
+    for (int t = 0; t < m; ++t)
+        for (int r = 0; r < n; ++r) {
+            double s = 0;
+            for (int c = 0; c < dim; ++c)
+                s += static_cast<double>(f16_value(rows[static_cast<size_t>(t) * dim + c])) *
+                     (static_cast<double>(wq[static_cast<size_t>(r) * dim + c]) * wd[(static_cast<size_t>(r) * dim + c) / 32]);
+            worst = std::max(worst, std::fabs(f16_value(out[static_cast<size_t>(t) * n + r]) - s));
+            rms += s * s;
+        }
+    EXPECT(worst < 2e-3 * std::sqrt(rms / (m * n)));
+}
+
 int main(int argc, char **argv) {
     const std::string mode = argc > 1 ? argv[1] : "cpu";
     try {
@@ -220,6 +276,7 @@ int main(int argc, char **argv) {
             check(lhip_init(0), "lhip_init");
             test_quantized_matvec_like_the_reference();
             test_quantized_matmul_and_graph_execution();
+            test_f16_graph();
         }
     } catch (const std::exception &e) {
         std::printf("FAIL unexpected exception: %s\n", e.what());
