@@ -377,9 +377,19 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
     const int my_groups = wave_global < n_groups ? (n_groups - wave_global + total_waves - 1) / total_waves : 0;
     const int T = my_groups * chunks;
 
+    // EPI_ADD: the residual of a row group is requested together with the group's first weight step, i.e. ahead
+    // of loads the pipeline waits for anyway.  Read at the group's end instead, it would be the youngest load in
+    // flight and waiting for it would drain the prefetched next step every time (wait counts retire in order).
+    auto residual_of = [&](const Located &l, bool live) -> float {
+        const int row = l.row0 + static_cast<int>(lane);
+        return (EPI == EPI_ADD && live && lane < static_cast<unsigned>(R) && row < l.n) ? f.residual[row] : 0.f;
+    };
+    float res_cur = 0.f, res_next = 0.f;
+
     StepBuf<R, S> a, b;
     {
         const Located l = locate<R>(p, wave_global < n_groups ? wave_global : 0);
+        res_cur = residual_of(l, T > 0);
         load_step(a, l.qs, l.ds, l.row0, l.n, k, 0, lane, T > 0);
     }
 
@@ -430,6 +440,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
     };
     auto issue = [&](StepBuf<R, S> &buf, int gg, int cc, bool live) {
         const Located l = locate<R>(p, live ? gg : 0);
+        if (EPI == EPI_ADD && cc == 0) res_next = residual_of(l, live);
         load_step(buf, l.qs, l.ds, l.row0, l.n, k, cc * S, lane, live);
     };
     auto finish_group = [&](int gg) {
@@ -458,9 +469,10 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
                 if (lane == static_cast<unsigned>(r)) out = sum[r];
             const int row = l.row0 + static_cast<int>(lane);
             if (lane < static_cast<unsigned>(R) && row < l.n) {
-                if (EPI == EPI_ADD) out += f.residual[row];
+                if (EPI == EPI_ADD) out += res_cur;
                 l.y[row] = out;
             }
+            if (EPI == EPI_ADD) res_cur = res_next;
         }
     };
 
