@@ -111,17 +111,21 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     gu32x4 a_reg[D][A_CHUNKS], b_reg[D][B_CHUNKS];
     uint32_t d_reg[D][B_CHUNKS];  // both f16 scale codes of the tile
     const int KT = K / kBK;
-    auto load_tile = [&](int set, int kt) {
+    // part p of P: the p-th share of the thread's chunks (P = 1: everything), the same split as store_tile's.
+    auto load_tile = [&](int set, int kt, int p = 0, int P = 1) {
         const int k0 = min(kt, KT - 1) * kBK;  // tiles past the end re-read the last one (never used)
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) a_reg[set][i] = *reinterpret_cast<const gu32x4 *>(a_src[i] + k0);
+        for (int i = 0; i < A_CHUNKS; ++i)
+            if (i * P / A_CHUNKS == p) a_reg[set][i] = *reinterpret_cast<const gu32x4 *>(a_src[i] + k0);
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
+            if (i * P / B_CHUNKS != p) continue;
             b_reg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
             d_reg[set][i] = d_src[i][k0 >> 6];
         }
     };
-    // part p of P: the p-th share of the thread's chunks (P = 1: everything).
+    // part p of P: the p-th share of the thread's chunks (P = 1: everything).  A weight chunk (16 quants -> two
+    // 16-byte halves of bf16) counts as two units, so its unpacking can be spread over two parts.
     auto store_tile = [&](int set, int buf, int p = 0, int P = 1) {
         unsigned char *A = lds + buf * (A_BYTES + B_BYTES);
         unsigned char *B = A + A_BYTES;
@@ -129,17 +133,22 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         for (int i = 0; i < A_CHUNKS; ++i)
             if (i * P / A_CHUNKS == p) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
 #pragma unroll
-        for (int i = 0; i < B_CHUNKS; ++i) {
-            if (i * P / B_CHUNKS != p) continue;
+        for (int u = 0; u < 2 * B_CHUNKS; ++u) {
+            if (u * P / (2 * B_CHUNKS) != p) continue;
+            const int i = u >> 1;
             // Opaque to the optimiser: keeps the unpacking of this set here, at its use,
             // instead of next to its loads (where it would wait for data just requested).
             asm volatile("" : "+v"(b_reg[set][i]), "+v"(d_reg[set][i]));
             const float d = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[set][i] >> d_shift[i])));
-            const uint2 w0 = dequant4_bf16(b_reg[set][i].x, d), w1 = dequant4_bf16(b_reg[set][i].y, d);
-            const uint2 w2 = dequant4_bf16(b_reg[set][i].z, d), w3 = dequant4_bf16(b_reg[set][i].w, d);
-            gu32x4 lo = {w0.x, w0.y, w1.x, w1.y}, hi = {w2.x, w2.y, w3.x, w3.y};
-            *reinterpret_cast<gu32x4 *>(B + b_dst[i]) = lo;
-            *reinterpret_cast<gu32x4 *>(B + b_dst[i] + 16) = hi;
+            if ((u & 1) == 0) {
+                const uint2 w0 = dequant4_bf16(b_reg[set][i].x, d), w1 = dequant4_bf16(b_reg[set][i].y, d);
+                gu32x4 lo = {w0.x, w0.y, w1.x, w1.y};
+                *reinterpret_cast<gu32x4 *>(B + b_dst[i]) = lo;
+            } else {
+                const uint2 w2 = dequant4_bf16(b_reg[set][i].z, d), w3 = dequant4_bf16(b_reg[set][i].w, d);
+                gu32x4 hi = {w2.x, w2.y, w3.x, w3.y};
+                *reinterpret_cast<gu32x4 *>(B + b_dst[i] + 16) = hi;
+            }
         }
     };
 
@@ -174,7 +183,11 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     // Pipelined form of compute_tile + store_tile: the operand fragments of step kk+1 are requested before the
     // MFMAs of step kk, and the dequantise-and-store of the next tile is dealt out over the four steps so its VALU
     // and LDS-write work sits between the MFMAs instead of after them (measured: +10 % on the large shapes).
-    auto compute_and_store = [&](int buf, int set, int next_buf) {
+    // The global loads of the tile after next are dealt out the same way: issued all at once at the top of a step
+    // by all eight waves, they fill the memory pipeline's queue (48 KiB per K tile at 64 B/clk is ~770 cycles) and
+    // the later waves sit in their load instructions for ~1000 cycles while the first wave of each SIMD runs its
+    // MFMAs alone; the two waves of a SIMD then work one after the other instead of side by side.
+    auto compute_and_store = [&](int buf, int set, int next_buf, int load_set, int load_kt) {
         const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
         const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
         bf16x8 af[2][FM], bfr[2][FN];
@@ -189,6 +202,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         for (int kk = 0; kk < kBK / 16; ++kk) {
             if (kk + 1 < kBK / 16) load_frags(kk + 1, (kk + 1) & 1);
             store_tile(set, next_buf, kk, kBK / 16);
+            load_tile(load_set, load_kt, kk, kBK / 16);
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -215,14 +229,14 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int j = 0; j < D; ++j) {
                 // set j held tile kt+j, already in LDS: refill it with tile kt+j+D
-                load_tile(j, kt + j + D);
-                // Keep the loads here, at the top of the step: if they sink towards the
-                // LDS stores below, the wait for the tile loaded D-1 steps ago also
-                // waits for them and the prefetch distance collapses.
-                __builtin_amdgcn_sched_barrier(0);
                 if constexpr (PIPE) {
-                    compute_and_store(j & 1, (j + 1) % D, (j + 1) & 1);
+                    compute_and_store(j & 1, (j + 1) % D, (j + 1) & 1, j, kt + j + D);
                 } else {
+                    load_tile(j, kt + j + D);
+                    // Keep the loads here, at the top of the step: if they sink towards the
+                    // LDS stores below, the wait for the tile loaded D-1 steps ago also
+                    // waits for them and the prefetch distance collapses.
+                    __builtin_amdgcn_sched_barrier(0);
                     compute_tile(j & 1);
                     store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
                 }
