@@ -203,7 +203,7 @@ def bench_prefill_gemm(args):
         "dtype": "int8 weights dequantised to bf16 x bf16 activations, f32 accumulate, bf16 out", "data": "synthetic",
         "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list)},
         "per_shape": per,
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true> (gate/up, M=2048)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true, __bf16> (gate/up, M=2048)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_us": round(us, 1)}}))
 
