@@ -147,6 +147,12 @@ lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, voi
  * whose surrounding operators are f32 wants instead of a bf16 round trip. */
 lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_dev, float *y_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream);
+/* Same GEMM over a weight whose rows are (gate, up) pairs (row 2j = gate_j, row 2j+1 = up_j, the order the fused
+ * matvec's SwiGLU epilogue uses), writing out[r][j] = up * swish(gate) (examples/llama/src/model.rs:24-32) as bf16,
+ * (m, N/2) row-major, 4-byte aligned: the f32 accumulators never leave the kernel.  Bit-equal to
+ * lhip_q8_0_matmul_bf16_f32out followed by lhip_swiglu_f32_bf16out(interleaved).  N % 4 == 0. */
+lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_dev, void *out_dev, int64_t m, int64_t n,
+                                         int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
  * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
  * K % 128 == 0, else LHIP_ERR_UNSUPPORTED). */

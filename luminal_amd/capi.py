@@ -40,6 +40,7 @@ SIGNATURES = {
                                                    _int, _int, _vp]),
     "lhip_q8_0_matmul_bf16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_bf16_f32out": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_bf16_swiglu": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_bf16_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

@@ -59,6 +59,10 @@ static inline size_t mx_scale_offset(int64_t n, int64_t k) {
 static inline size_t mx_planar_nbytes(int64_t n, int64_t k) {
     return mx_scale_offset(n, k) + static_cast<size_t>(mx_panels(n)) * static_cast<size_t>(mx_chunks(k)) * 64;
 }
+// up * swish(gate) in f32 (examples/llama/src/model.rs:24-32, src/hl_ops/unary.rs:169-177): one definition, so the
+// element-wise kernel and the GEMM epilogue give the same bits.
+__device__ __forceinline__ float swiglu_value(float gate, float up) { return up * (gate * (1.0f / (1.0f + expf(-gate)))); }
+
 // Piece index (in units of 16 nibble bytes / 1 scale byte) of block kb of row.
 __host__ __device__ static inline size_t mx_piece(int64_t row, int64_t kb, int64_t chunks) {
     return (static_cast<size_t>(row >> 4) * chunks + (kb >> 2)) * 64 + (kb & 3) * 16 + (row & 15);

@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
     const int j = static_cast<int>(i - s * f);
     const float g = gu[s * 2 * f + (interleaved ? 2 * j : j)];
     const float u = gu[s * 2 * f + (interleaved ? 2 * j + 1 : f + j)];
-    out[i] = static_cast<OutT>(u * (g * (1.0f / (1.0f + expf(-g)))));
+    out[i] = static_cast<OutT>(swiglu_value(g, u));
 }
 
 __global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ y,

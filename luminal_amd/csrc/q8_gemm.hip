@@ -53,7 +53,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
                                                                    const __half *__restrict__ ds,
                                                                    const __bf16 *__restrict__ x,
                                                                    OutT *__restrict__ y, int M, int N, int K,
-                                                                   int m_tiles, int n_tiles) {
+                                                                   int m_tiles, int n_tiles, int swiglu) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 MFMA tiles per wave
@@ -246,6 +246,32 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     }
 
     // Epilogue: acc element v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile.
+    if constexpr (sizeof(OutT) == 2) {
+        if (swiglu) {
+            // Columns are (gate, up) pairs (weight rows interleaved at load): y[row][c/2] = up * swish(gate), N/2
+            // columns of bf16.  A pair sits in neighbouring lanes; two pairs are packed into one 4-byte store.
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const int col = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                        const float mine = acc[i][j][v], other = __shfl_xor(mine, 1);
+                        const float act = (lane & 1) ? swiglu_value(other, mine) : swiglu_value(mine, other);
+                        const float act2 = __shfl_xor(act, 2);
+                        if ((lane & 3) == 0 && row < M && col < N) {
+                            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                            const bf16x2 pk = {static_cast<__bf16>(act), static_cast<__bf16>(act2)};
+                            *reinterpret_cast<bf16x2 *>(reinterpret_cast<__bf16 *>(y) +
+                                                        static_cast<size_t>(row) * (N >> 1) + (col >> 1)) = pk;
+                        }
+                    }
+                }
+            return;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -259,9 +285,12 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         }
 }
 
+// What the epilogue writes: bf16 (m, N), f32 (m, N), or bf16 (m, N/2) = up * swish(gate) of (gate, up) column pairs.
+enum { kOutBf16 = 0, kOutF32 = 1, kOutSwiglu = 2 };
+
 template <int BM, int BN, int WM, int WN, int D, bool PIPE, typename OutT>
 static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
-                                 hipStream_t s) {
+                                 int swiglu, hipStream_t s) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
@@ -272,25 +301,26 @@ static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void 
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     }
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad)), dim3(WM * WN * 64), lds_bytes, s, qs,
-                       ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m, n, k, m_tiles, n_tiles);
+                       ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m, n, k, m_tiles, n_tiles, swiglu);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
 template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
-static lhip_status launch_gemm(bool f32_out, const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n,
+static lhip_status launch_gemm(int out, const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n,
                                int k, hipStream_t s) {
-    return f32_out ? launch_gemm_t<BM, BN, WM, WN, D, PIPE, float>(qs, ds, x, y, m, n, k, s)
-                   : launch_gemm_t<BM, BN, WM, WN, D, PIPE, __bf16>(qs, ds, x, y, m, n, k, s);
+    return out == kOutF32 ? launch_gemm_t<BM, BN, WM, WN, D, PIPE, float>(qs, ds, x, y, m, n, k, 0, s)
+                          : launch_gemm_t<BM, BN, WM, WN, D, PIPE, __bf16>(qs, ds, x, y, m, n, k, out == kOutSwiglu, s);
 }
 
 static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
-                                 int tile, bool f32_out, void *stream) {
+                                 int tile, int out, void *stream) {
     if (!planar_dev || !x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_q8_shape(n, k)) return s;
     if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     if (k % kBK != 0) return LHIP_ERR_UNSUPPORTED;
-    if (!aligned(planar_dev, 256) || !aligned(x_dev, 16) || !aligned(y_dev, f32_out ? 4 : 2)) return LHIP_ERR_MISALIGNED;
+    if (out == kOutSwiglu && n % 4 != 0) return LHIP_ERR_INVALID_SHAPE;  // pairs, stored two at a time
+    if (!aligned(planar_dev, 256) || !aligned(x_dev, 16) || !aligned(y_dev, out == kOutBf16 ? 2 : 4)) return LHIP_ERR_MISALIGNED;
     auto *base = static_cast<const uint8_t *>(planar_dev);
     auto *qs = reinterpret_cast<const int8_t *>(base);
     auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
@@ -299,8 +329,8 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
     // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
     const bool deep = (k % (kBK * 4)) == 0;
 #define LHIP_TILE(BM, BN, WM, WN)                                                                  \
-    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s) \
-                : launch_gemm<BM, BN, WM, WN, 1>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
+    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s) \
+                : launch_gemm<BM, BN, WM, WN, 1>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
     switch (tile) {
         case 0: LHIP_TILE(256, 128, 4, 2);
         case 1: LHIP_TILE(128, 128, 2, 2);
@@ -309,7 +339,7 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
         case 4:  // 256x256 by eight 64x128 waves: 0.75 KiB of LDS operand reads per MFMA instead of 1; both
                  // LDS buffers together are 144 KiB, which leaves registers for a prefetch depth of two K tiles
             if (k % (kBK * 2) != 0) return LHIP_ERR_UNSUPPORTED;
-            return launch_gemm<256, 256, 4, 2, 2, true>(f32_out, qs, ds, x_dev, y_dev, mi, ni, ki, s);
+            return launch_gemm<256, 256, 4, 2, 2, true>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s);
         default: return LHIP_ERR_UNSUPPORTED;
     }
 #undef LHIP_TILE
@@ -336,17 +366,22 @@ extern "C" {
 
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, tile, false, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, tile, kOutBf16, stream);
 }
 
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), false, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), kOutBf16, stream);
 }
 
 lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_dev, float *y_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), true, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), kOutF32, stream);
+}
+
+lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_dev, void *out_dev, int64_t m, int64_t n,
+                                         int64_t k, void *stream) {
+    return gemm_dispatch(planar_dev, x_dev, out_dev, m, n, k, gemm_auto_tile(m, n, k), kOutSwiglu, stream);
 }
 
 }  // extern "C"

@@ -160,7 +160,6 @@ class LlamaQ8:
         attb = self._buf("attb", (s, d), bf)
         att = self._buf("att", (s, d))
         o = self._buf("o", (s, d))
-        gu = self._buf("gu", (s, 2 * cfg.ffn))
         actb = self._buf("actb", (s, cfg.ffn), bf)
         dn = self._buf("dn", (s, d))
 
@@ -193,8 +192,9 @@ class LlamaQ8:
                 capi.check(st, "lhip_attention_f32_bf16out")
             gemm(w[f"{i}.o"], attb, o, s)
             norm(o, w[f"{i}.ffn_norm"])                              # h += attention out; nb = norm(h)
-            gemm(w[f"{i}.gate_up"], nb, gu, s)
-            capi.check(lib.lhip_swiglu_f32_bf16out(gu.data_ptr(), actb.data_ptr(), s, cfg.ffn, 1, _s()), "swiglu")
+            gw = w[f"{i}.gate_up"]                                   # rows are (gate, up) pairs: SwiGLU in the epilogue
+            capi.check(lib.lhip_q8_0_matmul_bf16_swiglu(gw.planar.data_ptr(), nb.data_ptr(), actb.data_ptr(), s, gw.n,
+                                                        gw.k, _s()), "lhip_q8_0_matmul_bf16_swiglu")
             gemm(w[f"{i}.down"], actb, dn, s)
         if all_logits:
             norm(dn, w["out_norm"])

@@ -157,3 +157,25 @@ def test_f32_output_is_the_unrounded_accumulator(oracle, m, n, k):
     assert elem < TOL and norm < 4e-3, (elem, norm)
     assert lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr() + 2, m, n, k,
                                             st) == capi.LHIP_ERR_MISALIGNED
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 64, 64), (130, 200, 128), (512, 1024, 256), (300, 28672 // 8, 512)])
+def test_swiglu_epilogue_equals_gemm_then_swiglu(m, n, k):
+    """lhip_q8_0_matmul_bf16_swiglu == lhip_q8_0_matmul_bf16_f32out followed by lhip_swiglu_f32_bf16out on
+    interleaved (gate, up) columns, bit for bit, on every tile the library would pick and on ragged edges."""
+    lib = capi.load_library()
+    qs, d = synth.q8_0_random(n, k, seed=m + n + k)
+    w = upload(qs, d)
+    x = torch.from_numpy(synth.activations(m, k, seed=9)).to(DEV).to(torch.bfloat16)
+    s = torch.cuda.current_stream().cuda_stream
+    y32 = torch.empty(m, n, device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, s), "gemm")
+    want = torch.empty(m, n // 2, device=DEV, dtype=torch.bfloat16)
+    capi.check(lib.lhip_swiglu_f32_bf16out(y32.data_ptr(), want.data_ptr(), m, n // 2, 1, s), "swiglu")
+    got = torch.full((m, n // 2), 7.0, device=DEV, dtype=torch.bfloat16)
+    capi.check(lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), got.data_ptr(), m, n, k, s), "fused")
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # pairs are stored two at a time: N must be a multiple of 4
+    assert lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), got.data_ptr(), m, n - 2, k, s) \
+        == capi.LHIP_ERR_INVALID_SHAPE
