@@ -837,15 +837,17 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     MoeWorkspace w = carve(workspace_dev, t, h, i, e, topk);
     const int Hp = static_cast<int>(pad128(h)), Ip = static_cast<int>(pad128(i));
 
-    // Row tile: as many routed rows per expert as there are on average, 16..128.
+    // Row tile: tall enough for an expert with two standard deviations more rows than the average (rows per
+    // expert are roughly Poisson), so that nearly every expert is one tile and its weights are read once.
     const int avg = (R + E - 1) / E;
-    const int mt = avg > 96 ? 10 : avg > 64 ? 8 : (avg > 32 ? 4 : (avg > 16 ? 2 : 1));
+    const int need = avg + 2 * static_cast<int>(sqrtf(static_cast<float>(avg)) + 0.5f);
+    const int mt = need > 128 ? 10 : need > 64 ? 8 : (need > 32 ? 4 : (need > 16 ? 2 : 1));
     const int BM = 16 * mt;
     const int max_tiles = R / BM + E;
-    // A handful of routed rows in total (batch-1 decode and the like): stage each tile's
-    // activation rows whole and run the barrier-free weight stream.  With more rows per expert
-    // that staging costs more than it saves (measured at T = 64: 168 us against 108 us).
-    const bool decode_sized = R <= 4 * E / 2;
+    // One token's worth of routed rows (batch-1 decode): stage each tile's activation rows whole and run the
+    // barrier-free weight stream.  From two tokens on the chunked kernel below is faster (measured, us per layer,
+    // whole-row kernel / chunked: T = 1 31.6 / 39.5, T = 2 45.9 / 42.8, T = 8 80 / 64, T = 32 126 / 92).
+    const bool decode_sized = R <= 4;
 
     {
         const size_t items = static_cast<size_t>(T) * (Hp / 8);
@@ -871,10 +873,10 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         case 1:
             st = decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024
                      ? launch_moe_gemm_small<2, true>(a1, cb1, max_tiles, s)
-                                                       : launch_moe_gemm<1, 2, true>(a1, cb1, max_tiles, s);
+                                                       : launch_moe_gemm<1, 4, true>(a1, cb1w, max_tiles, s);
             break;
-        case 2: st = launch_moe_gemm<2, 2, true>(a1, cb1, max_tiles, s); break;
-        case 4: st = launch_moe_gemm<4, 4, true>(a1, cb1w, max_tiles, s); break;
+        case 2: st = launch_moe_gemm<2, 4, true>(a1, cb1w, max_tiles, s); break;
+        case 4: st = launch_moe_gemm<4, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
         case 8: st = launch_moe_gemm<8, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
         default: st = launch_moe_gemm<10, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
     }
@@ -895,12 +897,12 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     if (mt == 1) {
         st = decode_sized && moe_small_lds_bytes(Ip) <= 150 * 1024
                  ? launch_moe_gemm_small<1, false>(a2, (H + 63) / 64, max_tiles, s)
-                                                   : launch_moe_gemm<1, 1, false>(a2, (H + 63) / 64, max_tiles, s);
+                                                   : launch_moe_gemm<1, 2, false>(a2, (H + 127) / 128, max_tiles, s);
     } else {
         const int cb2 = (H + 127) / 128, cb2w = (H + 255) / 256;  // 4 waves x NT fragments of 16
         switch (mt) {
             case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
-            case 4: st = launch_moe_gemm<4, 4, false>(a2, cb2w, max_tiles, s); break;
+            case 4: st = launch_moe_gemm<4, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
             case 8: st = launch_moe_gemm<8, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
             default: st = launch_moe_gemm<10, 3, false, 2, 2>(a2, (H + 191) / 192, max_tiles, s); break;
         }
