@@ -267,6 +267,10 @@ struct MoeGemmArgs {
     int N;                              // output columns per expert (I or H)
     const int *tile_expert, *tile_row0, *tile_rows, *n_tiles;
     void *out;                          // bf16 [R][N] (gated) or f32 [R][N]
+    // Gated GEMM with NT == 4 only: when q_hi is set, the epilogue quantises its bf16 result for the next GEMM
+    // (planes of row stride q_kp, scales of row stride q_kp / 32) instead of writing `out`.
+    uint8_t *q_hi, *q_lo, *q_sc;
+    int q_kp;
 };
 
 // f(integral_constant<int, 1>) ... f(integral_constant<int, N-1>), expanded at compile time.
@@ -519,6 +523,51 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
     }
 
     // ---- epilogue: acc[i][f][v] is row i*16 + 4*grp + v, column fragment f, column r
+    if constexpr (GATED && NT == 4) {
+        if (g.q_hi) {
+            // The wave's two (gate, up) pairs are the 32 intermediate columns [32 b, 32 b + 32), b = 4 blockIdx.x +
+            // wave: one quantisation block of the next GEMM's activations.  Same arithmetic as
+            // mx_quantize_act_kernel on the bf16-rounded result (block maximum over the 16 lanes of a row group),
+            // so the intermediate activations never go through memory as bf16.
+            const int b = blockIdx.x * 4 + wave;
+#pragma unroll
+            for (int i = 0; i < MTW; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int m = (i * WR + wrow) * 16 + 4 * grp + v;
+                    if (m >= rows) continue;  // uniform over the 16 lanes that exchange values below
+                    float a[2];
+#pragma unroll
+                    for (int p = 0; p < 2; ++p) {
+                        const float gate = acc[i][2 * p][v], up = acc[i][2 * p + 1][v];
+                        const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
+                        a[p] = col[2 * p] < g.N ? static_cast<float>(static_cast<__bf16>(act)) : 0.f;
+                    }
+                    float amax = fmaxf(fabsf(a[0]), fabsf(a[1]));
+#pragma unroll
+                    for (int o = 1; o < 16; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+                    int e = 127;
+                    float inv = 1.0f;
+                    if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
+                        const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);
+                        e = max(ex - 7, 1);
+                        inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);
+                    }
+                    const float s0 = a[0] * inv, s1 = a[1] * inv;
+                    const int h = __builtin_amdgcn_cvt_pk_fp8_f32(s0, s1, 0, false);
+                    const float r0 = s0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), r1 = s1 - __builtin_amdgcn_cvt_f32_fp8(h, 1);
+                    const int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, 0, false);
+                    const size_t at = static_cast<size_t>(row0 + m) * g.q_kp + b * 32 + r;
+                    g.q_hi[at] = static_cast<uint8_t>(h);
+                    g.q_hi[at + 16] = static_cast<uint8_t>(h >> 8);
+                    g.q_lo[at] = static_cast<uint8_t>(l);
+                    g.q_lo[at + 16] = static_cast<uint8_t>(l >> 8);
+                    if (r == 0)
+                        g.q_sc[static_cast<size_t>(row0 + m) * (g.q_kp / 32) + b] = static_cast<uint8_t>(b * 32 < g.N ? e : 127);
+                }
+            return;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < MTW; ++i)
 #pragma unroll
@@ -865,14 +914,17 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
     a1.n_tiles = w.plan.n_tiles; a1.out = w.act;
+    const bool whole_rows = mt == 1 && decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024;
+    if (!whole_rows) {  // every chunked gated kernel has NT == 4 and quantises in its epilogue
+        a1.q_hi = w.a_hi; a1.q_lo = w.a_lo; a1.q_sc = w.a_sc; a1.q_kp = Ip;
+    }
     // Column blocks: 4 waves x (NT/2) gate/up pairs of 16.  Tall row tiles take 4 weight
     // fragments per wave, so each activation fragment read from LDS feeds twice the MFMAs.
     const int cb1 = (I + 63) / 64, cb1w = (I + 127) / 128;
     lhip_status st;
     switch (mt) {
         case 1:
-            st = decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024
-                     ? launch_moe_gemm_small<2, true>(a1, cb1, max_tiles, s)
+            st = whole_rows ? launch_moe_gemm_small<2, true>(a1, cb1, max_tiles, s)
                                                        : launch_moe_gemm<1, 4, true>(a1, cb1w, max_tiles, s);
             break;
         case 2: st = launch_moe_gemm<2, 4, true>(a1, cb1w, max_tiles, s); break;
@@ -881,7 +933,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         default: st = launch_moe_gemm<10, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
-    {
+    if (whole_rows) {
         const size_t threads = static_cast<size_t>(R) * (Ip / 8);
         hipLaunchKernelGGL(mx_quantize_act_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s,
                            w.act, w.a_hi, w.a_lo, w.a_sc, R, I, Ip);
