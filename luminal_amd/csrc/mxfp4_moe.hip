@@ -233,12 +233,6 @@ __device__ __forceinline__ void mx_quantize_act_item(size_t idx, const __bf16 *_
     if ((c8 & 3) == 0) sc[row * (Kp / 32) + (c8 >> 2)] = static_cast<uint8_t>(k < K ? e : 127);
 }
 
-__global__ __launch_bounds__(256) void mx_quantize_act_kernel(const __bf16 *__restrict__ x, uint8_t *__restrict__ hi,
-                                                              uint8_t *__restrict__ lo, uint8_t *__restrict__ sc,
-                                                              int rows, int K, int Kp) {
-    mx_quantize_act_item(static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x, x, hi, lo, sc, rows, K, Kp);
-}
-
 // The two independent first steps of a layer pass in one launch: workgroup 0 makes the plan, the others
 // quantise the layer input (1024 items each).
 __global__ __launch_bounds__(1024) void moe_prepare_kernel(const int *__restrict__ sel, int R, int E, int BM, MoePlan p,
@@ -527,7 +521,7 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
         if (g.q_hi) {
             // The wave's two (gate, up) pairs are the 32 intermediate columns [32 b, 32 b + 32), b = 4 blockIdx.x +
             // wave: one quantisation block of the next GEMM's activations.  Same arithmetic as
-            // mx_quantize_act_kernel on the bf16-rounded result (block maximum over the 16 lanes of a row group),
+            // mx_quantize_act_item on the bf16-rounded result (block maximum over the 16 lanes of a row group),
             // so the intermediate activations never go through memory as bf16.
             const int b = blockIdx.x * 4 + wave;
 #pragma unroll
@@ -718,6 +712,61 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
         }
     }
 
+    if constexpr (GATED && NT == 2) {
+        if (g.q_hi) {
+            // Quantise the result for the next GEMM here (same arithmetic as mx_quantize_act_item on the
+            // bf16-rounded values).  A wave holds 16 of a block's 32 columns; the two waves of a block exchange
+            // their row maxima through LDS, which the K loop no longer needs.
+            __syncthreads();  // every wave is done reading the staged activations
+            float *pmax = reinterpret_cast<float *>(lds);  // [4 waves][16 rows]
+            float a[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float gate = acc[0][v], up = acc[1][v];
+                const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
+                a[v] = col[0] < g.N ? static_cast<float>(static_cast<__bf16>(act)) : 0.f;
+                float mx = fabsf(a[v]);
+#pragma unroll
+                for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+                if (r == 0) pmax[wave * 16 + 4 * grp + v] = mx;
+            }
+            __syncthreads();
+            const int b = blockIdx.x * 2 + (wave >> 1);  // quantisation block of this wave's columns
+            const int half = (wave & 1) * 16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int m = 4 * grp + v;
+                if (m >= rows) continue;
+                const float amax = fmaxf(pmax[wave * 16 + m], pmax[(wave ^ 1) * 16 + m]);
+                int e = 127;
+                float inv = 1.0f;
+                if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
+                    const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);
+                    e = max(ex - 7, 1);
+                    inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);
+                }
+                const float s0 = a[v] * inv;
+                const int h = __builtin_amdgcn_cvt_pk_fp8_f32(s0, 0.f, 0, false);
+                const int l = __builtin_amdgcn_cvt_pk_fp8_f32(s0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), 0.f, 0, false);
+                const size_t at = static_cast<size_t>(row0 + m) * g.q_kp + b * 32 + half + r;
+                g.q_hi[at] = static_cast<uint8_t>(h);
+                g.q_lo[at] = static_cast<uint8_t>(l);
+                const size_t sc_at = static_cast<size_t>(row0 + m) * (g.q_kp / 32);
+                if (r == 0 && half == 0) g.q_sc[sc_at + b] = static_cast<uint8_t>(e);
+                // The last column block also fills the padding past N up to the padded row length: zeros, scale 2^0.
+                if (blockIdx.x == gridDim.x - 1 && wave == 0) {
+                    const int k0 = (g.N + 63) / 64 * 64;  // the column blocks end here
+                    for (int k = k0 + r; k < g.q_kp; k += 16) {
+                        g.q_hi[static_cast<size_t>(row0 + m) * g.q_kp + k] = 0;
+                        g.q_lo[static_cast<size_t>(row0 + m) * g.q_kp + k] = 0;
+                    }
+                    if (r == 0)
+                        for (int kb = k0 / 32; kb < g.q_kp / 32; ++kb) g.q_sc[sc_at + kb] = 127;
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int m = 4 * grp + v;
@@ -915,9 +964,8 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
     a1.n_tiles = w.plan.n_tiles; a1.out = w.act;
     const bool whole_rows = mt == 1 && decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024;
-    if (!whole_rows) {  // every chunked gated kernel has NT == 4 and quantises in its epilogue
-        a1.q_hi = w.a_hi; a1.q_lo = w.a_lo; a1.q_sc = w.a_sc; a1.q_kp = Ip;
-    }
+    // Every gated kernel launched below quantises its result for the down GEMM in its epilogue.
+    a1.q_hi = w.a_hi; a1.q_lo = w.a_lo; a1.q_sc = w.a_sc; a1.q_kp = Ip;
     // Column blocks: 4 waves x (NT/2) gate/up pairs of 16.  Tall row tiles take 4 weight
     // fragments per wave, so each activation fragment read from LDS feeds twice the MFMAs.
     const int cb1 = (I + 63) / 64, cb1w = (I + 127) / 128;
@@ -933,12 +981,6 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         default: st = launch_moe_gemm<10, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
-    if (whole_rows) {
-        const size_t threads = static_cast<size_t>(R) * (Ip / 8);
-        hipLaunchKernelGGL(mx_quantize_act_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s,
-                           w.act, w.a_hi, w.a_lo, w.a_sc, R, I, Ip);
-        LHIP_CHECK_LAUNCH();
-    }
     MoeGemmArgs a2{};
     a2.a_hi = w.a_hi; a2.a_lo = w.a_lo; a2.a_sc = w.a_sc;
     a2.a_index = nullptr; a2.a_div = 1;
