@@ -267,6 +267,16 @@ struct MoeGemmArgs {
     int q_kp;
 };
 
+// Maximum over the 16 lanes of a DPP row, in every lane of the row (quad swaps, then the two mirrors): register
+// moves only, where a shuffle would go through the LDS pipeline.
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)));
+    return v;
+}
+
 // f(integral_constant<int, 1>) ... f(integral_constant<int, N-1>), expanded at compile time.
 template <class F, int... Is>
 __device__ __forceinline__ void static_for_from1_impl(F &&f, std::integer_sequence<int, Is...>) {
@@ -537,9 +547,7 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
                         const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
                         a[p] = col[2 * p] < g.N ? static_cast<float>(static_cast<__bf16>(act)) : 0.f;
                     }
-                    float amax = fmaxf(fabsf(a[0]), fabsf(a[1]));
-#pragma unroll
-                    for (int o = 1; o < 16; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+                    const float amax = row16_max(fmaxf(fabsf(a[0]), fabsf(a[1])));
                     int e = 127;
                     float inv = 1.0f;
                     if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
@@ -725,9 +733,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
                 const float gate = acc[0][v], up = acc[1][v];
                 const float act = up * (gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * gate)));
                 a[v] = col[0] < g.N ? static_cast<float>(static_cast<__bf16>(act)) : 0.f;
-                float mx = fabsf(a[v]);
-#pragma unroll
-                for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+                const float mx = row16_max(fabsf(a[v]));
                 if (r == 0) pmax[wave * 16 + 4 * grp + v] = mx;
             }
             __syncthreads();
