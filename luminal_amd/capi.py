@@ -60,6 +60,7 @@ SIGNATURES = {
     "lhip_rope_kv_append_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp]),
     "lhip_attention_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lhip_attention_f32_bf16out": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "lhip_attention_bf16": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lhip_attention_decode_workspace_nbytes": (C.c_size_t, [_i64, _i64, _i64]),
     "lhip_attention_decode_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp]),
     "lhip_swiglu_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _int, _vp]),

@@ -16,6 +16,9 @@ namespace lhip {
 // attention_prefill.hip: matrix-core kernel for prompt-sized calls; false if the shape is not built.
 bool attention_prefill_launch(const float *qkv, const float *kc, const float *vc, void *out, bool out_bf16, const int *pos,
                               int tokens, int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s);
+// attention_prefill_bf16.hip: the same sweep with bf16 matrix-core operands, bf16 out.
+bool attention_prefill_bf16_launch(const float *qkv, const float *kc, const float *vc, void *out, const int *pos, int tokens,
+                                   int q_heads, int kv_heads, int head_dim, int max_seq, hipStream_t s);
 
 __device__ __forceinline__ float block_sum(float v, float *red) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -459,6 +462,23 @@ lhip_status lhip_attention_f32_bf16out(const float *qkv_dev, const float *k_cach
                                   static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
                                   static_cast<int>(max_seq), as_stream(stream)))
         return LHIP_ERR_UNSUPPORTED;  // only the matrix-core kernel writes bf16
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_attention_bf16(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
+                                void *out_bf16_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
+                                int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream) {
+    if (!qkv_dev || !k_cache_dev || !v_cache_dev || !out_bf16_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
+    if (tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_seq <= 0 || q_heads % kv_heads != 0 ||
+        tokens > kMaxDim || max_seq > kMaxDim)
+        return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(qkv_dev, 16) || !aligned(k_cache_dev, 16) || !aligned(v_cache_dev, 16) || !aligned(out_bf16_dev, 8))
+        return LHIP_ERR_MISALIGNED;
+    if (!attention_prefill_bf16_launch(qkv_dev, k_cache_dev, v_cache_dev, out_bf16_dev, pos_dev, static_cast<int>(tokens),
+                                       static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim),
+                                       static_cast<int>(max_seq), as_stream(stream)))
+        return LHIP_ERR_UNSUPPORTED;
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }

@@ -180,16 +180,18 @@ class LlamaQ8:
             capi.check(lib.lhip_rope_kv_append_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
                                                    self.v_cache[i].data_ptr(), self.pos.data_ptr(), s, cfg.q_heads,
                                                    cfg.kv_heads, hd, self.max_seq, cfg.theta, _s()), "rope")
-            st = lib.lhip_attention_f32_bf16out(qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
-                                                attb.data_ptr(), self.pos.data_ptr(), s, cfg.q_heads, cfg.kv_heads, hd,
-                                                self.max_seq, _s())
-            if st == capi.LHIP_ERR_UNSUPPORTED:  # head shape without a matrix-core kernel: f32 attention, then cast
-                capi.check(lib.lhip_attention_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
-                                                  self.v_cache[i].data_ptr(), att.data_ptr(), self.pos.data_ptr(), s,
-                                                  cfg.q_heads, cfg.kv_heads, hd, self.max_seq, _s()), "attention")
+            a_args = (qkv.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr())
+            a_dims = (self.pos.data_ptr(), s, cfg.q_heads, cfg.kv_heads, hd, self.max_seq, _s())
+            # bf16 matrix-core operands where the head shape has that kernel, else the f32 matrix-core kernel
+            # writing bf16, else (no matrix-core kernel at all) the f32 attention and a cast
+            st = lib.lhip_attention_bf16(*a_args, attb.data_ptr(), *a_dims)
+            if st == capi.LHIP_ERR_UNSUPPORTED:
+                st = lib.lhip_attention_f32_bf16out(*a_args, attb.data_ptr(), *a_dims)
+            if st == capi.LHIP_ERR_UNSUPPORTED:
+                capi.check(lib.lhip_attention_f32(*a_args, att.data_ptr(), *a_dims), "attention")
                 capi.check(lib.lhip_cast_f32_to_bf16(att.data_ptr(), attb.data_ptr(), s * d, _s()), "cast")
             else:
-                capi.check(st, "lhip_attention_f32_bf16out")
+                capi.check(st, "prompt attention")
             gemm(w[f"{i}.o"], attb, o, s)
             norm(o, w[f"{i}.ffn_norm"])                              # h += attention out; nb = norm(h)
             gw = w[f"{i}.gate_up"]                                   # rows are (gate, up) pairs: SwiGLU in the epilogue

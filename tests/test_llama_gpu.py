@@ -208,6 +208,102 @@ def test_prompt_attention_on_matrix_cores(hq, hkv, hd, S, pos0):
     assert err < 1e-5, err
 
 
+def _bf16(x):
+    """Round to bfloat16 (nearest even) and return as float64."""
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).bfloat16().double().numpy()
+
+
+def _attention_with_bf16_roundings(qkv, kc, vc, hq, hkv, hd, pos0):
+    """softmax(QK)V in f64 with the five roundings of the bf16 kernel placed where it places them: q / sqrt(hd), K and
+    V rounded once; per 32-key tile the weights exp(s - running max) rounded and the running sum taken over the
+    rounded weights; the quotient rounded at the store."""
+    S, g = qkv.shape[0], hq // hkv
+    q = _bf16(qkv[:, :hq].astype(np.float32) * (np.float32(1.0) / np.sqrt(np.float32(hd))))
+    kb, vb = _bf16(kc), _bf16(vc)
+    n_keys = pos0 + S
+    out = np.empty((S, hq, hd))
+    visible = np.arange(n_keys)[None, :] <= (pos0 + np.arange(S))[:, None]
+    for h in range(hq):
+        sc = np.where(visible, q[:, h] @ kb[h // g, :n_keys].T, -np.inf)
+        m = np.full(S, -np.inf)
+        l, acc = np.zeros(S), np.zeros((S, hd))
+        for k0 in range(0, n_keys, 32):
+            tile = sc[:, k0:k0 + 32]
+            m_new = np.maximum(m, tile.max(axis=1))
+            corr = np.exp(m - m_new)
+            w = _bf16(np.exp(tile - m_new[:, None]))
+            l = l * corr + w.sum(axis=1)
+            acc = acc * corr[:, None] + w @ vb[h // g, k0:k0 + 32][:w.shape[1]]
+            m = m_new
+        out[:, h] = _bf16(acc / l[:, None])
+    return out.reshape(S, -1)
+
+
+@pytest.mark.parametrize("hq,hkv,hd", [(8, 2, 128), (32, 8, 128), (16, 2, 64), (4, 2, 128), (8, 4, 64), (16, 2, 128)])
+@pytest.mark.parametrize("S,pos0", [(8, 0), (33, 0), (70, 5), (64, 64), (129, 31), (300, 0)])
+def test_prompt_attention_with_bf16_operands(hq, hkv, hd, S, pos0):
+    """The bf16 matrix-core form, for query blocks and key tiles that are ragged, start mid-cache and span several
+    tiles, against two references.
+
+    (1) f64 arithmetic with the kernel's five bf16 roundings (q, K, V, soft-max weights, result) in their places. What
+        is left is f32 against f64 accumulation and the roundings it tips, of which one at the store moves an element
+        by one bf16 ulp, at most 2^-7 of its size: max |y - r| / max(|r|, rms(r)) < 1e-2.
+    (2) the exact f64 softmax(QK)V = sum_j p_j v_j, with the error measured against the sum before cancellation,
+        a = sum_j p_j |v_j|, per element. bf16's unit roundoff is 2^-8: the roundings of V, of the weights and of
+        the result bound the error by 3 * 2^-8 * a = 1.2e-2 * a between them, and the rounding of q and K adds the
+        relative error of a weight that the soft-max makes of an error of a score (restated on the CPU, the five
+        together reach 1.1e-2 * a on these inputs): |y - t| < 2e-2 * a.
+    The f32-operand kernel behind lhip_attention_f32 and lhip_attention_f32_bf16out is the one held to 1e-5."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(hq * 100 + S + pos0 + 7)
+    max_seq = 384
+    kc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    vc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    qkv = rng.standard_normal((S, hq + 2 * hkv, hd)).astype(np.float32)
+    kd, vd, qd = (torch.from_numpy(a).to(DEV) for a in (kc, vc, qkv))
+    pos = torch.tensor([pos0], dtype=torch.int32, device=DEV)
+    out = torch.full((S, hq * hd), float("nan"), device=DEV, dtype=torch.bfloat16)
+    assert lib.lhip_attention_bf16(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), pos.data_ptr(), S, hq,
+                                   hkv, hd, max_seq, s()) == 0
+    got = out.double().cpu().numpy()
+    g = hq // hkv
+    exact, scale = np.empty((S, hq, hd)), np.empty((S, hq, hd))
+    for t in range(S):
+        n = pos0 + t + 1
+        for h in range(hq):
+            sc = kc[h // g, :n].astype(np.float64) @ qkv[t, h].astype(np.float64) / np.sqrt(hd)
+            w = np.exp(sc - sc.max())
+            w /= w.sum()
+            exact[t, h] = w @ vc[h // g, :n].astype(np.float64)
+            scale[t, h] = w @ np.abs(vc[h // g, :n].astype(np.float64))
+    rounded = _attention_with_bf16_roundings(qkv, kc, vc, hq, hkv, hd, pos0)
+    e1 = np.max(np.abs(got - rounded) / np.maximum(np.abs(rounded), np.sqrt(np.mean(rounded * rounded))))
+    e2 = np.max(np.abs(got - exact.reshape(S, -1)) / scale.reshape(S, -1))
+    assert e1 < 1e-2 and e2 < 2e-2, (e1, e2)
+    # a query that sees one key returns that key's V row, rounded
+    if pos0 == 0:
+        assert np.array_equal(got[0].reshape(hq, hd), np.repeat(_bf16(vc[:, 0]), g, axis=0))
+    # the caches are only read
+    assert np.array_equal(kd.cpu().numpy(), kc) and np.array_equal(vd.cpu().numpy(), vc)
+
+
+def test_bf16_prompt_attention_argument_errors():
+    lib = capi.load_library()
+    a = torch.zeros(1 << 16, device=DEV)
+    pos = torch.zeros(1, dtype=torch.int32, device=DEV)
+
+    def call(S=8, hq=8, hkv=2, hd=128, qkv=a.data_ptr(), out=a.data_ptr(), max_seq=8):
+        return lib.lhip_attention_bf16(qkv, a.data_ptr(), a.data_ptr(), out, pos.data_ptr(), S, hq, hkv, hd, max_seq, s())
+
+    assert call() == capi.LHIP_OK
+    assert call(hq=4, hkv=4) == capi.LHIP_ERR_UNSUPPORTED  # one query head per key head has no bf16 kernel
+    assert call(hq=32, hkv=2) == capi.LHIP_ERR_UNSUPPORTED and call(hd=32) == capi.LHIP_ERR_UNSUPPORTED
+    assert call(hq=7, hkv=2) == capi.LHIP_ERR_INVALID_SHAPE and call(max_seq=0) == capi.LHIP_ERR_INVALID_SHAPE
+    assert call(qkv=None) == capi.LHIP_ERR_NULL_PTR and call(out=None) == capi.LHIP_ERR_NULL_PTR
+    assert call(S=0) == capi.LHIP_ERR_INVALID_SHAPE
+    torch.cuda.synchronize()
+
+
 def test_decode_attention_argument_errors():
     lib = capi.load_library()
     a = torch.zeros(4096, device=DEV)
