@@ -140,7 +140,17 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
  * (crates/luminal_metal/src/quantized.rs:54-61,63-199,353-376).  Weights are
  * rounded to bf16 after dequantisation, so results are within 1e-2 of the f32
  * semantics, not bit-equal.  K must be a multiple of 64 (LHIP_ERR_UNSUPPORTED
- * otherwise). */
+ * otherwise).
+ *
+ * With m <= 128 (and K % 512 == 0, N % 4 == 0, y aligned to 8 bytes; 16 for the f32
+ * form below) the three entry points take a kernel that is bound by streaming the
+ * weights rather than by the matrix cores.  When the 128-row strips of the weight
+ * alone would not fill the chip it also splits K, keeps the f32 partial sums in a
+ * 32 MiB scratch array that the library owns (a __device__ array: nothing is
+ * allocated, one copy per device) and adds them in a fixed order in a second
+ * launch.  Every such call on a device shares that array: calls with m <= 128 that
+ * may overlap on one device (different streams, different host threads) race on it
+ * and must be ordered by the caller.  Results do not depend on timing. */
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream);
 /* Same GEMM with the f32 accumulators stored as they are (y (m, N) f32, 4-byte aligned): what a caller
@@ -155,7 +165,9 @@ lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_d
                                          int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
  * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
- * K % 128 == 0, else LHIP_ERR_UNSUPPORTED). */
+ * K % 128 == 0, else LHIP_ERR_UNSUPPORTED), 5 = the weight-streaming kernel for
+ * m <= 128 described above (LHIP_ERR_UNSUPPORTED for shapes it does not cover),
+ * 50 + S = the same with S slices of K (S clamped to K / 512). */
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream);
 

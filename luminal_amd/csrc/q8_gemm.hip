@@ -288,6 +288,13 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 // What the epilogue writes: bf16 (m, N), f32 (m, N), or bf16 (m, N/2) = up * swish(gate) of (gate, up) column pairs.
 enum { kOutBf16 = 0, kOutF32 = 1, kOutSwiglu = 2 };
 
+// q8_gemm_skinny.hip: the weight-streaming kernel for at most 128 activation rows.
+bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y);
+lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
+                                  int out, int splits, hipStream_t s);
+constexpr int kTileSkinny = 5;        // K slices chosen by the library
+constexpr int kTileSkinnySplit = 50;  // + number of K slices
+
 template <int BM, int BN, int WM, int WN, int D, bool PIPE, typename OutT>
 static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
                                  int swiglu, hipStream_t s) {
@@ -331,6 +338,10 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
 #define LHIP_TILE(BM, BN, WM, WN)                                                                  \
     return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s) \
                 : launch_gemm<BM, BN, WM, WN, 1>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
+    if (tile == kTileSkinny || (tile > kTileSkinnySplit && tile <= kTileSkinnySplit + 64)) {
+        if (!q8_gemm_skinny_supports(mi, ni, ki, out, y_dev)) return LHIP_ERR_UNSUPPORTED;
+        return q8_gemm_skinny_launch(qs, ds, x_dev, y_dev, mi, ni, ki, out, tile == kTileSkinny ? 0 : tile - kTileSkinnySplit, s);
+    }
     switch (tile) {
         case 0: LHIP_TILE(256, 128, 4, 2);
         case 1: LHIP_TILE(128, 128, 2, 2);
@@ -345,7 +356,11 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
 #undef LHIP_TILE
 }
 
-static int gemm_auto_tile(int64_t m, int64_t n, int64_t k) {
+static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *y) {
+    // Few activation rows: the product is bound by the weight stream
+    if (m <= 128 && n <= kMaxDim && k <= kMaxDim &&
+        q8_gemm_skinny_supports(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), out, y))
+        return kTileSkinny;
     // Largest tile that still gives at least three quarters of the 256 CUs a
     // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
     // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
@@ -371,17 +386,17 @@ lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev,
 
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), kOutBf16, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k, kOutBf16, y_dev), kOutBf16, stream);
 }
 
 lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_dev, float *y_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k), kOutF32, stream);
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k, kOutF32, y_dev), kOutF32, stream);
 }
 
 lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_dev, void *out_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream) {
-    return gemm_dispatch(planar_dev, x_dev, out_dev, m, n, k, gemm_auto_tile(m, n, k), kOutSwiglu, stream);
+    return gemm_dispatch(planar_dev, x_dev, out_dev, m, n, k, gemm_auto_tile(m, n, k, kOutSwiglu, out_dev), kOutSwiglu, stream);
 }
 
 }  // extern "C"

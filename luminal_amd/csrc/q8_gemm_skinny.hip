@@ -1,0 +1,416 @@
+// Q8_0 weights x bf16 activations for 2..128 activation rows (short prompts, small batches).
+//
+// With so few activation rows the product is bound by streaming the weights, not by the matrix cores, and the
+// 128/256-row tiles of q8_gemm.hip leave most of the chip idle.  Here a workgroup owns a strip of 128 weight rows
+// (and, when the strips alone would not fill the chip, a slice of K) and streams it from HBM straight into
+// registers in matrix-core operand order:
+//
+//   * waves 0-3 ("compute") take 32 weight rows each, two 16-row blocks.  Lane (r, g) = (lane % 16, lane / 16)
+//     loads the 16 codes k = 64*group + 16*g .. +16 of row r with one 16-byte load: the A operands of two
+//     v_mfma_f32_16x16x32_bf16 steps, whose k slots (g, e) are taken to mean k = 16*g + 8*step + e.  Eight groups
+//     (512 k) per row block are in flight per wave, reloaded in place as they are consumed; the codes are
+//     dequantised (q * d rounded to bf16, as in q8_gemm.hip) one group ahead of their MFMAs, in between them.
+//   * waves 4-7 ("loaders") stage the activations for all four compute waves: (16*MT) x (64*G) tiles of x go
+//     through their registers into one of three LDS buffers, two tiles ahead, one barrier per tile.  The compute
+//     waves never wait for an activation load, so their in-order load counter only ever sees the weight stream.
+//     In LDS a tile is G panels of 64 k, a row of a panel 128 bytes at pitch 160 (free of bank conflicts for the
+//     16-lane x 4-group operand reads), with its eight 16-byte pieces permuted so that piece g + 4*step holds
+//     k = 16*g + 8*step .. +8: the B operand of a step is one 16-byte read.
+//
+// K slices write f32 partial tiles to a scratch array owned by the library (one per device, shared by every
+// call on it) and a second kernel adds them in slice order and applies the output form, so results do not depend
+// on timing.
+#include <hip/hip_fp16.h>
+
+#include <type_traits>
+#include <utility>
+
+#include "common.h"
+
+namespace lhip {
+
+typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float sk_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
+
+enum { kSkOutBf16 = 0, kSkOutF32 = 1, kSkOutSwiglu = 2, kSkOutPartial = 3 };  // first three as in q8_gemm.hip
+
+constexpr int kSkRows = 128;    // weight rows per workgroup
+constexpr int kSkPitch = 160;   // bytes per activation row of a panel in LDS
+constexpr int kSkStages = 3;    // LDS buffers
+constexpr int kSkUnit = 512;     // K slices are whole multiples of this (eight groups of 64 k)
+constexpr size_t kSkScratchFloats = size_t{8} << 20;  // 32 MiB of partial sums
+
+static __device__ __align__(256) float sk_scratch[kSkScratchFloats];
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), expanded at compile time (a pragma gives up on
+// bodies this large, and register arrays indexed at run time land in scratch memory).
+template <class F, int... Is>
+__device__ __forceinline__ void sk_static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void sk_static_for(F &&f) {
+    sk_static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
+}
+
+template <int MT>
+struct SkShape {
+    static constexpr int G = MT >= 8 ? 2 : 4;  // groups per activation tile; a slice is an even number of tiles
+    static constexpr int PANEL = 16 * MT * kSkPitch;
+    static constexpr int STAGE = G * PANEL;
+    static constexpr int CHUNKS = 16 * MT * G * 8;             // 16-byte pieces per tile
+    static constexpr int CH = CHUNKS / 256;                    // per loader thread
+    static_assert(CHUNKS % 256 == 0 && 8 % G == 0, "tile split");
+    static constexpr size_t LDS = static_cast<size_t>(kSkStages) * STAGE;
+};
+
+// Two packed int8 (half `h` of a dword) -> two bf16 of q * d, packed.  A byte is converted as unsigned (one
+// instruction), so the dword arrives biased by 128 per byte (w = q ^ 0x80808080) and the fma takes the bias out
+// again: (q + 128) * d - 128 * d is exact in an fma because q * d has at most 19 significant bits, and the value
+// rounded to bf16 is that of q * d itself.
+__device__ __forceinline__ uint32_t sk_dequant2(uint32_t w, int h, float d, float off) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const float lo = fmaf(static_cast<float>((w >> (16 * h)) & 0xffu), d, off);
+    const float hi = fmaf(static_cast<float>((w >> (16 * h + 8)) & 0xffu), d, off);
+    const bf16x2 pk = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, pk);
+}
+
+// One output form for four consecutive weight rows n .. n+3 of activation row m.
+template <int OUT>
+__device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M, int N, int m, int n, sk_f32x4 v) {
+    if constexpr (OUT == kSkOutPartial) {
+        *reinterpret_cast<sk_f32x4 *>(part + (static_cast<size_t>(split) * M + m) * N + n) = v;
+    } else if constexpr (OUT == kSkOutF32) {
+        *reinterpret_cast<sk_f32x4 *>(static_cast<float *>(y) + static_cast<size_t>(m) * N + n) = v;
+    } else if constexpr (OUT == kSkOutBf16) {
+        typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+        const bf16x4 w = {static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1]), static_cast<__bf16>(v[2]),
+                          static_cast<__bf16>(v[3])};
+        *reinterpret_cast<bf16x4 *>(static_cast<__bf16 *>(y) + static_cast<size_t>(m) * N + n) = w;
+    } else {  // rows are (gate, up) pairs
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const bf16x2 w = {static_cast<__bf16>(swiglu_value(v[0], v[1])), static_cast<__bf16>(swiglu_value(v[2], v[3]))};
+        *reinterpret_cast<bf16x2 *>(static_cast<__bf16 *>(y) + static_cast<size_t>(m) * (N >> 1) + (n >> 1)) = w;
+    }
+}
+
+// grid (strips of 128 weight rows, K slices); 512 threads.  K % 512 == 0, N % 4 == 0, M <= 16 * MT.
+// A slice is `slice_groups` groups of 64 k (a multiple of 8); the last may be shorter (also a multiple of 8).
+// RING = groups in flight per wave and row block (8 or 16); a slice is a multiple of RING groups.
+template <int MT, int OUT, int RING>
+__global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
+                                                             const __bf16 *__restrict__ x, void *__restrict__ y,
+                                                             float *__restrict__ part, int M, int N, int K,
+                                                             int slice_groups) {
+    using S = SkShape<MT>;
+    constexpr int G = S::G;
+    extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int strip = blockIdx.x, split = blockIdx.y;
+    const int g_begin = split * slice_groups;
+    const int n_groups = min(slice_groups, (K >> 6) - g_begin);
+    const int n_tiles = n_groups / G;
+    // With few activation rows every strip starts its walk over K at a different place (a whole number of rings):
+    // the strips advance at the same pace and would otherwise all ask the same memory channels for the same k at
+    // the same time (measured: 39 -> 36 us for 28672 x 4096 at 16 rows).  With many rows the strips reading the
+    // same activation tile at the same time is worth more (57 against 64 us at 128 rows).
+    const int rot = MT <= 2 ? (strip % (n_groups / RING)) * RING : 0;
+
+    if (wave >= 4) {
+        // ---------------- loaders: x tiles -> LDS, two tiles ahead of the compute waves
+        const int lt = tid - 256;
+        const __bf16 *src[S::CH];
+        int dst[S::CH];
+#pragma unroll
+        for (int i = 0; i < S::CH; ++i) {
+            const int c = lt + i * 256;
+            const int m = c / (G * 8), j = c % (G * 8);
+            const int panel = j >> 3, jj = j & 7;
+            src[i] = x + static_cast<size_t>(min(m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
+            dst[i] = panel * S::PANEL + m * kSkPitch + ((jj >> 1) + 4 * (jj & 1)) * 16;
+        }
+        sk_u32x4 xr[2][S::CH];
+        auto load_x = [&](int slot, int t) __attribute__((always_inline)) {
+            int tt = min(t, n_tiles - 1) + rot / G;  // past the end: re-read, never used
+            if (tt >= n_tiles) tt -= n_tiles;
+            const size_t off = static_cast<size_t>(tt) * (G * 64);
+#pragma unroll
+            for (int i = 0; i < S::CH; ++i) xr[slot][i] = *reinterpret_cast<const sk_u32x4 *>(src[i] + off);
+        };
+        auto store_x = [&](int slot, int stage) __attribute__((always_inline)) {
+            unsigned char *base = sk_lds + stage * S::STAGE;
+#pragma unroll
+            for (int i = 0; i < S::CH; ++i) *reinterpret_cast<sk_u32x4 *>(base + dst[i]) = xr[slot][i];
+        };
+        load_x(0, 0);
+        load_x(1, 1);
+        store_x(0, 0);
+        load_x(0, 2);
+        store_x(1, 1);
+        load_x(1, 3);
+        __syncthreads();
+        int stage = 2;  // buffer of tile t + 2
+        for (int t = 0; t < n_tiles; t += 2) {  // two tiles per trip: no branch between them, so the counted waits
+                                                // are exact (the loads of a slot are two tiles old when it is stored)
+            store_x(0, stage);  // tile t + 2 (a buffer last read for tile t - 1)
+            load_x(0, t + 4);
+            stage = stage == 2 ? 0 : stage + 1;
+            __syncthreads();
+            store_x(1, stage);  // tile t + 3
+            load_x(1, t + 5);
+            stage = stage == 2 ? 0 : stage + 1;
+            __syncthreads();
+        }
+        return;
+    }
+
+    // ---------------- compute waves
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = strip * kSkRows + wave * 32;
+    const int8_t *a_ptr[2];
+    const __half *d_ptr[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        const int row = min(n0 + rb * 16 + r, N - 1);
+        a_ptr[rb] = qs + static_cast<size_t>(row) * K + static_cast<size_t>(g_begin) * 64 + 16 * g;
+        d_ptr[rb] = ds + static_cast<size_t>(row) * (K >> 5) + static_cast<size_t>(g_begin) * 2;
+    }
+    const int d_shift = (g >> 1) * 16;  // a lane's 16 codes lie in block 2*group + g/2
+    const int n_rounds = n_groups >> 2;
+
+    sk_u32x4 a_reg[RING][2], d_reg[RING / 4][2];
+    auto load_a = [&](int u, int group) __attribute__((always_inline)) {
+        int gg = min(group, n_groups - 1) + rot;
+        if (gg >= n_groups) gg -= n_groups;
+        const size_t off = static_cast<size_t>(gg) * 64;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+            a_reg[u][rb] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4 *>(a_ptr[rb] + off));
+    };
+    auto load_d = [&](int set, int round) __attribute__((always_inline)) {
+        int rr = min(round, n_rounds - 1) + rot / 4;
+        if (rr >= n_rounds) rr -= n_rounds;
+        const size_t off = static_cast<size_t>(rr) * 8;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) d_reg[set][rb] = *reinterpret_cast<const sk_u32x4 *>(d_ptr[rb] + off);
+    };
+    // Dequantisation of ring slot `un` in sixteen pieces of two codes: piece p belongs to row block p / 8,
+    // step (p / 4) % 2, dword p / 2 of the lane's four, half p % 2.
+    float d_next[2], off_next[2];
+    auto dequant_piece = [&](sk_u32x4 (&to)[2][2], int un, int p) __attribute__((always_inline)) {
+        const int rb = p >> 3, dw = (p >> 1) & 3;
+        // Opaque to the optimiser: keeps the unpacking here, at its use, instead of next to the load
+        asm volatile("" : "+v"(a_reg[un][rb]));
+        if ((p & 7) == 0) {
+            const uint32_t bits = (d_reg[un >> 2][rb][un & 3] >> d_shift) & 0xffffu;
+            d_next[rb] = __half2float(__ushort_as_half(static_cast<unsigned short>(bits)));
+            off_next[rb] = -128.f * d_next[rb];
+        }
+        if ((p & 1) == 0) a_reg[un][rb][dw] ^= 0x80808080u;
+        to[rb][(p >> 2) & 1][(p >> 1) & 1 ? 2 + (p & 1) : (p & 1)] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
+    };
+
+    // the loop reloads in the order a0 a1 a2 a3 d0 a4 a5 a6 a7 d1: the same order here, so the counted waits of the
+    // first trip are those of the steady state
+#pragma unroll
+    for (int u = 0; u < RING; ++u) {
+        load_a(u, u);
+        if ((u & 3) == 3) load_d(u >> 2, u >> 2);
+    }
+
+    sk_f32x4 acc[2][MT];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < MT; ++cb) acc[rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // A group is UNITS = 2 * MT units (step, column block): one B operand read and two MFMAs each.  W reads are
+    // kept in flight, running ahead into the next group (whose tile was complete in LDS a barrier ago), and the
+    // next group's dequantisation is dealt out over the units, so that LDS latency and VALU work sit under MFMAs.
+    constexpr int UNITS = 2 * MT;
+    constexpr int W = UNITS < 4 ? UNITS : 4;
+    auto b_read = [&](const unsigned char *xb, int i) __attribute__((always_inline)) {
+        return *reinterpret_cast<const sk_bf16x8 *>(xb + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
+    };
+    sk_u32x4 af[2][2];  // [row block][step] of the group being multiplied, as packed bf16
+    sk_bf16x8 bw[W];
+#pragma unroll
+    for (int p = 0; p < 16; ++p) dequant_piece(af, 0, p);
+    const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
+    __syncthreads();  // tiles 0 and 1 are staged
+#pragma unroll
+    for (int i = 0; i < W; ++i) bw[i] = b_read(xb_cur, i);
+    int stage = 0;
+    for (int R = 0; R < n_rounds; R += RING / 4) {
+        sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
+            constexpr int u = decltype(uc)::value;
+            constexpr int un = (u + 1) % RING;  // ring slot of the next group
+            constexpr bool tile_ends = (u + 1) % G == 0;
+            const int gl = R * 4 + u;
+            const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
+            const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
+            sk_u32x4 af_next[2][2];
+            sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                const sk_bf16x8 b = bw[i % W];
+                bw[i % W] = i + W < UNITS ? b_read(xb_cur, i + W) : b_read(xb_next, i + W - UNITS);
+                sk_static_for<16>([&](auto pc) __attribute__((always_inline)) {
+                    constexpr int p = decltype(pc)::value;
+                    if constexpr (p * UNITS / 16 == i) {
+                        dequant_piece(af_next, un, p);
+                        if constexpr (p == 15 && (un & 3) == 3) {
+                            // the four groups of this round are unpacked: request the round after next, 256
+                            // consecutive bytes of every row back to back
+                            sk_static_for<4>([&](auto qc) __attribute__((always_inline)) {
+                                constexpr int q = decltype(qc)::value;
+                                load_a(un - 3 + q, gl + 1 - 3 + q + RING);
+                            });
+                            load_d(un >> 2, R + RING / 4 + (un >> 2));
+                        }
+                    }
+                });
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    acc[rb][i % MT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[rb][i / MT]), b,
+                                                                              acc[rb][i % MT], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int st = 0; st < 2; ++st) af[rb][st] = af_next[rb][st];
+            xb_cur = xb_next;
+            if constexpr (tile_ends) {
+                stage = stage_next;
+                __syncthreads();
+            }
+        });
+    }
+
+    // ---------------- lane (r, g) holds activation row 16*cb + r and weight rows n0 + 16*rb + 4*g .. +4
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        const int n = n0 + rb * 16 + 4 * g;
+        if (n >= N) continue;  // N % 4 == 0: the four rows are in or out together
+#pragma unroll
+        for (int cb = 0; cb < MT; ++cb) {
+            const int m = cb * 16 + r;
+            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[rb][cb]);
+        }
+    }
+}
+
+// Sum of the K slices in slice order, then the output form.  One thread per four weight rows.
+template <int OUT>
+__global__ __launch_bounds__(256) void q8_gemm_skinny_reduce_kernel(const float *__restrict__ part, void *__restrict__ y,
+                                                                    int M, int N, int splits) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t quads = static_cast<size_t>(M) * (N >> 2);
+    if (i >= quads) return;
+    const size_t plane = static_cast<size_t>(M) * N;
+    sk_f32x4 v = *reinterpret_cast<const sk_f32x4 *>(part + 4 * i);
+    for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const sk_f32x4 *>(part + s * plane + 4 * i);
+    const int m = static_cast<int>(i / (N >> 2)), n = static_cast<int>(i % (N >> 2)) * 4;
+    sk_store4<OUT>(y, nullptr, 0, M, N, m, n, v);
+}
+
+// Scratch address per device (a __device__ array has one copy, at its own address, on every device).
+static float *sk_scratch_ptr() {
+    static float *ptrs[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    float *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(sk_scratch)) != hipSuccess) return nullptr;
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+    }
+    return p;
+}
+
+// K slices for a product: enough workgroups for the 256 CUs, slices of whole 512-k units, partial sums within the
+// scratch array.
+int q8_gemm_skinny_splits(int m, int n, int k) {
+    const int strips = (n + kSkRows - 1) / kSkRows, units = k / kSkUnit;
+    int s = 256 / strips;
+    if (s < 1) s = 1;
+    if (s > units) s = units;
+    while (s > 1 && static_cast<size_t>(s) * m * n > kSkScratchFloats) --s;
+    const int per = (units + s - 1) / s;
+    return (units + per - 1) / per;
+}
+
+bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y) {
+    return m >= 1 && m <= 128 && k % kSkUnit == 0 && n % 4 == 0 && aligned(y, out == kSkOutF32 ? 16 : (out == kSkOutBf16 ? 8 : 4));
+}
+
+template <int MT, int OUT, int RING>
+static lhip_status sk_launch_r(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
+                               int k, int splits, int slice_groups, hipStream_t s) {
+    auto kern = q8_gemm_skinny_kernel<MT, OUT, RING>;
+    constexpr size_t lds_bytes = SkShape<MT>::LDS;
+    if (lds_bytes > 64 * 1024)  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
+        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(lds_bytes)));
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits)),
+                       dim3(512), lds_bytes, s, qs, ds, x, y, part, m, n, k, slice_groups);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+template <int MT, int OUT>
+static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
+                               int k, int splits, hipStream_t s) {
+    const int units = k / kSkUnit, per = (units + splits - 1) / splits;
+    return sk_launch_r<MT, OUT, 8>(qs, ds, x, y, part, m, n, k, splits, per * 8, s);
+}
+
+template <int MT>
+static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m,
+                                int n, int k, int splits, hipStream_t s) {
+    if (splits > 1) return sk_launch_t<MT, kSkOutPartial>(qs, ds, x, y, part, m, n, k, splits, s);
+    switch (out) {
+        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16>(qs, ds, x, y, part, m, n, k, 1, s);
+        case kSkOutF32: return sk_launch_t<MT, kSkOutF32>(qs, ds, x, y, part, m, n, k, 1, s);
+        default: return sk_launch_t<MT, kSkOutSwiglu>(qs, ds, x, y, part, m, n, k, 1, s);
+    }
+}
+
+// `splits` = 0: chosen here.  The caller has checked q8_gemm_skinny_supports.
+lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
+                                  int out, int splits, hipStream_t s) {
+    const int units = k / kSkUnit;
+    if (splits <= 0) splits = q8_gemm_skinny_splits(m, n, k);
+    if (splits > units) splits = units;
+    {
+        const int per = (units + splits - 1) / splits;
+        splits = (units + per - 1) / per;  // no empty slice
+    }
+    float *part = nullptr;
+    if (splits > 1) {
+        if (static_cast<size_t>(splits) * m * n > kSkScratchFloats) return LHIP_ERR_UNSUPPORTED;
+        part = sk_scratch_ptr();
+        if (!part) return LHIP_ERR_HIP;
+    }
+    const __bf16 *x = static_cast<const __bf16 *>(x_bf16);
+    lhip_status st;
+    if (m <= 16) st = sk_launch_mt<1>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    else if (m <= 32) st = sk_launch_mt<2>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    else if (m <= 64) st = sk_launch_mt<4>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    else st = sk_launch_mt<8>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    if (st != LHIP_OK || splits == 1) return st;
+    const size_t quads = static_cast<size_t>(m) * (n >> 2);
+    const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
+    switch (out) {
+        case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
+        case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
+        default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
+    }
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+}  // namespace lhip

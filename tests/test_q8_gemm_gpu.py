@@ -122,6 +122,98 @@ def test_full_size_prefill_shapes(oracle, name, m):
     assert not ye[np.arange(m) != m // 2].any()
 
 
+# ---- the weight-streaming kernel for at most 128 activation rows (K % 512 == 0, N % 4 == 0): tile id 5 lets
+# the library choose the number of K slices, 50 + S asks for S of them
+
+SKINNY_AUTO, SKINNY_SLICES = 5, 50
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 128, 512), (15, 100, 1024), (16, 260, 512), (17, 4, 1536), (33, 1024, 2048),
+                                   (64, 132, 4096), (100, 516, 1024), (127, 128, 512), (128, 256, 14336)])
+def test_weight_streaming_gemm_vs_oracle(oracle, m, n, k):
+    """Every activation-row bracket (16, 32, 64, 128), ragged strips of weight rows, one to eight K slices (more
+    slices than K has 512-element units are clamped).  The f32 output is held to the bar against the f64 product;
+    the bf16 output is that result rounded once; another number of K slices only changes the order of the f32
+    additions, which may tip the final rounding of a few elements by one bf16 step (or, where a sum cancelled,
+    show the f32 rounding of its terms)."""
+    lib = capi.load_library()
+    st = torch.cuda.current_stream().cuda_stream
+    qs, d = synth.q8_0_random(n, k, seed=m + n + k)
+    xf, bits = bf16_activations(oracle, m, k, seed=m * n + 1)
+    w = upload(qs, d)
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y32 = torch.full((m, n), float("nan"), device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st), "f32out")
+    elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+    auto = run(w, bits, SKINNY_AUTO)
+    assert np.array_equal(auto, y32.to(torch.bfloat16).float().cpu().numpy())
+    for slices in (1, 2, 3, 8):
+        y = run(w, bits, SKINNY_SLICES + slices)
+        # one bf16 step where the rounding tipped, and f32 rounding of the terms where the sum cancelled
+        step = np.abs(auto) * 2.0 ** -7 + 1e-4 * float(np.sqrt(np.mean(auto * auto)))
+        assert np.all(np.abs(y - auto) <= step) and np.mean(y == auto) > 0.98, slices
+
+
+def test_weight_streaming_gemm_is_the_one_chosen_and_is_repeatable(oracle):
+    """For m <= 128 the plain entry point takes the weight-streaming kernel (same bits as asking for it), K slices
+    are added in a fixed order (two runs agree bit for bit, and a product that is exact in f32 is the same for
+    every number of slices), and shapes it does not cover fall back to the tiled kernels."""
+    lib = capi.load_library()
+    s = torch.cuda.current_stream().cuda_stream
+    m, n, k = 48, 4096, 4096
+    qs, d = synth.q8_0_random(n, k, seed=77)
+    w = upload(qs, d)
+    _, bits = bf16_activations(oracle, m, k, seed=78)
+    a = run(w, bits)
+    assert np.array_equal(a, run(w, bits, SKINNY_AUTO)) and np.array_equal(a, run(w, bits))
+    assert not np.array_equal(a, run(w, bits, 2))  # the tiled kernel adds in another order
+    # small integers and power-of-two scales: every partial sum is exact
+    rng = np.random.default_rng(5)
+    m, n, k = 70, 152, 2048
+    qi = rng.integers(-8, 9, (n, k), dtype=np.int8)
+    di = (2.0 ** rng.integers(-2, 2, (n, k // 32))).astype(np.float16)
+    x = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    xb = (x.view(np.uint32) >> 16).astype(np.uint16)
+    want = x.astype(np.float64) @ (qi.astype(np.float64) * np.repeat(di.astype(np.float64), 32, axis=1)).T
+    want_bf16 = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).float().numpy()
+    wi = upload(qi, di)
+    for tile in (None, SKINNY_AUTO, SKINNY_SLICES + 1, SKINNY_SLICES + 2, SKINNY_SLICES + 4):
+        assert np.array_equal(run(wi, xb, tile), want_bf16), tile
+    # not covered: K not a multiple of 512, N not a multiple of 4, more than 128 rows
+    xd = torch.zeros((129, 4096), dtype=torch.bfloat16, device=DEV)
+    yd = torch.zeros((129, 4096), dtype=torch.bfloat16, device=DEV)
+
+    def cfg(mm, nn, kk):
+        return lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), xd.data_ptr(), yd.data_ptr(), mm, nn, kk, SKINNY_AUTO, s)
+
+    assert cfg(129, 64, 512) == capi.LHIP_ERR_UNSUPPORTED and cfg(8, 64, 576) == capi.LHIP_ERR_UNSUPPORTED
+    assert cfg(8, 66, 512) == capi.LHIP_ERR_UNSUPPORTED and cfg(8, 64, 512) == capi.LHIP_OK
+    torch.cuda.synchronize()
+
+
+def test_weight_streaming_gemm_output_forms(oracle):
+    """f32, bf16 and SwiGLU outputs of the same product, with and without K slices: bf16 is the f32 result rounded
+    once, SwiGLU is lhip_swiglu_f32_bf16out of it."""
+    lib = capi.load_library()
+    s = torch.cuda.current_stream().cuda_stream
+    for (m, n, k) in ((24, 28672 // 4, 4096), (128, 512, 4096), (9, 4096, 14336)):  # one slice, then several
+        qs, d = synth.q8_0_random(n, k, seed=m + n)
+        w = upload(qs, d)
+        x = torch.from_numpy(synth.activations(m, k, seed=3)).to(DEV).to(torch.bfloat16)
+        y32 = torch.empty(m, n, device=DEV)
+        y16 = torch.empty(m, n, device=DEV, dtype=torch.bfloat16)
+        act = torch.empty(m, n // 2, device=DEV, dtype=torch.bfloat16)
+        want = torch.empty_like(act)
+        capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, s), "f32")
+        capi.check(lib.lhip_q8_0_matmul_bf16(w.planar.data_ptr(), x.data_ptr(), y16.data_ptr(), m, n, k, s), "bf16")
+        capi.check(lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), act.data_ptr(), m, n, k, s), "swiglu")
+        capi.check(lib.lhip_swiglu_f32_bf16out(y32.data_ptr(), want.data_ptr(), m, n // 2, 1, s), "swiglu of f32")
+        torch.cuda.synchronize()
+        assert torch.equal(y32.to(torch.bfloat16), y16)
+        assert torch.equal(act.view(torch.int16), want.view(torch.int16))
+
+
 def test_gemm_argument_errors():
     lib = capi.load_library()
     w = upload(*synth.q8_0_random(64, 96, seed=1))
@@ -159,7 +251,8 @@ def test_f32_output_is_the_unrounded_accumulator(oracle, m, n, k):
                                             st) == capi.LHIP_ERR_MISALIGNED
 
 
-@pytest.mark.parametrize("m,n,k", [(5, 64, 64), (130, 200, 128), (512, 1024, 256), (300, 28672 // 8, 512)])
+@pytest.mark.parametrize("m,n,k", [(5, 64, 64), (130, 200, 128), (512, 1024, 256), (300, 28672 // 8, 512),
+                                   (16, 384, 512), (100, 4096, 1024), (128, 28672 // 8, 4096)])
 def test_swiglu_epilogue_equals_gemm_then_swiglu(m, n, k):
     """lhip_q8_0_matmul_bf16_swiglu == lhip_q8_0_matmul_bf16_f32out followed by lhip_swiglu_f32_bf16out on
     interleaved (gate, up) columns, bit for bit, on every tile the library would pick and on ragged edges."""
