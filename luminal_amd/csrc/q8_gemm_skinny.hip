@@ -5,12 +5,12 @@
 // (and, when the strips alone would not fill the chip, a slice of K) and streams it from HBM straight into
 // registers in matrix-core operand order:
 //
-//   * waves 0-3 ("compute") take 32 weight rows each, two 16-row blocks.  Lane (r, g) = (lane % 16, lane / 16)
-//     loads the 16 codes k = 64*group + 16*g .. +16 of row r with one 16-byte load: the A operands of two
+//   * the compute waves (four of 32 weight rows, or eight of 16 for at most 64 activation rows) work in blocks of
+//     16 weight rows.  Lane (r, g) = (lane % 16, lane / 16) loads the 16 codes k = 64*group + 16*g .. +16 of row r with one 16-byte load: the A operands of two
 //     v_mfma_f32_16x16x32_bf16 steps, whose k slots (g, e) are taken to mean k = 16*g + 8*step + e.  Eight groups
 //     (512 k) per row block are in flight per wave, reloaded in place as they are consumed; the codes are
 //     dequantised (q * d rounded to bf16, as in q8_gemm.hip) one group ahead of their MFMAs, in between them.
-//   * waves 4-7 ("loaders") stage the activations for all four compute waves: (16*MT) x (64*G) tiles of x go
+//   * four more waves ("loaders") stage the activations for all the compute waves: (16*MT) x (64*G) tiles of x go
 //     through their registers into one of three LDS buffers, two tiles ahead, one barrier per tile.  The compute
 //     waves never wait for an activation load, so their in-order load counter only ever sees the weight stream.
 //     In LDS a tile is G panels of 64 k, a row of a panel 128 bytes at pitch 160 (free of bank conflicts for the
@@ -96,16 +96,17 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
     }
 }
 
-// grid (strips of 128 weight rows, K slices); 512 threads.  K % 512 == 0, N % 4 == 0, M <= 16 * MT.
+// grid (strips of 128 weight rows, K slices); 8 / RB compute waves of RB row blocks each and four loader waves.  K % 512 == 0, N % 4 == 0, M <= 16 * MT.
 // A slice is `slice_groups` groups of 64 k (a multiple of 8); the last may be shorter (also a multiple of 8).
 // RING = groups in flight per wave and row block (8 or 16); a slice is a multiple of RING groups.
-template <int MT, int OUT, int RING>
-__global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
+template <int MT, int OUT, int RING, int RB>
+__global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
                                                              const __bf16 *__restrict__ x, void *__restrict__ y,
                                                              float *__restrict__ part, int M, int N, int K,
                                                              int slice_groups) {
     using S = SkShape<MT>;
     constexpr int G = S::G;
+    constexpr int CW = 8 / RB;  // compute waves, RB blocks of 16 weight rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -120,9 +121,9 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
     // same activation tile at the same time is worth more (57 against 64 us at 128 rows).
     const int rot = MT <= 2 ? (strip % (n_groups / RING)) * RING : 0;
 
-    if (wave >= 4) {
+    if (wave >= CW) {
         // ---------------- loaders: x tiles -> LDS, two tiles ahead of the compute waves
-        const int lt = tid - 256;
+        const int lt = tid - CW * 64;
         const __bf16 *src[S::CH];
         int dst[S::CH];
 #pragma unroll
@@ -170,11 +171,11 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
 
     // ---------------- compute waves
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = strip * kSkRows + wave * 32;
-    const int8_t *a_ptr[2];
-    const __half *d_ptr[2];
+    const int n0 = strip * kSkRows + wave * (16 * RB);
+    const int8_t *a_ptr[RB];
+    const __half *d_ptr[RB];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
         const int row = min(n0 + rb * 16 + r, N - 1);
         a_ptr[rb] = qs + static_cast<size_t>(row) * K + static_cast<size_t>(g_begin) * 64 + 16 * g;
         d_ptr[rb] = ds + static_cast<size_t>(row) * (K >> 5) + static_cast<size_t>(g_begin) * 2;
@@ -182,13 +183,13 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
     const int d_shift = (g >> 1) * 16;  // a lane's 16 codes lie in block 2*group + g/2
     const int n_rounds = n_groups >> 2;
 
-    sk_u32x4 a_reg[RING][2], d_reg[RING / 4][2];
+    sk_u32x4 a_reg[RING][RB], d_reg[RING / 4][RB];
     auto load_a = [&](int u, int group) __attribute__((always_inline)) {
         int gg = min(group, n_groups - 1) + rot;
         if (gg >= n_groups) gg -= n_groups;
         const size_t off = static_cast<size_t>(gg) * 64;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
             a_reg[u][rb] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4 *>(a_ptr[rb] + off));
     };
     auto load_d = [&](int set, int round) __attribute__((always_inline)) {
@@ -196,12 +197,12 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
         if (rr >= n_rounds) rr -= n_rounds;
         const size_t off = static_cast<size_t>(rr) * 8;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) d_reg[set][rb] = *reinterpret_cast<const sk_u32x4 *>(d_ptr[rb] + off);
+        for (int rb = 0; rb < RB; ++rb) d_reg[set][rb] = *reinterpret_cast<const sk_u32x4 *>(d_ptr[rb] + off);
     };
     // Dequantisation of ring slot `un` in sixteen pieces of two codes: piece p belongs to row block p / 8,
     // step (p / 4) % 2, dword p / 2 of the lane's four, half p % 2.
-    float d_next[2], off_next[2];
-    auto dequant_piece = [&](sk_u32x4 (&to)[2][2], int un, int p) __attribute__((always_inline)) {
+    float d_next[RB], off_next[RB];
+    auto dequant_piece = [&](sk_u32x4 (&to)[RB][2], int un, int p) __attribute__((always_inline)) {
         const int rb = p >> 3, dw = (p >> 1) & 3;
         // Opaque to the optimiser: keeps the unpacking here, at its use, instead of next to the load
         asm volatile("" : "+v"(a_reg[un][rb]));
@@ -222,9 +223,9 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
         if ((u & 3) == 3) load_d(u >> 2, u >> 2);
     }
 
-    sk_f32x4 acc[2][MT];
+    sk_f32x4 acc[RB][MT];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int cb = 0; cb < MT; ++cb) acc[rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -236,10 +237,10 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
     auto b_read = [&](const unsigned char *xb, int i) __attribute__((always_inline)) {
         return *reinterpret_cast<const sk_bf16x8 *>(xb + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
     };
-    sk_u32x4 af[2][2];  // [row block][step] of the group being multiplied, as packed bf16
+    sk_u32x4 af[RB][2];  // [row block][step] of the group being multiplied, as packed bf16
     sk_bf16x8 bw[W];
 #pragma unroll
-    for (int p = 0; p < 16; ++p) dequant_piece(af, 0, p);
+    for (int p = 0; p < 8 * RB; ++p) dequant_piece(af, 0, p);
     const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
     __syncthreads();  // tiles 0 and 1 are staged
 #pragma unroll
@@ -253,16 +254,16 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
             const int gl = R * 4 + u;
             const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
             const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
-            sk_u32x4 af_next[2][2];
+            sk_u32x4 af_next[RB][2];
             sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
                 const sk_bf16x8 b = bw[i % W];
                 bw[i % W] = i + W < UNITS ? b_read(xb_cur, i + W) : b_read(xb_next, i + W - UNITS);
-                sk_static_for<16>([&](auto pc) __attribute__((always_inline)) {
+                sk_static_for<8 * RB>([&](auto pc) __attribute__((always_inline)) {
                     constexpr int p = decltype(pc)::value;
-                    if constexpr (p * UNITS / 16 == i) {
+                    if constexpr (p * UNITS / (8 * RB) == i) {
                         dequant_piece(af_next, un, p);
-                        if constexpr (p == 15 && (un & 3) == 3) {
+                        if constexpr (p == 8 * RB - 1 && (un & 3) == 3) {
                             // the four groups of this round are unpacked: request the round after next, 256
                             // consecutive bytes of every row back to back
                             sk_static_for<4>([&](auto qc) __attribute__((always_inline)) {
@@ -274,13 +275,13 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
                     }
                 });
 #pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
+                for (int rb = 0; rb < RB; ++rb)
                     acc[rb][i % MT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[rb][i / MT]), b,
                                                                               acc[rb][i % MT], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             });
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
+            for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
                 for (int st = 0; st < 2; ++st) af[rb][st] = af_next[rb][st];
             xb_cur = xb_next;
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(512) void q8_gemm_skinny_kernel(const int8_t *__res
 
     // ---------------- lane (r, g) holds activation row 16*cb + r and weight rows n0 + 16*rb + 4*g .. +4
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
         const int n = n0 + rb * 16 + 4 * g;
         if (n >= N) continue;  // N % 4 == 0: the four rows are in or out together
 #pragma unroll
@@ -347,16 +348,16 @@ bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y) {
     return m >= 1 && m <= 128 && k % kSkUnit == 0 && n % 4 == 0 && aligned(y, out == kSkOutF32 ? 16 : (out == kSkOutBf16 ? 8 : 4));
 }
 
-template <int MT, int OUT, int RING>
+template <int MT, int OUT, int RING, int RB>
 static lhip_status sk_launch_r(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
                                int k, int splits, int slice_groups, hipStream_t s) {
-    auto kern = q8_gemm_skinny_kernel<MT, OUT, RING>;
+    auto kern = q8_gemm_skinny_kernel<MT, OUT, RING, RB>;
     constexpr size_t lds_bytes = SkShape<MT>::LDS;
     if (lds_bytes > 64 * 1024)  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits)),
-                       dim3(512), lds_bytes, s, qs, ds, x, y, part, m, n, k, slice_groups);
+                       dim3((8 / RB + 4) * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, slice_groups);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
@@ -365,7 +366,10 @@ template <int MT, int OUT>
 static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
                                int k, int splits, hipStream_t s) {
     const int units = k / kSkUnit, per = (units + splits - 1) / splits;
-    return sk_launch_r<MT, OUT, 8>(qs, ds, x, y, part, m, n, k, splits, per * 8, s);
+    // Up to 64 activation rows: eight compute waves of 16 weight rows, two per SIMD, so that one's waits sit under
+    // the other's instructions (36.5 -> 34 us on 28672 x 4096 at 16 rows, 173 -> 156 us on lm_head).  At 128 rows the
+    // B operand reads per MFMA double that way and four waves of 32 rows are faster (58 against 62 us).
+    return sk_launch_r<MT, OUT, 8, (MT >= 8 ? 2 : 1)>(qs, ds, x, y, part, m, n, k, splits, per * 8, s);
 }
 
 template <int MT>
