@@ -34,6 +34,11 @@ HBM_PEAK_GBS = 8000.0
 # committed rocprofv3 counter runs (FETCH_SIZE scaled by the copy-kernel factor
 # 2.0, plus WRITE_SIZE); None until measured.
 TRAFFIC_PER_LAUNCH = 138310222
+# The same for the dominant kernel of the prefill GEMM set (gate/up 14336 x 4096 at M = 2048: FETCH_SIZE
+# 173 100 KiB x 2.0 + WRITE_SIZE 60 045 KiB) and for the two grouped GEMMs of the MoE layer at T = 64
+# (FETCH_SIZE 158 755 + 82 880 KiB, x 2.0; the layer's other kernels move under 2 MiB).
+GEMM_TRAFFIC_PER_LAUNCH = (2 * 173100 + 60045) * 1024
+MOE_T64_TRAFFIC = 2 * (158755 + 82880) * 1024
 
 
 def parse():
@@ -205,7 +210,8 @@ def bench_prefill_gemm(args):
         "per_shape": per,
         "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true, __bf16> (gate/up, M=2048)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_us": round(us, 1)}}))
+                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_TRAFFIC_PER_LAUNCH,
+                     "avg_launch_us": round(us, 1)}}))
 
 
 def bench_moe(args):
@@ -289,7 +295,7 @@ def bench_moe(args):
         "per_tokens": per,
         "roofline": {"bound": "hbm", "kernel": "whole layer at T=64 (plan, quantise, 2 grouped GEMMs, combine)",
                      "achieved": t64["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": t64["frac_hbm"],
-                     "traffic": None}}))
+                     "traffic": MOE_T64_TRAFFIC}}))
 
 
 def llama_decode(torch):
