@@ -167,7 +167,11 @@ lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_d
  * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
  * K % 128 == 0, else LHIP_ERR_UNSUPPORTED), 5 = the weight-streaming kernel for
  * m <= 128 described above (LHIP_ERR_UNSUPPORTED for shapes it does not cover),
- * 50 + S = the same with S slices of K (S clamped to K / 512). */
+ * 50 + S = the same with S slices of K (S clamped to K / 512), 120 + S = the 256x128
+ * tile over S slices of K with the partial sums in the same scratch array (2 <= S <= 16,
+ * K / 64 / S a whole multiple of 4, S * m * N <= 8 Mi; what the plain entry
+ * points take for K >= 8192 when whole-K tiles would leave most of the chip idle, so
+ * the note on overlapping calls above applies to those shapes too). */
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream);
 

@@ -52,8 +52,8 @@ template <int BM, int BN, int WM, int WN, int D, bool PIPE = false, typename Out
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
                                                                    const __half *__restrict__ ds,
                                                                    const __bf16 *__restrict__ x,
-                                                                   OutT *__restrict__ y, int M, int N, int K,
-                                                                   int m_tiles, int n_tiles, int swiglu) {
+                                                                   OutT *__restrict__ y_all, int M, int N, int K,
+                                                                   int m_tiles, int n_tiles, int swiglu, int kt_slice) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 MFMA tiles per wave
@@ -81,6 +81,11 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int nblk = K >> 5;
+    // kt_slice > 0: blockIdx.y takes K tiles [kt0, kt0 + KT) and writes its f32 partial result to plane blockIdx.y
+    // of y (the caller adds the planes); 0: all of K.
+    const int kt0 = kt_slice > 0 ? static_cast<int>(blockIdx.y) * kt_slice : 0;
+    const int KT = kt_slice > 0 ? min(kt_slice, K / kBK - kt0) : K / kBK;
+    OutT *__restrict__ y = y_all + (kt_slice > 0 ? static_cast<size_t>(blockIdx.y) * M * N : 0);
 
     // Per-thread global sources (rows past the edge re-read the last row; their results are not stored).
     const __bf16 *a_src[A_CHUNKS];
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     for (int i = 0; i < A_CHUNKS; ++i) {
         const int c = tid + i * T;
         const int row = c >> 3, col = (c & 7) * 8;
-        a_src[i] = x + static_cast<size_t>(min(m0 + row, M - 1)) * K + col;
+        a_src[i] = x + static_cast<size_t>(min(m0 + row, M - 1)) * K + col + kt0 * kBK;
         a_dst[i] = row * kRowBytes + col * 2;
     }
     const int8_t *b_src[B_CHUNKS];
@@ -101,8 +106,8 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         const int c = tid + i * T;
         const int row = c >> 2, q16 = c & 3;
         const int grow = min(n0 + row, N - 1);
-        b_src[i] = qs + static_cast<size_t>(grow) * K + q16 * 16;
-        d_src[i] = reinterpret_cast<const uint32_t *>(ds + static_cast<size_t>(grow) * nblk);
+        b_src[i] = qs + static_cast<size_t>(grow) * K + q16 * 16 + kt0 * kBK;
+        d_src[i] = reinterpret_cast<const uint32_t *>(ds + static_cast<size_t>(grow) * nblk) + kt0;
         d_shift[i] = (q16 >> 1) * 16;
         b_dst[i] = row * kRowBytes + q16 * 32;
     }
@@ -110,7 +115,6 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     // D register sets: tile t lives in set t % D from its load until it is written to LDS.
     gu32x4 a_reg[D][A_CHUNKS], b_reg[D][B_CHUNKS];
     uint32_t d_reg[D][B_CHUNKS];  // both f16 scale codes of the tile
-    const int KT = K / kBK;
     // part p of P: the p-th share of the thread's chunks (P = 1: everything), the same split as store_tile's.
     auto load_tile = [&](int set, int kt, int p = 0, int P = 1) {
         const int k0 = min(kt, KT - 1) * kBK;  // tiles past the end re-read the last one (never used)
@@ -292,12 +296,15 @@ enum { kOutBf16 = 0, kOutF32 = 1, kOutSwiglu = 2 };
 bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y);
 lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
                                   int out, int splits, hipStream_t s);
+float *q8_gemm_scratch(size_t *floats);  // the library's partial-sum array on the current device
+lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s);
 constexpr int kTileSkinny = 5;        // K slices chosen by the library
 constexpr int kTileSkinnySplit = 50;  // + number of K slices
+constexpr int kTileSliced = 120;      // + number of K slices: the 256x128 tile over slices of K, then a reduction
 
 template <int BM, int BN, int WM, int WN, int D, bool PIPE, typename OutT>
 static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
-                                 int swiglu, hipStream_t s) {
+                                 int swiglu, hipStream_t s, int slices = 1) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
@@ -307,8 +314,10 @@ static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void 
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     }
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad)), dim3(WM * WN * 64), lds_bytes, s, qs,
-                       ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m, n, k, m_tiles, n_tiles, swiglu);
+    const int kt_slice = slices > 1 ? (k / kBK + slices - 1) / slices : 0;
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad), static_cast<unsigned>(slices)),
+                       dim3(WM * WN * 64), lds_bytes, s, qs, ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m,
+                       n, k, m_tiles, n_tiles, swiglu, kt_slice);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
@@ -342,6 +351,21 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
         if (!q8_gemm_skinny_supports(mi, ni, ki, out, y_dev)) return LHIP_ERR_UNSUPPORTED;
         return q8_gemm_skinny_launch(qs, ds, x_dev, y_dev, mi, ni, ki, out, tile == kTileSkinny ? 0 : tile - kTileSkinnySplit, s);
     }
+    if (tile > kTileSliced && tile <= kTileSliced + 16) {
+        // Few output tiles and a long K (the down projection of a 512-token prompt: 64 tiles of 256x128): slices of K
+        // fill the chip, f32 partial planes go to the scratch array and are added in slice order.
+        const int slices = tile - kTileSliced;
+        const int kt = ki / kBK;
+        size_t cap = 0;
+        float *part = q8_gemm_scratch(&cap);
+        if (!part) return LHIP_ERR_HIP;
+        if (slices < 2 || kt % slices != 0 || (kt / slices) % 4 != 0 || static_cast<size_t>(slices) * mi * ni > cap ||
+            ni % 4 != 0 || !aligned(y_dev, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4)))
+            return LHIP_ERR_UNSUPPORTED;
+        if (lhip_status st = launch_gemm_t<256, 128, 4, 2, 4, true, float>(qs, ds, x_dev, part, mi, ni, ki, 0, s, slices))
+            return st;
+        return q8_gemm_reduce_launch(part, y_dev, mi, ni, slices, out, s);
+    }
     switch (tile) {
         case 0: LHIP_TILE(256, 128, 4, 2);
         case 1: LHIP_TILE(128, 128, 2, 2);
@@ -365,6 +389,16 @@ static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *
     // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
     // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
     auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    // Long K and few 256x128 tiles: slices of K until the chip is full, when the partial planes (written and read
+    // once more: 4 * slices / K bytes per flop) stay small next to the product.  Measured for 4096 x 14336: 102 -> 55 us
+    // at 256 rows (8 slices), 115 -> 83 us at 512 (4), 236 -> 142 us at 1024 (2); no gain for K = 4096.
+    if (m > 128 && k >= 8192 && n % 4 == 0 && aligned(y, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4))) {
+        const int64_t b0 = blocks(256, 128), kt = k / kBK;
+        for (int slices = 8; slices >= 2; slices >>= 1)
+            if (b0 * slices <= 256 && kt % slices == 0 && (kt / slices) % 4 == 0 &&
+                static_cast<size_t>(slices) * m * n <= (size_t{8} << 20))
+                return kTileSliced + slices;
+    }
     int tile = 3;
     if (m > 128 && k % (kBK * 2) == 0 && blocks(256, 256) >= 192) tile = 4;
     else if (m > 128 && blocks(256, 128) >= 192) tile = 0;

@@ -332,6 +332,24 @@ static float *sk_scratch_ptr() {
     return p;
 }
 
+float *q8_gemm_scratch(size_t *floats) {
+    *floats = kSkScratchFloats;
+    return sk_scratch_ptr();
+}
+
+// Adds `slices` f32 planes of (m, n) in order and writes the output form (as the GEMM epilogues: bf16, f32, SwiGLU).
+lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s) {
+    const size_t quads = static_cast<size_t>(m) * (n >> 2);
+    const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
+    switch (out) {
+        case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
+        case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
+        default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
+    }
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
 // K slices for a product: enough workgroups for the 256 CUs, slices of whole 512-k units, partial sums within the
 // scratch array.
 int q8_gemm_skinny_splits(int m, int n, int k) {
@@ -406,15 +424,7 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
     else if (m <= 64) st = sk_launch_mt<4>(out, qs, ds, x, y, part, m, n, k, splits, s);
     else st = sk_launch_mt<8>(out, qs, ds, x, y, part, m, n, k, splits, s);
     if (st != LHIP_OK || splits == 1) return st;
-    const size_t quads = static_cast<size_t>(m) * (n >> 2);
-    const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
-    switch (out) {
-        case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
-        case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
-        default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, splits); break;
-    }
-    LHIP_CHECK_LAUNCH();
-    return LHIP_OK;
+    return q8_gemm_reduce_launch(part, y, m, n, splits, out, s);
 }
 
 }  // namespace lhip

@@ -214,6 +214,43 @@ def test_weight_streaming_gemm_output_forms(oracle):
         assert torch.equal(act.view(torch.int16), want.view(torch.int16))
 
 
+def test_k_sliced_tiled_gemm(oracle):
+    """Long K and few output tiles: the 256x128 tile runs over slices of K (tile id 120 + slices) and the f32 planes
+    are added in slice order.  Against the f64 product on the f32 output; bf16 and SwiGLU outputs are that result's
+    forms; the plain entry point picks the sliced form for such shapes (same bits) and two runs agree."""
+    lib = capi.load_library()
+    st = torch.cuda.current_stream().cuda_stream
+    m, n, k = 300, 512, 8192
+    qs, d = synth.q8_0_random(n, k, seed=41)
+    xf, bits = bf16_activations(oracle, m, k, seed=42)
+    w = upload(qs, d)
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y32 = torch.full((m, n), float("nan"), device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st), "f32out")
+    elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+    auto = run(w, bits)
+    assert np.array_equal(auto, y32.to(torch.bfloat16).float().cpu().numpy())
+    assert np.array_equal(auto, run(w, bits, 120 + 8)) and np.array_equal(auto, run(w, bits))
+    ref = run(w, bits, 0)  # the same tile over all of K: another order of the f32 additions
+    for tile in (120 + 2, 120 + 4):
+        y = run(w, bits, tile)
+        step = np.abs(ref) * 2.0 ** -7 + 1e-4 * float(np.sqrt(np.mean(ref * ref)))
+        assert np.all(np.abs(y - ref) <= step) and np.mean(y == ref) > 0.98, tile
+    act = torch.empty(m, n // 2, device=DEV, dtype=torch.bfloat16)
+    want = torch.empty_like(act)
+    capi.check(lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), act.data_ptr(), m, n, k, st), "swiglu")
+    capi.check(lib.lhip_swiglu_f32_bf16out(y32.data_ptr(), want.data_ptr(), m, n // 2, 1, st), "swiglu of f32")
+    torch.cuda.synchronize()
+    assert torch.equal(act.view(torch.int16), want.view(torch.int16))
+    # slices must divide K into whole rounds of four 64-wide tiles
+    yd = torch.empty(m, n, device=DEV, dtype=torch.bfloat16)
+    assert lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), x.data_ptr(), yd.data_ptr(), m, n, k, 120 + 3,
+                                         st) == capi.LHIP_ERR_UNSUPPORTED
+    assert lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), x.data_ptr(), yd.data_ptr(), m, n, k, 120 + 32,
+                                         st) == capi.LHIP_ERR_UNSUPPORTED
+
+
 def test_gemm_argument_errors():
     lib = capi.load_library()
     w = upload(*synth.q8_0_random(64, 96, seed=1))
