@@ -190,7 +190,9 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         const size_t off = static_cast<size_t>(gg) * 64;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
-            a_reg[u][rb] = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4 *>(a_ptr[rb] + off));
+            // plain, not non-temporal: an instruction takes half a 128-byte line of each of its 16 rows and the next
+            // group's takes the other half; kept in L1 the line is fetched once (30 -> 23 us for one 128 x 4096 strip)
+            a_reg[u][rb] = *reinterpret_cast<const sk_u32x4 *>(a_ptr[rb] + off);
     };
     auto load_d = [&](int set, int round) __attribute__((always_inline)) {
         int rr = min(round, n_rounds - 1) + rot / 4;
