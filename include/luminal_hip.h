@@ -284,7 +284,9 @@ lhip_status lhip_attention_f32_bf16out(const float *qkv_dev, const float *k_cach
                                        int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
 /* Prompt attention with bf16 matrix-core operands: Q / sqrt(head_dim), K, V and the soft-max weights are rounded to
  * bf16 for the matrix instructions, scores, soft-max and sums stay f32, output bf16 — for a prompt pass whose
- * attention output feeds a bf16 GEMM (results within the 1e-2 bar of the bf16 paths, not the 2e-3 of the f32 ones).
+ * attention output feeds a bf16 GEMM.  Five roundings of unit roundoff 2^-8 enter, one of them through the soft-max:
+ * every output is within 2e-2 * sum_j p_j |v_j| of the exact softmax(QK)V (the sum before cancellation), against 1e-5
+ * for the f32-operand kernel behind lhip_attention_f32_bf16out.
  * No counterpart in the reference (model.rs:112-139 builds attention from f16 primitives).  Built for head_dim 64 or
  * 128 and q_heads / kv_heads in {2, 4, 8}: LHIP_ERR_UNSUPPORTED otherwise (use lhip_attention_f32_bf16out). */
 lhip_status lhip_attention_bf16(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,

@@ -67,8 +67,8 @@ struct SkShape {
 
 // Two packed int8 (half `h` of a dword) -> two bf16 of q * d, packed.  A byte is converted as unsigned (one
 // instruction), so the dword arrives biased by 128 per byte (w = q ^ 0x80808080) and the fma takes the bias out
-// again: (q + 128) * d - 128 * d is exact in an fma because q * d has at most 19 significant bits, and the value
-// rounded to bf16 is that of q * d itself.
+// again: for a finite scale (q + 128) * d - 128 * d is exact in an fma because q * d has at most 19 significant bits,
+// and the value rounded to bf16 is that of q * d itself (an infinite scale gives NaN here, not +-inf).
 __device__ __forceinline__ uint32_t sk_dequant2(uint32_t w, int h, float d, float off) {
     typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
     const float lo = fmaf(static_cast<float>((w >> (16 * h)) & 0xffu), d, off);
