@@ -100,7 +100,8 @@ def test_reference_metal_matmul_case(oracle):
     assert np.max(np.abs(y - truth) / np.maximum(np.abs(truth), 1.0)) < 2.0 ** -8
 
 
-@pytest.mark.parametrize("name,m", [("q", 128), ("k", 512), ("down", 128), ("gate", 2048)])
+@pytest.mark.parametrize("name,m", [("q", 128), ("k", 512), ("down", 128), ("gate", 2048), ("gate", 40), ("lm_head", 100),
+                                    ("down", 512)])
 def test_full_size_prefill_shapes(oracle, name, m):
     """The Llama-3-8B prefill shapes (M in {128, 512, 2048}); the oracle runs on a sample of weight rows."""
     n, k = synth.LLAMA3_8B_PROJ[name]
