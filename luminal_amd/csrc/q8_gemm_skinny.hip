@@ -33,7 +33,7 @@ typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float sk_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
 
-enum { kSkOutBf16 = 0, kSkOutF32 = 1, kSkOutSwiglu = 2, kSkOutPartial = 3 };  // first three as in q8_gemm.hip
+enum { kSkOutBf16 = 0, kSkOutF32 = 1, kSkOutSwiglu = 2, kSkOutPartial = 3, kSkOutF16 = 4 };  // first three as in q8_gemm.hip
 
 constexpr int kSkRows = 128;    // weight rows per workgroup
 constexpr int kSkPitch = 160;   // bytes per activation row of a panel in LDS
@@ -54,12 +54,17 @@ __device__ __forceinline__ void sk_static_for(F &&f) {
     sk_static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
 }
 
-template <int MT>
+// SPLIT: f32 / f16 activations held as three bf16 planes (see q8_gemm_skinny_kernel), at most 64 rows, 64 k per
+// panel row as before but fewer panels per tile.
+template <int MT, bool SPLIT = false>
 struct SkShape {
-    static constexpr int G = MT >= 8 ? 2 : 4;  // groups per activation tile; a slice is an even number of tiles
+    static_assert(!SPLIT || MT <= 4, "the split form takes at most 64 activation rows");
+    static constexpr int G = SPLIT ? (MT >= 4 ? 1 : (MT == 2 ? 2 : 4))
+                                   : (MT >= 8 ? 2 : 4);  // groups per activation tile; a slice is an even number of tiles
     static constexpr int PANEL = 16 * MT * kSkPitch;
-    static constexpr int STAGE = G * PANEL;
-    static constexpr int CHUNKS = 16 * MT * G * 8;             // 16-byte pieces per tile
+    static constexpr int PLANE = G * PANEL;
+    static constexpr int STAGE = (SPLIT ? 3 : 1) * PLANE;
+    static constexpr int CHUNKS = 16 * MT * G * 8;             // pieces of 8 k per tile
     static constexpr int CH = CHUNKS / 256;                    // per loader thread
     static_assert(CHUNKS % 256 == 0 && 8 % G == 0, "tile split");
     static constexpr size_t LDS = static_cast<size_t>(kSkStages) * STAGE;
@@ -77,6 +82,26 @@ __device__ __forceinline__ uint32_t sk_dequant2(uint32_t w, int h, float d, floa
     return __builtin_bit_cast(uint32_t, pk);
 }
 
+// Two f32 -> three packed bf16 pairs whose sums are the two values exactly: limb[0] the bf16 roundings, limb[1]
+// the roundings of what that left, limb[2] of what is left then (8 + 8 + 8 significant bits cover an f32).
+__device__ __forceinline__ void sk_split2(float a, float b, uint32_t (&limb)[3]) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        const bf16x2 h = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
+        limb[l] = __builtin_bit_cast(uint32_t, h);
+        a -= __uint_as_float(limb[l] << 16);
+        b -= __uint_as_float(limb[l] & 0xffff0000u);
+    }
+}
+
+// The same two codes as the three limbs of q * d.
+__device__ __forceinline__ void sk_dequant2_split(uint32_t w, int h, float d, float off, uint32_t (&limb)[3]) {
+    const float lo = fmaf(static_cast<float>((w >> (16 * h)) & 0xffu), d, off);
+    const float hi = fmaf(static_cast<float>((w >> (16 * h + 8)) & 0xffu), d, off);
+    sk_split2(lo, hi, limb);
+}
+
 // One output form for four consecutive weight rows n .. n+3 of activation row m.
 template <int OUT>
 __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M, int N, int m, int n, sk_f32x4 v) {
@@ -89,6 +114,11 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
         const bf16x4 w = {static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1]), static_cast<__bf16>(v[2]),
                           static_cast<__bf16>(v[3])};
         *reinterpret_cast<bf16x4 *>(static_cast<__bf16 *>(y) + static_cast<size_t>(m) * N + n) = w;
+    } else if constexpr (OUT == kSkOutF16) {
+        typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+        const f16x4 w = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1]), static_cast<_Float16>(v[2]),
+                         static_cast<_Float16>(v[3])};
+        *reinterpret_cast<f16x4 *>(static_cast<_Float16 *>(y) + static_cast<size_t>(m) * N + n) = w;
     } else {  // rows are (gate, up) pairs
         typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
         const bf16x2 w = {static_cast<__bf16>(swiglu_value(v[0], v[1])), static_cast<__bf16>(swiglu_value(v[2], v[3]))};
@@ -96,15 +126,25 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
     }
 }
 
-// grid (strips of 128 weight rows, K slices); 8 / RB compute waves of RB row blocks each and four loader waves.  K % 512 == 0, N % 4 == 0, M <= 16 * MT.
+// grid (strips of 128 weight rows, K slices); 8 / RB compute waves of RB row blocks each and four loader waves.
+// K % 512 == 0, N % 4 == 0, M <= 16 * MT.
 // A slice is `slice_groups` groups of 64 k (a multiple of 8); the last may be shorter (also a multiple of 8).
-// RING = groups in flight per wave and row block (8 or 16); a slice is a multiple of RING groups.
-template <int MT, int OUT, int RING, int RB>
+// RING = groups in flight per wave and row block; a slice is a multiple of RING groups.
+//
+// XT = __bf16: the product as described above.  XT = float or __half ("split"): the f32-exact form behind the
+// f32 / f16 matmul operators for more than a few activation rows.  Both operands are carried as three bf16 limbs
+// whose sum is the f32 value exactly (x = x0 + x1 + x2, likewise q * d, which has 19 significant bits), and six
+// products are accumulated per step, smallest first: x0*w2 + x2*w0 + x1*w1 + x1*w0 + x0*w1 + x0*w0.  Each is
+// exact in f32; what is dropped (x1*w2, x2*w1, x2*w2) is below 2^-24 of a term, so the result differs from the
+// matvec kernels' only by the order of the f32 additions.  The loaders split x on its way into LDS (three planes
+// per tile), the compute waves split q * d as they unpack it.  At most 64 activation rows (MT <= 4).
+template <int MT, int OUT, int RING, int RB, typename XT = __bf16>
 __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
-                                                             const __bf16 *__restrict__ x, void *__restrict__ y,
+                                                             const XT *__restrict__ x, void *__restrict__ y,
                                                              float *__restrict__ part, int M, int N, int K,
                                                              int slice_groups) {
-    using S = SkShape<MT>;
+    constexpr bool SPLIT = !std::is_same<XT, __bf16>::value;
+    using S = SkShape<MT, SPLIT>;
     constexpr int G = S::G;
     constexpr int CW = 8 / RB;  // compute waves, RB blocks of 16 weight rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
@@ -124,7 +164,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     if (wave >= CW) {
         // ---------------- loaders: x tiles -> LDS, two tiles ahead of the compute waves
         const int lt = tid - CW * 64;
-        const __bf16 *src[S::CH];
+        const XT *src[S::CH];
         int dst[S::CH];
 #pragma unroll
         for (int i = 0; i < S::CH; ++i) {
@@ -134,18 +174,46 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             src[i] = x + static_cast<size_t>(min(m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
             dst[i] = panel * S::PANEL + m * kSkPitch + ((jj >> 1) + 4 * (jj & 1)) * 16;
         }
-        sk_u32x4 xr[2][S::CH];
+        constexpr int XL = sizeof(XT) == 4 ? 2 : 1;  // 16-byte loads per piece of 8 k
+        sk_u32x4 xr[2][S::CH][XL];
         auto load_x = [&](int slot, int t) __attribute__((always_inline)) {
             int tt = min(t, n_tiles - 1) + rot / G;  // past the end: re-read, never used
             if (tt >= n_tiles) tt -= n_tiles;
             const size_t off = static_cast<size_t>(tt) * (G * 64);
 #pragma unroll
-            for (int i = 0; i < S::CH; ++i) xr[slot][i] = *reinterpret_cast<const sk_u32x4 *>(src[i] + off);
+            for (int i = 0; i < S::CH; ++i)
+#pragma unroll
+                for (int l = 0; l < XL; ++l)
+                    xr[slot][i][l] = reinterpret_cast<const sk_u32x4 *>(src[i] + off)[l];
         };
         auto store_x = [&](int slot, int stage) __attribute__((always_inline)) {
             unsigned char *base = sk_lds + stage * S::STAGE;
 #pragma unroll
-            for (int i = 0; i < S::CH; ++i) *reinterpret_cast<sk_u32x4 *>(base + dst[i]) = xr[slot][i];
+            for (int i = 0; i < S::CH; ++i) {
+                if constexpr (!SPLIT) {
+                    *reinterpret_cast<sk_u32x4 *>(base + dst[i]) = xr[slot][i][0];
+                } else {
+                    float v[8];
+                    if constexpr (sizeof(XT) == 4) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[e] = __uint_as_float(xr[slot][i][e >> 2][e & 3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            v[e] = __half2float(__ushort_as_half(static_cast<unsigned short>(xr[slot][i][0][e >> 1] >> (16 * (e & 1)))));
+                    }
+                    sk_u32x4 limbs[3];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        uint32_t l3[3];
+                        sk_split2(v[2 * e], v[2 * e + 1], l3);
+#pragma unroll
+                        for (int l = 0; l < 3; ++l) limbs[l][e] = l3[l];
+                    }
+#pragma unroll
+                    for (int l = 0; l < 3; ++l) *reinterpret_cast<sk_u32x4 *>(base + l * S::PLANE + dst[i]) = limbs[l];
+                }
+            }
         };
         load_x(0, 0);
         load_x(1, 1);
@@ -204,7 +272,8 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     // Dequantisation of ring slot `un` in sixteen pieces of two codes: piece p belongs to row block p / 8,
     // step (p / 4) % 2, dword p / 2 of the lane's four, half p % 2.
     float d_next[RB], off_next[RB];
-    auto dequant_piece = [&](sk_u32x4 (&to)[RB][2], int un, int p) __attribute__((always_inline)) {
+    constexpr int P = SPLIT ? 3 : 1;  // operand planes: the bf16 value, or its three limbs
+    auto dequant_piece = [&](sk_u32x4 (&to)[P][RB][2], int un, int p) __attribute__((always_inline)) {
         const int rb = p >> 3, dw = (p >> 1) & 3;
         // Opaque to the optimiser: keeps the unpacking here, at its use, instead of next to the load
         asm volatile("" : "+v"(a_reg[un][rb]));
@@ -214,7 +283,15 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             off_next[rb] = -128.f * d_next[rb];
         }
         if ((p & 1) == 0) a_reg[un][rb][dw] ^= 0x80808080u;
-        to[rb][(p >> 2) & 1][(p >> 1) & 1 ? 2 + (p & 1) : (p & 1)] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
+        const int st = (p >> 2) & 1, e = (p >> 1) & 1 ? 2 + (p & 1) : (p & 1);
+        if constexpr (SPLIT) {
+            uint32_t l3[3];
+            sk_dequant2_split(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb], l3);
+#pragma unroll
+            for (int l = 0; l < 3; ++l) to[l][rb][st][e] = l3[l];
+        } else {
+            to[0][rb][st][e] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
+        }
     };
 
     // the loop reloads in the order a0 a1 a2 a3 d0 a4 a5 a6 a7 d1: the same order here, so the counted waits of the
@@ -225,28 +302,35 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         if ((u & 3) == 3) load_d(u >> 2, u >> 2);
     }
 
-    sk_f32x4 acc[RB][MT];
+    // Split form: the five small products of a step go to an accumulator of their own, so that their sum, 2^-8 of the
+    // main one, is rounded at its own scale and the main accumulator sees one addition per step, as in the plain form.
+    constexpr int NA = SPLIT ? 2 : 1;
+    sk_f32x4 acc[NA][RB][MT];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+    for (int a = 0; a < NA; ++a)
 #pragma unroll
-        for (int cb = 0; cb < MT; ++cb) acc[rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < MT; ++cb) acc[a][rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
 
     // A group is UNITS = 2 * MT units (step, column block): one B operand read and two MFMAs each.  W reads are
     // kept in flight, running ahead into the next group (whose tile was complete in LDS a barrier ago), and the
     // next group's dequantisation is dealt out over the units, so that LDS latency and VALU work sit under MFMAs.
     constexpr int UNITS = 2 * MT;
-    constexpr int W = UNITS < 4 ? UNITS : 4;
-    auto b_read = [&](const unsigned char *xb, int i) __attribute__((always_inline)) {
-        return *reinterpret_cast<const sk_bf16x8 *>(xb + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
+    constexpr int W = SPLIT ? 2 : (UNITS < 4 ? UNITS : 4);  // units of B operands in flight (P reads each)
+    auto b_read = [&](const unsigned char *xb, int i, int plane) __attribute__((always_inline)) {
+        return *reinterpret_cast<const sk_bf16x8 *>(xb + plane * S::PLANE + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
     };
-    sk_u32x4 af[RB][2];  // [row block][step] of the group being multiplied, as packed bf16
-    sk_bf16x8 bw[W];
+    sk_u32x4 af[P][RB][2];  // [plane][row block][step] of the group being multiplied, as packed bf16
+    sk_bf16x8 bw[W][P];
 #pragma unroll
     for (int p = 0; p < 8 * RB; ++p) dequant_piece(af, 0, p);
     const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
     __syncthreads();  // tiles 0 and 1 are staged
 #pragma unroll
-    for (int i = 0; i < W; ++i) bw[i] = b_read(xb_cur, i);
+    for (int i = 0; i < W; ++i)
+#pragma unroll
+        for (int pl = 0; pl < P; ++pl) bw[i][pl] = b_read(xb_cur, i, pl);
     int stage = 0;
     for (int R = 0; R < n_rounds; R += RING / 4) {
         sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
@@ -256,11 +340,15 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             const int gl = R * 4 + u;
             const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
             const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
-            sk_u32x4 af_next[RB][2];
+            sk_u32x4 af_next[P][RB][2];
             sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                const sk_bf16x8 b = bw[i % W];
-                bw[i % W] = i + W < UNITS ? b_read(xb_cur, i + W) : b_read(xb_next, i + W - UNITS);
+                sk_bf16x8 b[P];
+#pragma unroll
+                for (int pl = 0; pl < P; ++pl) {
+                    b[pl] = bw[i % W][pl];
+                    bw[i % W][pl] = i + W < UNITS ? b_read(xb_cur, i + W, pl) : b_read(xb_next, i + W - UNITS, pl);
+                }
                 sk_static_for<8 * RB>([&](auto pc) __attribute__((always_inline)) {
                     constexpr int p = decltype(pc)::value;
                     if constexpr (p * UNITS / (8 * RB) == i) {
@@ -277,15 +365,29 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                     }
                 });
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb)
-                    acc[rb][i % MT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[rb][i / MT]), b,
-                                                                              acc[rb][i % MT], 0, 0, 0);
+                for (int rb = 0; rb < RB; ++rb) {
+                    auto prod = [&](sk_f32x4 &c, int wl, int xl) __attribute__((always_inline)) {
+                        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[wl][rb][i / MT]), b[xl], c, 0, 0, 0);
+                    };
+                    if constexpr (SPLIT) {  // the small terms, smallest first
+                        sk_f32x4 c = acc[1][rb][i % MT];
+                        prod(c, 2, 0);
+                        prod(c, 0, 2);
+                        prod(c, 1, 1);
+                        prod(c, 0, 1);
+                        prod(c, 1, 0);
+                        acc[1][rb][i % MT] = c;
+                    }
+                    prod(acc[0][rb][i % MT], 0, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             });
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
+            for (int pl = 0; pl < P; ++pl)
 #pragma unroll
-                for (int st = 0; st < 2; ++st) af[rb][st] = af_next[rb][st];
+                for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                    for (int st = 0; st < 2; ++st) af[pl][rb][st] = af_next[pl][rb][st];
             xb_cur = xb_next;
             if constexpr (tile_ends) {
                 stage = stage_next;
@@ -302,7 +404,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
 #pragma unroll
         for (int cb = 0; cb < MT; ++cb) {
             const int m = cb * 16 + r;
-            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[rb][cb]);
+            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, SPLIT ? acc[0][rb][cb] + acc[NA - 1][rb][cb] : acc[0][rb][cb]);
         }
     }
 }
@@ -339,13 +441,14 @@ float *q8_gemm_scratch(size_t *floats) {
     return sk_scratch_ptr();
 }
 
-// Adds `slices` f32 planes of (m, n) in order and writes the output form (as the GEMM epilogues: bf16, f32, SwiGLU).
+// Adds `slices` f32 planes of (m, n) in order and writes the output form (as the GEMM epilogues: bf16, f32, f16, SwiGLU).
 lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s) {
     const size_t quads = static_cast<size_t>(m) * (n >> 2);
     const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
     switch (out) {
         case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
         case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
+        case kSkOutF16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF16>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
         default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
     }
     LHIP_CHECK_LAUNCH();
@@ -427,6 +530,71 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
     else st = sk_launch_mt<8>(out, qs, ds, x, y, part, m, n, k, splits, s);
     if (st != LHIP_OK || splits == 1) return st;
     return q8_gemm_reduce_launch(part, y, m, n, splits, out, s);
+}
+
+// ---- the f32-accurate ("split") form behind the f32 / f16 operators
+
+template <int MT, int OUT, typename XT>
+static lhip_status sk_launch_split_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
+                                     int k, int splits, hipStream_t s) {
+    auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, 1, XT>;
+    constexpr size_t lds_bytes = SkShape<MT, true>::LDS;
+    if (lds_bytes > 64 * 1024)
+        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(lds_bytes)));
+    const int units = k / kSkUnit, per = (units + splits - 1) / splits;
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits)),
+                       dim3(12 * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+template <typename XT, int OUT>
+static lhip_status sk_launch_split_rows(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
+                                        int k, int splits, hipStream_t s) {
+    if (splits > 1) {
+        if (m <= 16) return sk_launch_split_t<1, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
+        if (m <= 32) return sk_launch_split_t<2, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
+        return sk_launch_split_t<4, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
+    }
+    if (m <= 16) return sk_launch_split_t<1, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
+    if (m <= 32) return sk_launch_split_t<2, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
+    return sk_launch_split_t<4, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
+}
+
+bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16) {
+    return k % kSkUnit == 0 && n % 4 == 0 && aligned(x, 16) && aligned(y, f16 ? 8 : 16);
+}
+
+// y (m, N) = x (m, K) W^T for f32 or f16 activations and results, any m: 64 rows at a time, each pass streaming
+// the weights once.  `splits` = 0: chosen here.  The caller has checked q8_gemm_split_supports.
+lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void *x, void *y, int64_t m, int n, int k,
+                                 bool f16, int splits_arg, hipStream_t s) {
+    const int units = k / kSkUnit;
+    const size_t esz = f16 ? 2 : 4;
+    for (int64_t m0 = 0; m0 < m; m0 += 64) {
+        const int mc = static_cast<int>(m - m0 < 64 ? m - m0 : 64);
+        int splits = splits_arg > 0 ? splits_arg : q8_gemm_skinny_splits(mc, n, k);
+        if (splits > units) splits = units;
+        const int per = (units + splits - 1) / splits;
+        splits = (units + per - 1) / per;
+        while (splits > 1 && static_cast<size_t>(splits) * mc * n > kSkScratchFloats) --splits;
+        float *part = nullptr;
+        if (splits > 1) {
+            part = sk_scratch_ptr();
+            if (!part) return LHIP_ERR_HIP;
+        }
+        const auto *xc = static_cast<const unsigned char *>(x) + static_cast<size_t>(m0) * k * esz;
+        auto *yc = static_cast<unsigned char *>(y) + static_cast<size_t>(m0) * n * esz;
+        lhip_status st = f16 ? sk_launch_split_rows<__half, kSkOutF16>(qs, ds, reinterpret_cast<const __half *>(xc), yc, part,
+                                                                       mc, n, k, splits, s)
+                             : sk_launch_split_rows<float, kSkOutF32>(qs, ds, reinterpret_cast<const float *>(xc), yc, part,
+                                                                      mc, n, k, splits, s);
+        if (st != LHIP_OK) return st;
+        if (splits > 1)
+            if (lhip_status r = q8_gemm_reduce_launch(part, yc, mc, n, splits, f16 ? kSkOutF16 : kSkOutF32, s)) return r;
+    }
+    return LHIP_OK;
 }
 
 }  // namespace lhip
