@@ -1,4 +1,4 @@
-// Q8_0 weights x bf16 activations for 2..128 activation rows (short prompts, small batches).
+// Q8_0 weights x activations for up to 128 activation rows per pass (short prompts, small batches).
 //
 // With so few activation rows the product is bound by streaming the weights, not by the matrix cores, and the
 // 128/256-row tiles of q8_gemm.hip leave most of the chip idle.  Here a workgroup owns a strip of 128 weight rows
@@ -20,6 +20,9 @@
 // K slices write f32 partial tiles to a scratch array owned by the library (one per device, shared by every
 // call on it) and a second kernel adds them in slice order and applies the output form, so results do not depend
 // on timing.
+//
+// The same kernel with f32 or f16 activations is the f32-exact form of the f32 / f16 matmul operators for several
+// activation rows: three bf16 limbs per operand, six limb products per step (see the kernel's comment).
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
