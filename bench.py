@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode_projection_set",
-                    choices=["decode_projection_set", "prefill_gemm", "moe"],
+                    choices=["decode_projection_set", "prefill_gemm", "moe", "rows_f32"],
                     help="decode_projection_set (default, the headline metric), prefill_gemm (the Q8_0 prefill GEMM set), "
                          "moe (the MXFP4 expert layer)")
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
@@ -138,6 +138,74 @@ def _event_us(torch, fn, reps):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def bench_rows_f32(args):
+    """The reference's own operator on a prompt: QuantizedMatmul<f32> (lhip_q8_0_matmul_f32) with M in
+    {16, 128, 512} activation rows over the Llama-3-8B weight shapes, f32 in and out at f32 accuracy.  From six
+    rows on the library runs it on the matrix cores with three-limb bf16 operands (six products, weights streamed
+    once per 64 rows); the one-matvec-per-row-group form the reference's launch corresponds to is timed beside it
+    on the 128-row gate shape.  A step is one pass over all shapes at all three M."""
+    import torch
+
+    from luminal_amd import capi
+
+    lib = capi.load_library()
+    dev = torch.device("cuda:0")
+    capi.check(lib.lhip_init(0), "lhip_init")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0x5EED + 5)
+    stream = torch.cuda.current_stream().cuda_stream
+    shapes = {"q/o": (4096, 4096), "k/v": (1024, 4096), "gate/up": (14336, 4096), "down": (4096, 14336)}
+    ms_list = (16, 128, 512)
+    bufs = {nm: [make_weight(torch, lib, capi, n, k, gen, dev) for _ in range(4)] for nm, (n, k) in shapes.items()}
+    xs = {(m, k): torch.randn((m, k), device=dev, generator=gen) for m in ms_list for k in (4096, 14336)}
+    ys = {(m, n): torch.empty((m, n), device=dev) for m in ms_list for n in (4096, 1024, 14336)}
+
+    def run(nm, m, b):
+        n, k = shapes[nm]
+        capi.check(lib.lhip_q8_0_matmul_f32(b.data_ptr(), xs[(m, k)].data_ptr(), ys[(m, n)].data_ptr(), m, n, k, stream),
+                   "lhip_q8_0_matmul_f32")
+
+    def step():
+        for nm in shapes:
+            for m in ms_list:
+                run(nm, m, bufs[nm][0])
+
+    flops_step = sum(2.0 * m * n * k for (n, k) in shapes.values() for m in ms_list)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = {}
+    for nm, (n, k) in shapes.items():
+        for m in ms_list:
+            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3) / len(bufs[nm])
+            passes = (m + 63) // 64
+            per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(2.0 * m * n * k / us / 1e6, 1),
+                                  "weight_gbs": round(passes * n * k * 34 / 32 / us / 1e3, 1)}
+    # the matvec form (a launch shape given: never the matrix-core form) on gate at 128 rows
+    n, k, m = 14336, 4096, 128
+    b = bufs["gate/up"][0]
+    mv_us = _event_us(torch, lambda: capi.check(lib.lhip_q8_0_matmul_f32_cfg(
+        b.data_ptr(), xs[(m, k)].data_ptr(), ys[(m, n)].data_ptr(), m, n, k, 2, 4, 4, 4, stream), "cfg"), 3)
+    g = per["gate/up M=128"]
+    print(json.dumps({
+        "metric": "Q8_0 f32 matmul operator with several activation rows (f32-exact on bf16 MFMA): TFLOP/s, 1 GPU",
+        "value": round(flops_step / (wall / args.steps) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 weights x f32 activations as three bf16 limbs each, six products, f32 accumulate, f32 out",
+        "data": "synthetic", "config": {"workload": "llama3_8b_q8_0_f32_rows_set", "m": list(ms_list)},
+        "per_shape": per, "matvec_form_gate_m128_us": round(mv_us, 1),
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, 1, float> (gate/up, M=128: two passes)",
+                     "achieved": round(6 * g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(6 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "note": "achieved counts the six bf16 products issued per useful multiply-add"}}))
 
 
 def bench_prefill_gemm(args):
@@ -349,6 +417,8 @@ def main():
         return bench_prefill_gemm(args)
     if args.workload == "moe":
         return bench_moe(args)
+    if args.workload == "rows_f32":
+        return bench_rows_f32(args)
 
     import torch
 
