@@ -143,9 +143,9 @@ def _event_us(torch, fn, reps):
 def bench_rows_f32(args):
     """The reference's own operator on a prompt: QuantizedMatmul<f32> (lhip_q8_0_matmul_f32) with M in
     {16, 128, 512} activation rows over the Llama-3-8B weight shapes, f32 in and out at f32 accuracy.  From six
-    rows on the library runs it on the matrix cores with three-limb bf16 operands (six products, weights streamed
-    once per 64 rows); the one-matvec-per-row-group form the reference's launch corresponds to is timed beside it
-    on the 128-row gate shape.  A step is one pass over all shapes at all three M."""
+    rows on the library runs it on the matrix cores (codes as exact bf16, x as three bf16 limbs: three products per
+    step, the block scale applied to each block's f32 sum; weights streamed once per 64 rows); the one-matvec-per-
+    row-group form the reference's launch corresponds to is timed beside it on the 128-row gate shape.  A step is one pass over all shapes at all three M."""
     import torch
 
     from luminal_amd import capi
@@ -199,13 +199,13 @@ def bench_rows_f32(args):
         "value": round(flops_step / (wall / args.steps) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 weights x f32 activations as three bf16 limbs each, six products, f32 accumulate, f32 out",
+        "dtype": "int8 codes as bf16 x f32 activations as three bf16 limbs, three products per step, block scales and sums in f32, f32 out",
         "data": "synthetic", "config": {"workload": "llama3_8b_q8_0_f32_rows_set", "m": list(ms_list)},
         "per_shape": per, "matvec_form_gate_m128_us": round(mv_us, 1),
         "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, 1, float> (gate/up, M=128: two passes)",
-                     "achieved": round(6 * g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(6 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "note": "achieved counts the six bf16 products issued per useful multiply-add"}}))
+                     "achieved": round(3 * g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(3 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "note": "achieved counts the three bf16 products issued per useful multiply-add"}}))
 
 
 def bench_prefill_gemm(args):

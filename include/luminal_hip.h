@@ -96,10 +96,11 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
 
 /* The same operator for several activation rows on the matrix cores.  The reference's launch (quantized.rs:159) is
  * one matvec per activation row, i.e. the weights are streamed once per row; this form streams them once per 64
- * rows.  x and q*d are each carried as three bf16 limbs whose sum is the f32 value exactly, and six of the nine limb
- * products (all but the three below 2^-24 of a term) are accumulated in f32 on the matrix cores: the result differs
- * from the matvec form only by the order of the f32 additions (measured 1e-6 of the rms against 5e-7), and products
- * of small integers stay exact.  The f16 form is the f32 form on the widened inputs, rounded once.  Any m >= 1.
+ * rows.  The int8 codes go to the matrix cores as they are (exact in bf16), x as three bf16 limbs whose sum is the
+ * f32 value exactly; per Q8_0 block the three products are summed in f32 and the block's scale is applied to that
+ * sum, as the matvec kernels do.  Every product is exact, so the result differs from the matvec form only by the
+ * order of the f32 additions (measured 5e-7 to 9e-7 of the rms for both), and products of small integers stay
+ * exact.  The f16 form is the f32 form on the widened inputs, rounded once.  Any m >= 1.
  * LHIP_ERR_UNSUPPORTED unless K % 512 == 0, N % 4 == 0, x 16-byte and y 16-byte (f16: 8-byte) aligned.
  * lhip_q8_0_matmul_f32 and lhip_q8_0_matmul_f16 take this form by themselves from six rows on where those
  * conditions hold (the _cfg entry never does).  May keep partial sums in the library's scratch array, see the

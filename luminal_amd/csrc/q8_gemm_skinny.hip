@@ -98,13 +98,6 @@ __device__ __forceinline__ void sk_split2(float a, float b, uint32_t (&limb)[3])
     }
 }
 
-// The same two codes as the three limbs of q * d.
-__device__ __forceinline__ void sk_dequant2_split(uint32_t w, int h, float d, float off, uint32_t (&limb)[3]) {
-    const float lo = fmaf(static_cast<float>((w >> (16 * h)) & 0xffu), d, off);
-    const float hi = fmaf(static_cast<float>((w >> (16 * h + 8)) & 0xffu), d, off);
-    sk_split2(lo, hi, limb);
-}
-
 // One output form for four consecutive weight rows n .. n+3 of activation row m.
 template <int OUT>
 __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M, int N, int m, int n, sk_f32x4 v) {
@@ -135,12 +128,9 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
 // RING = groups in flight per wave and row block; a slice is a multiple of RING groups.
 //
 // XT = __bf16: the product as described above.  XT = float or __half ("split"): the f32-exact form behind the
-// f32 / f16 matmul operators for more than a few activation rows.  Both operands are carried as three bf16 limbs
-// whose sum is the f32 value exactly (x = x0 + x1 + x2, likewise q * d, which has 19 significant bits), and six
-// products are accumulated per step, smallest first: x0*w2 + x2*w0 + x1*w1 + x1*w0 + x0*w1 + x0*w0.  Each is
-// exact in f32; what is dropped (x1*w2, x2*w1, x2*w2) is below 2^-24 of a term, so the result differs from the
-// matvec kernels' only by the order of the f32 additions.  The loaders split x on its way into LDS (three planes
-// per tile), the compute waves split q * d as they unpack it.  At most 64 activation rows (MT <= 4).
+// f32 / f16 matmul operators for more than a few activation rows (at most 64 per pass, MT <= 4, RB = 1); its
+// compute path is the `if constexpr (SPLIT)` block below, its loaders write x as three bf16 limbs whose sum is the
+// f32 value exactly (three planes per tile, pieces in natural order).
 template <int MT, int OUT, int RING, int RB, typename XT = __bf16>
 __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
                                                              const XT *__restrict__ x, void *__restrict__ y,
@@ -175,7 +165,8 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             const int m = c / (G * 8), j = c % (G * 8);
             const int panel = j >> 3, jj = j & 7;
             src[i] = x + static_cast<size_t>(min(m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
-            dst[i] = panel * S::PANEL + m * kSkPitch + ((jj >> 1) + 4 * (jj & 1)) * 16;
+            // plain form: pieces permuted to its operand order; split form: natural order (a step is one Q8_0 block)
+            dst[i] = panel * S::PANEL + m * kSkPitch + (SPLIT ? jj : (jj >> 1) + 4 * (jj & 1)) * 16;
         }
         constexpr int XL = sizeof(XT) == 4 ? 2 : 1;  // 16-byte loads per piece of 8 k
         sk_u32x4 xr[2][S::CH][XL];
@@ -243,6 +234,116 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     // ---------------- compute waves
     const int r = lane & 15, g = lane >> 4;
     const int n0 = strip * kSkRows + wave * (16 * RB);
+
+    if constexpr (SPLIT) {
+        // ---- f32-exact form.  The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block
+        // scale is applied to the f32 sum of each block, as the matvec kernels do; only x is split, into three bf16
+        // limbs.  An MFMA step is one Q8_0 block: lane (r, g) supplies codes 8g .. 8g+7 of the block (one 8-byte
+        // load) and the matching x pieces lie in natural order in LDS.  Per block and column block three chained
+        // MFMAs (x2, x1, x0; exact products, 96 f32 additions) and four fmas acc += d * sum.
+        static_assert(RB == 1, "one row block per compute wave");
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        const int n_rounds = n_groups >> 2;
+        const int8_t *a_ptr = qs + static_cast<size_t>(min(n0 + r, N - 1)) * K + static_cast<size_t>(g_begin) * 64 + 8 * g;
+        const __half *d_ptr[4];  // scales of the four weight rows this lane accumulates: n0 + 4g + v
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            d_ptr[v] = ds + static_cast<size_t>(min(n0 + 4 * g + v, N - 1)) * (K >> 5) + static_cast<size_t>(g_begin) * 2;
+        u32x2 a_reg[RING][2];
+        sk_u32x4 d_reg[RING / 4][4];
+        auto load_a = [&](int u, int group) __attribute__((always_inline)) {
+            int gg = min(group, n_groups - 1) + rot;
+            if (gg >= n_groups) gg -= n_groups;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+                a_reg[u][b] = *reinterpret_cast<const u32x2 *>(a_ptr + static_cast<size_t>(gg) * 64 + 32 * b);
+        };
+        auto load_d = [&](int set, int round) __attribute__((always_inline)) {
+            int rr = min(round, n_rounds - 1) + rot / 4;
+            if (rr >= n_rounds) rr -= n_rounds;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) d_reg[set][v] = *reinterpret_cast<const sk_u32x4 *>(d_ptr[v] + static_cast<size_t>(rr) * 8);
+        };
+        // same order of requests in the prologue as in the loop: a0 .. a3, d0, a4 .. a7, d1
+#pragma unroll
+        for (int u = 0; u < RING; ++u) {
+            load_a(u, u);
+            if ((u & 3) == 3) load_d(u >> 2, u >> 2);
+        }
+        sk_f32x4 acc[MT];
+#pragma unroll
+        for (int cb = 0; cb < MT; ++cb) acc[cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
+
+        constexpr int UNITS = 2 * MT;  // (block, column block) pairs of a group
+        auto b_read = [&](const unsigned char *xb, int i, int limb) __attribute__((always_inline)) {
+            return *reinterpret_cast<const sk_bf16x8 *>(xb + limb * S::PLANE + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
+        };
+        const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
+        __syncthreads();  // tiles 0 and 1 are staged
+        sk_bf16x8 bn[3];  // the operands of the next unit, requested one unit ahead (into the next group's tile too)
+#pragma unroll
+        for (int l = 0; l < 3; ++l) bn[l] = b_read(xb_cur, 0, l);
+        int stage = 0;
+        for (int R = 0; R < n_rounds; R += RING / 4) {
+            sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
+                constexpr int u = decltype(uc)::value;
+                constexpr bool tile_ends = (u + 1) % G == 0;
+                const int gl = R * 4 + u;
+                const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
+                const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
+                // the eight codes of each block as bf16
+                asm volatile("" : "+v"(a_reg[u][0]), "+v"(a_reg[u][1]));
+                sk_u32x4 a_bf[2];
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t w = a_reg[u][b][e >> 1];
+                        const float lo = static_cast<float>(static_cast<signed char>(w >> (16 * (e & 1))));
+                        const float hi = static_cast<float>(static_cast<signed char>(w >> (16 * (e & 1) + 8)));
+                        a_bf[b][e] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+                    }
+                float dv[2][4];
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        dv[b][v] = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[u >> 2][v][u & 3] >> (16 * b))));
+                load_a(u, gl + RING);
+                if constexpr ((u & 3) == 3) load_d(u >> 2, R + RING / 4 + (u >> 2));
+                sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    sk_bf16x8 b[3];
+#pragma unroll
+                    for (int l = 0; l < 3; ++l) {
+                        b[l] = bn[l];
+                        bn[l] = i + 1 < UNITS ? b_read(xb_cur, i + 1, l) : b_read(xb_next, 0, l);
+                    }
+                    const sk_bf16x8 a = __builtin_bit_cast(sk_bf16x8, a_bf[i / MT]);
+                    sk_f32x4 t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[2], sk_f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[1], t, 0, 0, 0);
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[0], t, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[i % MT][v] = fmaf(dv[i / MT][v], t[v], acc[i % MT][v]);
+                });
+                xb_cur = xb_next;
+                if constexpr (tile_ends) {
+                    stage = stage_next;
+                    __syncthreads();
+                }
+            });
+        }
+        const int n = n0 + 4 * g;
+        if (n < N) {
+#pragma unroll
+            for (int cb = 0; cb < MT; ++cb) {
+                const int m = cb * 16 + r;
+                if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[cb]);
+            }
+        }
+        return;
+    }
+
     const int8_t *a_ptr[RB];
     const __half *d_ptr[RB];
 #pragma unroll
@@ -275,8 +376,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     // Dequantisation of ring slot `un` in sixteen pieces of two codes: piece p belongs to row block p / 8,
     // step (p / 4) % 2, dword p / 2 of the lane's four, half p % 2.
     float d_next[RB], off_next[RB];
-    constexpr int P = SPLIT ? 3 : 1;  // operand planes: the bf16 value, or its three limbs
-    auto dequant_piece = [&](sk_u32x4 (&to)[P][RB][2], int un, int p) __attribute__((always_inline)) {
+    auto dequant_piece = [&](sk_u32x4 (&to)[RB][2], int un, int p) __attribute__((always_inline)) {
         const int rb = p >> 3, dw = (p >> 1) & 3;
         // Opaque to the optimiser: keeps the unpacking here, at its use, instead of next to the load
         asm volatile("" : "+v"(a_reg[un][rb]));
@@ -286,15 +386,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             off_next[rb] = -128.f * d_next[rb];
         }
         if ((p & 1) == 0) a_reg[un][rb][dw] ^= 0x80808080u;
-        const int st = (p >> 2) & 1, e = (p >> 1) & 1 ? 2 + (p & 1) : (p & 1);
-        if constexpr (SPLIT) {
-            uint32_t l3[3];
-            sk_dequant2_split(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb], l3);
-#pragma unroll
-            for (int l = 0; l < 3; ++l) to[l][rb][st][e] = l3[l];
-        } else {
-            to[0][rb][st][e] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
-        }
+        to[rb][(p >> 2) & 1][(p >> 1) & 1 ? 2 + (p & 1) : (p & 1)] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
     };
 
     // the loop reloads in the order a0 a1 a2 a3 d0 a4 a5 a6 a7 d1: the same order here, so the counted waits of the
@@ -305,35 +397,28 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         if ((u & 3) == 3) load_d(u >> 2, u >> 2);
     }
 
-    // Split form: the five small products of a step go to an accumulator of their own, so that their sum, 2^-8 of the
-    // main one, is rounded at its own scale and the main accumulator sees one addition per step, as in the plain form.
-    constexpr int NA = SPLIT ? 2 : 1;
-    sk_f32x4 acc[NA][RB][MT];
+    sk_f32x4 acc[RB][MT];
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (int cb = 0; cb < MT; ++cb) acc[a][rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int cb = 0; cb < MT; ++cb) acc[rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
 
     // A group is UNITS = 2 * MT units (step, column block): one B operand read and two MFMAs each.  W reads are
     // kept in flight, running ahead into the next group (whose tile was complete in LDS a barrier ago), and the
     // next group's dequantisation is dealt out over the units, so that LDS latency and VALU work sit under MFMAs.
     constexpr int UNITS = 2 * MT;
-    constexpr int W = SPLIT ? 2 : (UNITS < 4 ? UNITS : 4);  // units of B operands in flight (P reads each)
-    auto b_read = [&](const unsigned char *xb, int i, int plane) __attribute__((always_inline)) {
-        return *reinterpret_cast<const sk_bf16x8 *>(xb + plane * S::PLANE + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
+    constexpr int W = UNITS < 4 ? UNITS : 4;
+    auto b_read = [&](const unsigned char *xb, int i) __attribute__((always_inline)) {
+        return *reinterpret_cast<const sk_bf16x8 *>(xb + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
     };
-    sk_u32x4 af[P][RB][2];  // [plane][row block][step] of the group being multiplied, as packed bf16
-    sk_bf16x8 bw[W][P];
+    sk_u32x4 af[RB][2];  // [row block][step] of the group being multiplied, as packed bf16
+    sk_bf16x8 bw[W];
 #pragma unroll
     for (int p = 0; p < 8 * RB; ++p) dequant_piece(af, 0, p);
     const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
     __syncthreads();  // tiles 0 and 1 are staged
 #pragma unroll
-    for (int i = 0; i < W; ++i)
-#pragma unroll
-        for (int pl = 0; pl < P; ++pl) bw[i][pl] = b_read(xb_cur, i, pl);
+    for (int i = 0; i < W; ++i) bw[i] = b_read(xb_cur, i);
     int stage = 0;
     for (int R = 0; R < n_rounds; R += RING / 4) {
         sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
@@ -343,15 +428,11 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             const int gl = R * 4 + u;
             const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
             const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
-            sk_u32x4 af_next[P][RB][2];
+            sk_u32x4 af_next[RB][2];
             sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                sk_bf16x8 b[P];
-#pragma unroll
-                for (int pl = 0; pl < P; ++pl) {
-                    b[pl] = bw[i % W][pl];
-                    bw[i % W][pl] = i + W < UNITS ? b_read(xb_cur, i + W, pl) : b_read(xb_next, i + W - UNITS, pl);
-                }
+                const sk_bf16x8 b = bw[i % W];
+                bw[i % W] = i + W < UNITS ? b_read(xb_cur, i + W) : b_read(xb_next, i + W - UNITS);
                 sk_static_for<8 * RB>([&](auto pc) __attribute__((always_inline)) {
                     constexpr int p = decltype(pc)::value;
                     if constexpr (p * UNITS / (8 * RB) == i) {
@@ -368,29 +449,15 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                     }
                 });
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb) {
-                    auto prod = [&](sk_f32x4 &c, int wl, int xl) __attribute__((always_inline)) {
-                        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[wl][rb][i / MT]), b[xl], c, 0, 0, 0);
-                    };
-                    if constexpr (SPLIT) {  // the small terms, smallest first
-                        sk_f32x4 c = acc[1][rb][i % MT];
-                        prod(c, 2, 0);
-                        prod(c, 0, 2);
-                        prod(c, 1, 1);
-                        prod(c, 0, 1);
-                        prod(c, 1, 0);
-                        acc[1][rb][i % MT] = c;
-                    }
-                    prod(acc[0][rb][i % MT], 0, 0);
-                }
+                for (int rb = 0; rb < RB; ++rb)
+                    acc[rb][i % MT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[rb][i / MT]), b,
+                                                                              acc[rb][i % MT], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             });
 #pragma unroll
-            for (int pl = 0; pl < P; ++pl)
+            for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-                    for (int st = 0; st < 2; ++st) af[pl][rb][st] = af_next[pl][rb][st];
+                for (int st = 0; st < 2; ++st) af[rb][st] = af_next[rb][st];
             xb_cur = xb_next;
             if constexpr (tile_ends) {
                 stage = stage_next;
@@ -407,7 +474,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
 #pragma unroll
         for (int cb = 0; cb < MT; ++cb) {
             const int m = cb * 16 + r;
-            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, SPLIT ? acc[0][rb][cb] + acc[NA - 1][rb][cb] : acc[0][rb][cb]);
+            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[rb][cb]);
         }
     }
 }

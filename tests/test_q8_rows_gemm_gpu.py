@@ -2,11 +2,12 @@
 (lhip_q8_0_matmul_f32_gemm, lhip_q8_0_matmul_f16_gemm), through the C ABI.
 
 The reference's operator (QuantizedMatmul<T>::process, crates/luminal_cuda/src/quantized.rs:116-168) runs one
-matvec per activation row; this form streams the weights once per 64 rows with both operands carried as three
-bf16 limbs whose sum is the f32 value, and six of the nine limb products.  Bars: the operator's own (conftest.rel_err
-< 2e-3: every element, with a floor of 1e-3 rms) and max |y - t| / rms(t) < 5e-6 against the f64 product (the
-matvec kernels reach 1e-6, two limbs 2e-5, bf16 operands alone 5e-3); integer cases exact; the f16 form bit-equal
-to the f32 form on the widened inputs rounded once.
+matvec per activation row; this form streams the weights once per 64 rows: the codes enter the matrix cores as
+exact bf16, x as three bf16 limbs whose sum is the f32 value, and each block's f32 sum is scaled as in the matvec
+kernels.  Bars: the operator's own (conftest.rel_err < 2e-3: every element, with a floor of 1e-3 rms) and
+max |y - t| / rms(t) < 5e-6 against the f64 product (measured 1e-6, like the matvec kernels; two limbs of x and of
+q * d give 2e-5, bf16 operands alone 5e-3); integer cases exact; a one-hot row returns the weight column bit for
+bit; the f16 form is bit-equal to the f32 form on the widened inputs rounded once.
 """
 import numpy as np
 import pytest
@@ -94,7 +95,7 @@ def test_rows_gemm_integer_exact_and_wide_dynamic_range(oracle):
 
 def test_rows_gemm_full_size_one_hot(oracle):
     """gate (14336 x 4096) at 128 rows (two passes): zero rows give zero, a one-hot row gives the weight column
-    exactly (q * d has 19 significant bits, the three limbs carry 24)."""
+    exactly (one exact product, one exact scaling)."""
     n, k = synth.LLAMA3_8B_PROJ["gate"]
     qs, d = synth.q8_0_random(n, k, seed=77)
     w = upload(qs, d)
