@@ -9,7 +9,7 @@ torch = pytest.importorskip("torch")
 
 from conftest import rel_err  # noqa: E402
 from luminal_amd import capi, synth  # noqa: E402
-from luminal_amd.llama import LlamaConfig, LlamaQ8, fuse_rows, interleave_rows  # noqa: E402
+from luminal_amd.llama import LlamaConfig, LlamaQ8, fuse_rows, interleave_rows, random_weights  # noqa: E402
 from luminal_amd.quantized import Q8Weight  # noqa: E402
 from oracle import llama_oracle as lo  # noqa: E402
 
@@ -440,6 +440,38 @@ def test_bf16_output_forms_equal_the_rounded_f32_forms():
     assert torch.equal(a16, rounded(a32))
     assert lib.lhip_attention_f32_bf16out(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), a16.data_ptr(), pos.data_ptr(),
                                           S, 6, 2, hd, max_seq, s()) == capi.LHIP_ERR_UNSUPPORTED
+
+
+def test_prompt_pass_replays_from_a_graph():
+    """The bf16 prompt pass allocates nothing once its buffers exist (the K-sliced GEMMs keep their partial sums in
+    the library's own scratch array), so it can be captured; every replay, with eager passes and synchronisations
+    in between, gives the eager logits bit for bit."""
+    cfg = LlamaConfig(vocab=1000, dim=1024, layers=3, q_heads=8, kv_heads=2, ffn=2048)
+    eng = LlamaQ8(cfg, random_weights(cfg, seed=4, device=DEV), max_seq=128)
+    n = 16
+    t = torch.as_tensor(np.random.default_rng(0).integers(0, cfg.vocab, n).astype(np.float32)).to(DEV)
+    eng.reset()
+    ref = eng.forward(t, n, bf16=True).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eng.reset()
+        eng.forward(t, n, bf16=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eng.reset()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = eng.forward(t, n, bf16=True)
+    for _ in range(3):
+        eng.reset()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref)
+        eng.reset()
+        other = eng.forward(t.flip(0).contiguous(), n, bf16=True).clone()  # eager work between the replays
+        torch.cuda.synchronize()
+        assert not torch.equal(other, ref)
 
 
 def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
