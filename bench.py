@@ -202,7 +202,7 @@ def bench_rows_f32(args):
         "dtype": "int8 codes as bf16 x f32 activations as three bf16 limbs, three products per step, block scales and sums in f32, f32 out",
         "data": "synthetic", "config": {"workload": "llama3_8b_q8_0_f32_rows_set", "m": list(ms_list)},
         "per_shape": per, "matvec_form_gate_m128_us": round(mv_us, 1),
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, 1, float> (gate/up, M=128: two passes)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, 1, float> (gate/up, M=128: two passes of 64 rows in one launch)",
                      "achieved": round(3 * g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(3 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "note": "achieved counts the three bf16 products issued per useful multiply-add"}}))

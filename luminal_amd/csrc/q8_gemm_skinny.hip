@@ -148,6 +148,8 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     const int g_begin = split * slice_groups;
     const int n_groups = min(slice_groups, (K >> 6) - g_begin);
     const int n_tiles = n_groups / G;
+    // split form: blockIdx.z takes 64 activation rows of the M in all (one launch streams the weights once per pass)
+    const int m_base = SPLIT ? static_cast<int>(blockIdx.z) * 64 : 0;
     // With few activation rows every strip starts its walk over K at a different place (a whole number of rings):
     // the strips advance at the same pace and would otherwise all ask the same memory channels for the same k at
     // the same time (measured: 39 -> 36 us for 28672 x 4096 at 16 rows).  With many rows the strips reading the
@@ -164,7 +166,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             const int c = lt + i * 256;
             const int m = c / (G * 8), j = c % (G * 8);
             const int panel = j >> 3, jj = j & 7;
-            src[i] = x + static_cast<size_t>(min(m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
+            src[i] = x + static_cast<size_t>(min(m_base + m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
             // plain form: pieces permuted to its operand order; split form: natural order (a step is one Q8_0 block)
             dst[i] = panel * S::PANEL + m * kSkPitch + (SPLIT ? jj : (jj >> 1) + 4 * (jj & 1)) * 16;
         }
@@ -337,7 +339,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         if (n < N) {
 #pragma unroll
             for (int cb = 0; cb < MT; ++cb) {
-                const int m = cb * 16 + r;
+                const int m = m_base + cb * 16 + r;
                 if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[cb]);
             }
         }
@@ -606,49 +608,57 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
 
 template <int MT, int OUT, typename XT>
 static lhip_status sk_launch_split_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
-                                     int k, int splits, hipStream_t s) {
+                                     int k, int splits, int passes, hipStream_t s) {
     auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, 1, XT>;
     constexpr size_t lds_bytes = SkShape<MT, true>::LDS;
     if (lds_bytes > 64 * 1024)
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)));
     const int units = k / kSkUnit, per = (units + splits - 1) / splits;
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits)),
+    hipLaunchKernelGGL(kern,
+                       dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits),
+                            static_cast<unsigned>(passes)),
                        dim3(12 * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
+// m rows in all; passes of 64 rows (one: the tile height follows m).
 template <typename XT, int OUT>
 static lhip_status sk_launch_split_rows(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
-                                        int k, int splits, hipStream_t s) {
+                                        int k, int splits, int passes, hipStream_t s) {
     if (splits > 1) {
-        if (m <= 16) return sk_launch_split_t<1, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
-        if (m <= 32) return sk_launch_split_t<2, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
-        return sk_launch_split_t<4, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, s);
+        if (passes == 1 && m <= 16) return sk_launch_split_t<1, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
+        if (passes == 1 && m <= 32) return sk_launch_split_t<2, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
+        return sk_launch_split_t<4, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, passes, s);
     }
-    if (m <= 16) return sk_launch_split_t<1, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
-    if (m <= 32) return sk_launch_split_t<2, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
-    return sk_launch_split_t<4, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, s);
+    if (passes == 1 && m <= 16) return sk_launch_split_t<1, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+    if (passes == 1 && m <= 32) return sk_launch_split_t<2, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+    return sk_launch_split_t<4, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, passes, s);
 }
 
 bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16) {
     return k % kSkUnit == 0 && n % 4 == 0 && aligned(x, 16) && aligned(y, f16 ? 8 : 16);
 }
 
-// y (m, N) = x (m, K) W^T for f32 or f16 activations and results, any m: 64 rows at a time, each pass streaming
-// the weights once.  `splits` = 0: chosen here.  The caller has checked q8_gemm_split_supports.
+// y (m, N) = x (m, K) W^T for f32 or f16 activations and results, any m: passes of 64 rows, each streaming the
+// weights once, as blockIdx.z of one launch; K is sliced only while strips x passes leave the chip unfilled.  At most
+// kSkMaxPasses passes per launch (the grid's z extent).  `splits` = 0: chosen here.  The caller has checked
+// q8_gemm_split_supports.
 lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void *x, void *y, int64_t m, int n, int k,
                                  bool f16, int splits_arg, hipStream_t s) {
-    const int units = k / kSkUnit;
+    constexpr int64_t kSkMaxPasses = 1024;
+    const int units = k / kSkUnit, strips = (n + kSkRows - 1) / kSkRows;
     const size_t esz = f16 ? 2 : 4;
-    for (int64_t m0 = 0; m0 < m; m0 += 64) {
-        const int mc = static_cast<int>(m - m0 < 64 ? m - m0 : 64);
-        int splits = splits_arg > 0 ? splits_arg : q8_gemm_skinny_splits(mc, n, k);
+    for (int64_t m0 = 0; m0 < m; m0 += 64 * kSkMaxPasses) {
+        const int mc = static_cast<int>(m - m0 < 64 * kSkMaxPasses ? m - m0 : 64 * kSkMaxPasses);
+        const int passes = (mc + 63) / 64;
+        int splits = splits_arg > 0 ? splits_arg : 256 / (strips * passes);
+        if (splits < 1) splits = 1;
         if (splits > units) splits = units;
-        const int per = (units + splits - 1) / splits;
-        splits = (units + per - 1) / per;
         while (splits > 1 && static_cast<size_t>(splits) * mc * n > kSkScratchFloats) --splits;
+        const int per = (units + splits - 1) / splits;
+        splits = (units + per - 1) / per;  // no empty slice
         float *part = nullptr;
         if (splits > 1) {
             part = sk_scratch_ptr();
@@ -657,9 +667,9 @@ lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void 
         const auto *xc = static_cast<const unsigned char *>(x) + static_cast<size_t>(m0) * k * esz;
         auto *yc = static_cast<unsigned char *>(y) + static_cast<size_t>(m0) * n * esz;
         lhip_status st = f16 ? sk_launch_split_rows<__half, kSkOutF16>(qs, ds, reinterpret_cast<const __half *>(xc), yc, part,
-                                                                       mc, n, k, splits, s)
+                                                                       mc, n, k, splits, passes, s)
                              : sk_launch_split_rows<float, kSkOutF32>(qs, ds, reinterpret_cast<const float *>(xc), yc, part,
-                                                                      mc, n, k, splits, s);
+                                                                      mc, n, k, splits, passes, s);
         if (st != LHIP_OK) return st;
         if (splits > 1)
             if (lhip_status r = q8_gemm_reduce_launch(part, yc, mc, n, splits, f16 ? kSkOutF16 : kSkOutF32, s)) return r;
