@@ -354,6 +354,92 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     }
 }
 
+// The same pick in two launches for long rows: kArgmaxBlocks workgroups each leave the best (value, index) of
+// their contiguous part (one memory round trip instead of a single workgroup's many), a wave picks among those
+// and the n % 4 trailing entries.  The partial results live in a small per-device array; calls that overlap on
+// one device race for it, like every other call that shares scratch memory.
+constexpr int kArgmaxBlocks = 64;
+static __device__ __align__(256) float argmax_part[2 * kArgmaxBlocks];
+
+__device__ inline void argmax_take(float &v, int &idx, float c, int j) {
+    if (j >= 0 && (idx < 0 || c > v || (c == v && j > idx))) {
+        v = c;
+        idx = j;
+    }
+}
+
+__global__ __launch_bounds__(1024) void argmax_partial_kernel(const float4 *__restrict__ x4, int n4,
+                                                              float *__restrict__ part) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const int per = (n4 + kArgmaxBlocks - 1) / kArgmaxBlocks;
+    const int begin = blockIdx.x * per, end = min(n4, begin + per);
+    float v = -3.4e38f;
+    int idx = -1;
+    constexpr int U = 2;
+    for (int j0 = begin + threadIdx.x; j0 < end; j0 += U * 1024) {
+        float4 c[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = j0 + u * 1024;
+            c[u] = j < end ? x4[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = j0 + u * 1024;
+            if (j < end) {
+                argmax_take(v, idx, c[u].x, 4 * j); argmax_take(v, idx, c[u].y, 4 * j + 1);
+                argmax_take(v, idx, c[u].z, 4 * j + 2); argmax_take(v, idx, c[u].w, 4 * j + 3);
+            }
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) argmax_take(v, idx, __shfl_xor(v, o), __shfl_xor(idx, o));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        bv[wave] = v;
+        bi[wave] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        v = lane < 16 ? bv[lane] : 0.f;
+        idx = lane < 16 ? bi[lane] : -1;
+        for (int o = 8; o > 0; o >>= 1) argmax_take(v, idx, __shfl_xor(v, o), __shfl_xor(idx, o));
+        if (lane == 0) {
+            part[2 * blockIdx.x] = v;
+            part[2 * blockIdx.x + 1] = __int_as_float(idx);
+        }
+    }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restrict__ part, const float *__restrict__ x,
+                                                          int n4, int n, float *__restrict__ id_f32,
+                                                          int *__restrict__ id_i32, int *__restrict__ pos_dev,
+                                                          int advance) {
+    const int lane = threadIdx.x;
+    float v = part[2 * lane];
+    int idx = __float_as_int(part[2 * lane + 1]);
+    const int t = 4 * n4 + lane;  // at most three trailing entries
+    if (t < n) argmax_take(v, idx, x[t], t);
+    for (int o = 32; o > 0; o >>= 1) argmax_take(v, idx, __shfl_xor(v, o), __shfl_xor(idx, o));
+    if (lane == 0) {
+        if (id_f32) *id_f32 = static_cast<float>(idx);
+        if (id_i32) *id_i32 = idx;
+        if (pos_dev) *pos_dev += advance;
+    }
+}
+
+static float *argmax_part_ptr() {
+    static float *ptrs[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    float *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(argmax_part)) != hipSuccess) return nullptr;
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+    }
+    return p;
+}
+
 template <typename OutT>
 static lhip_status rms_norm_any(const float *x_dev, const float *residual_dev, float *x_out_dev, const float *w_dev,
                                 OutT *y_dev, int64_t rows, int64_t dim, float eps, void *stream) {
@@ -524,6 +610,18 @@ lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, in
                             int32_t advance, void *stream) {
     if (!x_dev || (!id_f32_dev && !id_i32_dev)) return LHIP_ERR_NULL_PTR;
     if (n <= 0 || n > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (n >= 16384 && aligned(x_dev, 16)) {  // long rows: partial picks over the chip, then one wave
+        float *part = argmax_part_ptr();
+        if (!part) return LHIP_ERR_HIP;
+        const int n4 = static_cast<int>(n >> 2);
+        hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxBlocks), dim3(1024), 0, as_stream(stream),
+                           reinterpret_cast<const float4 *>(x_dev), n4, part);
+        LHIP_CHECK_LAUNCH();
+        hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(64), 0, as_stream(stream), part, x_dev, n4,
+                           static_cast<int>(n), id_f32_dev, id_i32_dev, pos_dev, advance);
+        LHIP_CHECK_LAUNCH();
+        return LHIP_OK;
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x_dev, static_cast<int>(n), id_f32_dev,
                        id_i32_dev, pos_dev, advance);
     LHIP_CHECK_LAUNCH();

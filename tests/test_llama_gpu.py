@@ -134,6 +134,43 @@ def test_rope_attention_swiglu_gather_argmax():
     assert int(idi.item()) == 4021 == lo.argmax_last(v) and idf.item() == 4021.0 and int(pos.item()) == pos0 + 3
 
 
+@pytest.mark.parametrize("n", [16384, 16387, 128256, 128259, 1 << 20])
+def test_argmax_of_long_rows(n):
+    """Rows long enough for the two-launch pick (partial picks over 64 workgroups, then one wave): ties in several
+    workgroups' parts (the last index wins), the maximum among the n % 4 trailing entries, an unaligned row (the
+    single-workgroup kernel), all entries equal, and rows of -inf / lowest finite values."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(n)
+    idi = torch.zeros(1, dtype=torch.int32, device=DEV)
+    idf = torch.zeros(1, device=DEV)
+    pos = torch.tensor([5], dtype=torch.int32, device=DEV)
+
+    def pick(v, offset=0):
+        buf = torch.zeros(len(v) + 4, device=DEV)
+        buf[offset:offset + len(v)] = torch.from_numpy(v).to(DEV)
+        assert lib.lhip_argmax_f32(buf.data_ptr() + 4 * offset, len(v), idf.data_ptr(), idi.data_ptr(), pos.data_ptr(), 1,
+                                   s()) == 0
+        assert idf.item() == float(idi.item())
+        return int(idi.item())
+
+    v = rng.standard_normal(n).astype(np.float32)
+    assert pick(v) == lo.argmax_last(v)
+    ties = rng.choice(n, 9, replace=False)
+    v[ties] = 11.0
+    assert pick(v) == int(ties.max()) == lo.argmax_last(v)
+    assert pick(v, offset=1) == int(ties.max())            # row not 16-byte aligned
+    v[n - 1] = 12.0                                        # in the trailing entries when n % 4 != 0
+    assert pick(v) == n - 1
+    v[0] = 13.0
+    assert pick(v) == 0
+    assert pick(np.full(n, 2.5, np.float32)) == n - 1
+    assert pick(np.full(n, -np.inf, np.float32)) == n - 1
+    low = np.full(n, np.finfo(np.float32).min, np.float32)
+    low[n // 2] = -np.inf
+    assert pick(low) == n - 1
+    assert int(pos.item()) == 5 + 8
+
+
 @pytest.mark.parametrize("hq,hkv,hd", [(8, 2, 128), (32, 8, 128), (4, 4, 64), (16, 2, 64), (4, 2, 128)])
 @pytest.mark.parametrize("pos0", [0, 1, 63, 64, 200, 1500])
 def test_decode_attention_equals_rope_append_attention(hq, hkv, hd, pos0):
