@@ -96,8 +96,8 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
 
 /* The same operator for several activation rows on the matrix cores.  The reference's launch (quantized.rs:159) is
  * one matvec per activation row, i.e. the weights are streamed once per row; this form streams them once per 64
- * rows.  The int8 codes go to the matrix cores as they are (exact in bf16), x as three bf16 limbs whose sum is the
- * f32 value exactly; per Q8_0 block the three products are summed in f32 and the block's scale is applied to that
+ * rows.  The int8 codes go to the matrix cores as they are (exact in bf16), x as three bf16 limbs (an f16 x as
+ * two) whose sum is the value exactly; per Q8_0 block the limb products are summed in f32 and the block's scale is applied to that
  * sum, as the matvec kernels do.  Every product is exact, so the result differs from the matvec form only by the
  * order of the f32 additions (measured 5e-7 to 9e-7 of the rms for both), and products of small integers stay
  * exact.  The f16 form is the f32 form on the widened inputs, rounded once.  Any m >= 1.

@@ -22,7 +22,8 @@
 // on timing.
 //
 // The same kernel with f32 or f16 activations is the f32-exact form of the f32 / f16 matmul operators for several
-// activation rows: three bf16 limbs per operand, six limb products per step (see the kernel's comment).
+// activation rows: the codes as exact bf16, x as three bf16 limbs (two for f16), the block scales applied in f32
+// (see the kernel's comment).
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
@@ -57,16 +58,17 @@ __device__ __forceinline__ void sk_static_for(F &&f) {
     sk_static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
 }
 
-// SPLIT: f32 / f16 activations held as three bf16 planes (see q8_gemm_skinny_kernel), at most 64 rows, 64 k per
-// panel row as before but fewer panels per tile.
-template <int MT, bool SPLIT = false>
+// NL > 0 ("split"): f32 / f16 activations held as NL bf16 planes (see q8_gemm_skinny_kernel), at most 64 rows,
+// 64 k per panel row as before but fewer panels per tile.
+template <int MT, int NL = 0>
 struct SkShape {
+    static constexpr bool SPLIT = NL > 0;
     static_assert(!SPLIT || MT <= 4, "the split form takes at most 64 activation rows");
     static constexpr int G = SPLIT ? (MT >= 4 ? 1 : (MT == 2 ? 2 : 4))
                                    : (MT >= 8 ? 2 : 4);  // groups per activation tile; a slice is an even number of tiles
     static constexpr int PANEL = 16 * MT * kSkPitch;
     static constexpr int PLANE = G * PANEL;
-    static constexpr int STAGE = (SPLIT ? 3 : 1) * PLANE;
+    static constexpr int STAGE = (SPLIT ? NL : 1) * PLANE;
     static constexpr int CHUNKS = 16 * MT * G * 8;             // pieces of 8 k per tile
     static constexpr int CH = CHUNKS / 256;                    // per loader thread
     static_assert(CHUNKS % 256 == 0 && 8 % G == 0, "tile split");
@@ -85,12 +87,14 @@ __device__ __forceinline__ uint32_t sk_dequant2(uint32_t w, int h, float d, floa
     return __builtin_bit_cast(uint32_t, pk);
 }
 
-// Two f32 -> three packed bf16 pairs whose sums are the two values exactly: limb[0] the bf16 roundings, limb[1]
-// the roundings of what that left, limb[2] of what is left then (8 + 8 + 8 significant bits cover an f32).
-__device__ __forceinline__ void sk_split2(float a, float b, uint32_t (&limb)[3]) {
+// Two f32 -> NL packed bf16 pairs whose sums are the two values exactly: limb[0] the bf16 roundings, limb[1]
+// the roundings of what that left, limb[2] of what is left then (8 + 8 + 8 significant bits cover an f32, 8 + 8 the
+// 11 of a widened f16).
+template <int NL>
+__device__ __forceinline__ void sk_split2(float a, float b, uint32_t (&limb)[NL]) {
     typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int l = 0; l < 3; ++l) {
+    for (int l = 0; l < NL; ++l) {
         const bf16x2 h = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
         limb[l] = __builtin_bit_cast(uint32_t, h);
         a -= __uint_as_float(limb[l] << 16);
@@ -129,15 +133,17 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
 //
 // XT = __bf16: the product as described above.  XT = float or __half ("split"): the f32-exact form behind the
 // f32 / f16 matmul operators for more than a few activation rows (at most 64 per pass, MT <= 4, RB = 1); its
-// compute path is the `if constexpr (SPLIT)` block below, its loaders write x as three bf16 limbs whose sum is the
-// f32 value exactly (three planes per tile, pieces in natural order).
+// compute path is the `if constexpr (SPLIT)` block below, its loaders write x as bf16 limbs whose sum is the value
+// exactly (three planes per tile for f32, two for f16, whose 11 significant bits two limbs hold; pieces in natural
+// order).
 template <int MT, int OUT, int RING, int RB, typename XT = __bf16>
 __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
                                                              const XT *__restrict__ x, void *__restrict__ y,
                                                              float *__restrict__ part, int M, int N, int K,
                                                              int slice_groups) {
     constexpr bool SPLIT = !std::is_same<XT, __bf16>::value;
-    using S = SkShape<MT, SPLIT>;
+    constexpr int NL = SPLIT ? (sizeof(XT) == 4 ? 3 : 2) : 0;  // bf16 limbs of an activation
+    using S = SkShape<MT, NL>;
     constexpr int G = S::G;
     constexpr int CW = 8 / RB;  // compute waves, RB blocks of 16 weight rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
@@ -198,16 +204,17 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                         for (int e = 0; e < 8; ++e)
                             v[e] = __half2float(__ushort_as_half(static_cast<unsigned short>(xr[slot][i][0][e >> 1] >> (16 * (e & 1)))));
                     }
-                    sk_u32x4 limbs[3];
+                    constexpr int NLS = NL > 0 ? NL : 1;
+                    sk_u32x4 limbs[NLS];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        uint32_t l3[3];
-                        sk_split2(v[2 * e], v[2 * e + 1], l3);
+                        uint32_t l3[NLS];
+                        sk_split2<NLS>(v[2 * e], v[2 * e + 1], l3);
 #pragma unroll
-                        for (int l = 0; l < 3; ++l) limbs[l][e] = l3[l];
+                        for (int l = 0; l < NLS; ++l) limbs[l][e] = l3[l];
                     }
 #pragma unroll
-                    for (int l = 0; l < 3; ++l) *reinterpret_cast<sk_u32x4 *>(base + l * S::PLANE + dst[i]) = limbs[l];
+                    for (int l = 0; l < NLS; ++l) *reinterpret_cast<sk_u32x4 *>(base + l * S::PLANE + dst[i]) = limbs[l];
                 }
             }
         };
@@ -239,10 +246,11 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
 
     if constexpr (SPLIT) {
         // ---- f32-exact form.  The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block
-        // scale is applied to the f32 sum of each block, as the matvec kernels do; only x is split, into three bf16
+        // scale is applied to the f32 sum of each block, as the matvec kernels do; only x is split, into NL bf16
         // limbs.  An MFMA step is one Q8_0 block: lane (r, g) supplies codes 8g .. 8g+7 of the block (one 8-byte
-        // load) and the matching x pieces lie in natural order in LDS.  Per block and column block three chained
-        // MFMAs (x2, x1, x0; exact products, 96 f32 additions) and four fmas acc += d * sum.
+        // load) and the matching x pieces lie in natural order in LDS.  Per block and column block NL chained
+        // MFMAs (x2, x1, x0 for f32; exact products, 96 f32 additions; an f16's x2 is zero and has no MFMA, which
+        // leaves every sum as it is) and four fmas acc += d * sum.
         static_assert(RB == 1, "one row block per compute wave");
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         const int n_rounds = n_groups >> 2;
@@ -282,9 +290,9 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         };
         const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
         __syncthreads();  // tiles 0 and 1 are staged
-        sk_bf16x8 bn[3];  // the operands of the next unit, requested one unit ahead (into the next group's tile too)
+        sk_bf16x8 bn[NL];  // the operands of the next unit, requested one unit ahead (into the next group's tile too)
 #pragma unroll
-        for (int l = 0; l < 3; ++l) bn[l] = b_read(xb_cur, 0, l);
+        for (int l = 0; l < NL; ++l) bn[l] = b_read(xb_cur, 0, l);
         int stage = 0;
         for (int R = 0; R < n_rounds; R += RING / 4) {
             sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
@@ -315,16 +323,16 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                 if constexpr ((u & 3) == 3) load_d(u >> 2, R + RING / 4 + (u >> 2));
                 sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
                     constexpr int i = decltype(ic)::value;
-                    sk_bf16x8 b[3];
+                    sk_bf16x8 b[NL];
 #pragma unroll
-                    for (int l = 0; l < 3; ++l) {
+                    for (int l = 0; l < NL; ++l) {
                         b[l] = bn[l];
                         bn[l] = i + 1 < UNITS ? b_read(xb_cur, i + 1, l) : b_read(xb_next, 0, l);
                     }
                     const sk_bf16x8 a = __builtin_bit_cast(sk_bf16x8, a_bf[i / MT]);
-                    sk_f32x4 t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[2], sk_f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                    t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[1], t, 0, 0, 0);
-                    t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[0], t, 0, 0, 0);
+                    sk_f32x4 t = sk_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int l = NL - 1; l >= 0; --l) t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[l], t, 0, 0, 0);
 #pragma unroll
                     for (int v = 0; v < 4; ++v) acc[i % MT][v] = fmaf(dv[i / MT][v], t[v], acc[i % MT][v]);
                 });
@@ -610,7 +618,7 @@ template <int MT, int OUT, typename XT>
 static lhip_status sk_launch_split_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
                                      int k, int splits, int passes, hipStream_t s) {
     auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, 1, XT>;
-    constexpr size_t lds_bytes = SkShape<MT, true>::LDS;
+    constexpr size_t lds_bytes = SkShape<MT, sizeof(XT) == 4 ? 3 : 2>::LDS;
     if (lds_bytes > 64 * 1024)
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)));

@@ -3,7 +3,7 @@
 
 The reference's operator (QuantizedMatmul<T>::process, crates/luminal_cuda/src/quantized.rs:116-168) runs one
 matvec per activation row; this form streams the weights once per 64 rows: the codes enter the matrix cores as
-exact bf16, x as three bf16 limbs whose sum is the f32 value, and each block's f32 sum is scaled as in the matvec
+exact bf16, x as three bf16 limbs whose sum is the f32 value (an f16 x: two), and each block's f32 sum is scaled as in the matvec
 kernels.  Bars: the operator's own (conftest.rel_err < 2e-3: every element, with a floor of 1e-3 rms) and
 max |y - t| / rms(t) < 5e-6 against the f64 product (measured 1e-6, like the matvec kernels; two limbs of x and of
 q * d give 2e-5, bf16 operands alone 5e-3); integer cases exact; a one-hot row returns the weight column bit for
