@@ -315,7 +315,9 @@ lhip_status lhip_cast_bf16_to_f32(const void *x_dev, float *y_dev, int64_t n, vo
 /* x += y */
 lhip_status lhip_add_f32(float *x_dev, const float *y_dev, int64_t n, void *stream);
 /* Greedy pick (examples/llama/src/main.rs:194-198; the last index wins exact ties): the index
- * goes to *id_f32_dev and/or *id_i32_dev, and *pos_dev (if given) is advanced by `advance`. */
+ * goes to *id_f32_dev and/or *id_i32_dev, and *pos_dev (if given) is advanced by `advance`.
+ * Rows of 16384 entries or more (16-byte aligned) take two launches whose partial picks pass through a small
+ * array the library owns, one per device: picks that overlap in time on one device (two streams) race for it. */
 lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
                             int32_t advance, void *stream);
 
