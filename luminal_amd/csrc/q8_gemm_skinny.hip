@@ -228,14 +228,18 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         int stage = 2;  // buffer of tile t + 2
         for (int t = 0; t < n_tiles; t += 2) {  // two tiles per trip: no branch between them, so the counted waits
                                                 // are exact (the loads of a slot are two tiles old when it is stored)
+            // The fences keep the arithmetic on one slot's values (the limb split) behind the barrier before it:
+            // moved up, it waits for loads that are only one tile old instead of two.
             store_x(0, stage);  // tile t + 2 (a buffer last read for tile t - 1)
             load_x(0, t + 4);
             stage = stage == 2 ? 0 : stage + 1;
             __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
             store_x(1, stage);  // tile t + 3
             load_x(1, t + 5);
             stage = stage == 2 ? 0 : stage + 1;
             __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
         }
         return;
     }
@@ -290,9 +294,15 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         };
         const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
         __syncthreads();  // tiles 0 and 1 are staged
-        sk_bf16x8 bn[NL];  // the operands of the next unit, requested one unit ahead (into the next group's tile too)
+        // The x operands of a unit are requested two units ahead (into the next group's tile too, which is staged
+        // by then) in four rotating register sets, three of them live at a time; the fence keeps the request where
+        // it is, or the reads sink to their use and every unit waits a full LDS round trip.
+        sk_bf16x8 bq[4][NL];
 #pragma unroll
-        for (int l = 0; l < NL; ++l) bn[l] = b_read(xb_cur, 0, l);
+        for (int l = 0; l < NL; ++l) {
+            bq[0][l] = b_read(xb_cur, 0, l);
+            bq[1][l] = UNITS > 1 ? b_read(xb_cur, 1 % UNITS, l) : b_read(xb_cur, 0, l);
+        }
         int stage = 0;
         for (int R = 0; R < n_rounds; R += RING / 4) {
             sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
@@ -320,22 +330,25 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                     for (int v = 0; v < 4; ++v)
                         dv[b][v] = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[u >> 2][v][u & 3] >> (16 * b))));
                 load_a(u, gl + RING);
-                if constexpr ((u & 3) == 3) load_d(u >> 2, R + RING / 4 + (u >> 2));
                 sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
                     constexpr int i = decltype(ic)::value;
-                    sk_bf16x8 b[NL];
+                    constexpr int U = u * UNITS + i;  // RING * UNITS is a multiple of four: the sets rotate statically
+                    constexpr int ahead = i + 2;
 #pragma unroll
-                    for (int l = 0; l < NL; ++l) {
-                        b[l] = bn[l];
-                        bn[l] = i + 1 < UNITS ? b_read(xb_cur, i + 1, l) : b_read(xb_next, 0, l);
-                    }
+                    for (int l = 0; l < NL; ++l)
+                        bq[(U + 2) % 4][l] = ahead < UNITS ? b_read(xb_cur, ahead, l) : b_read(xb_next, ahead - UNITS, l);
+                    __builtin_amdgcn_sched_barrier(0);
                     const sk_bf16x8 a = __builtin_bit_cast(sk_bf16x8, a_bf[i / MT]);
                     sk_f32x4 t = sk_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int l = NL - 1; l >= 0; --l) t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[l], t, 0, 0, 0);
+                    for (int l = NL - 1; l >= 0; --l)
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[U % 4][l], t, 0, 0, 0);
 #pragma unroll
                     for (int v = 0; v < 4; ++v) acc[i % MT][v] = fmaf(dv[i / MT][v], t[v], acc[i % MT][v]);
                 });
+                // a set of scales is requested again once its last group has read it (requested earlier, the load
+                // gets other registers and a copy at the end of the trip that waits for every load in flight)
+                if constexpr ((u & 3) == 3) load_d(u >> 2, R + RING / 4 + (u >> 2));
                 xb_cur = xb_next;
                 if constexpr (tile_ends) {
                     stage = stage_next;
