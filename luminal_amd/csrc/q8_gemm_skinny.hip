@@ -283,6 +283,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         for (int u = 0; u < RING; ++u) {
             load_a(u, u);
             if ((u & 3) == 3) load_d(u >> 2, u >> 2);
+            __builtin_amdgcn_sched_barrier(0);  // or the requests are regrouped and the loop's counted waits follow
         }
         sk_f32x4 acc[MT];
 #pragma unroll
@@ -304,7 +305,8 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             bq[1][l] = UNITS > 1 ? b_read(xb_cur, 1 % UNITS, l) : b_read(xb_cur, 0, l);
         }
         int stage = 0;
-        for (int R = 0; R < n_rounds; R += RING / 4) {
+        int R = 0;
+        do {  // a slice is never empty: no guard, so the requests above stay where the fences put them
             sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
                 constexpr int u = decltype(uc)::value;
                 constexpr bool tile_ends = (u + 1) % G == 0;
@@ -355,7 +357,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                     __syncthreads();
                 }
             });
-        }
+        } while ((R += RING / 4) < n_rounds);
         const int n = n0 + 4 * g;
         if (n < N) {
 #pragma unroll
