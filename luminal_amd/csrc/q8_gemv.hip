@@ -209,6 +209,9 @@ __device__ __forceinline__ void load_step(StepBuf<R, S> &b, const int8_t *__rest
             b.d[s][r] = __builtin_nontemporal_load(reinterpret_cast<const unsigned short *>(drow + (s * 64u + doff)));
         }
     }
+    // The offsets stay live past the last request: otherwise their registers may become the destination of that
+    // request, and the next step, which writes the offsets again, first has to wait for it.
+    asm volatile("" ::"v"(qoff), "v"(doff));
 }
 
 template <int R, int S>
