@@ -642,8 +642,12 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
         col[f] = n0 + r;
         const size_t panel = (static_cast<size_t>(expert) * g.rows_per_expert + wrow0) >> 4;
         w_tile[f] = g.w_nib + (panel * chunks * 64 + lane) * 16;
-        s_tile[f] = g.w_sc + panel * chunks * 64 + lane;
+        s_tile[f] = g.w_sc + panel * chunks * 64 + (lane & ~3);  // the dword that holds this lane's scale byte
     }
+    // A lane's scale is requested as the aligned dword around it and shifted down at its use: a byte load is
+    // widened after the loop's phi, i.e. at the top of every trip for all D sets, and that widening waits for the
+    // set requested last.
+    const int s_shift = 8 * (lane & 3);
     BSet<1, NT> bs[D];
     auto load_b = [&](int set, int c) {
         bs[set].valid = c < chunks;
@@ -651,7 +655,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
 #pragma unroll
         for (int f = 0; f < NT; ++f) {
             bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
-            bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+            bs[set].s[f] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(s_tile[f] + cc * 64));
         }
     };
     // Weights first: their HBM round trip overlaps the staging of the activations.
@@ -703,7 +707,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
             asm volatile("" : "+v"(bs[set].q[f]), "+v"(bs[set].s[f]));
             const mu32x4 zero = {0, 0, 0, 0};
             const mu32x4 q = bs[set].valid ? bs[set].q[f] : zero;
-            const int sb = bs[set].valid ? static_cast<int>(bs[set].s[f]) : 127;
+            const int sb = bs[set].valid ? static_cast<int>(bs[set].s[f] >> s_shift) : 127;  // the matrix core reads byte 0
             const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
             acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[f], 0, 4, 0, sa, 0, sb);
             acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[f], 0, 4, 0, sa, 0, sb);
