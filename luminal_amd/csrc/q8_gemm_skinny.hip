@@ -251,26 +251,42 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     if constexpr (SPLIT) {
         // ---- f32-exact form.  The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block
         // scale is applied to the f32 sum of each block, as the matvec kernels do; only x is split, into NL bf16
-        // limbs.  An MFMA step is one Q8_0 block: lane (r, g) supplies codes 8g .. 8g+7 of the block (one 8-byte
-        // load) and the matching x pieces lie in natural order in LDS.  Per block and column block NL chained
-        // MFMAs (x2, x1, x0 for f32; exact products, 96 f32 additions; an f16's x2 is zero and has no MFMA, which
-        // leaves every sum as it is) and four fmas acc += d * sum.
+        // limbs.  An MFMA step is one Q8_0 block and a lane supplies eight of its codes; the x pieces lie in natural
+        // order in LDS and a lane reads the one that matches its codes.  Two ways to get the codes:
+        //  - WIDE (few activation rows, where the weight stream is what bounds the kernel): lane (r, g) requests the
+        //    16 codes 16g .. 16g+15 of a group of two blocks (one 16-byte load: a row's 64 bytes are contiguous over
+        //    its four lanes) and a swap between the wave's halves (lanes l and l + 32, i.e. g and g + 2) leaves it
+        //    with eight codes of each block: codes 0-7, 16-23, 8-15, 24-31 for g = 0 .. 3;
+        //  - otherwise two 8-byte loads, codes 8g .. 8g+7 of each block (from 64 rows on: measured 3-8 % faster
+        //    there for f32 activations than the wide loads, 3-5 % slower for f16; one choice for both types keeps
+        //    the order of additions, and so the f16 result, equal to the f32 form's).
+        // Per block and column block NL chained MFMAs (x2, x1, x0 for f32; exact products, 96 f32 additions; an
+        // f16's x2 is zero and has no MFMA, which leaves every sum as it is) and four fmas acc += d * sum.
+        constexpr bool WIDE = MT <= 2;
         static_assert(RB == 1, "one row block per compute wave");
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         const int n_rounds = n_groups >> 2;
-        const int8_t *a_ptr = qs + static_cast<size_t>(min(n0 + r, N - 1)) * K + static_cast<size_t>(g_begin) * 64 + 8 * g;
+        const int8_t *a_ptr = qs + static_cast<size_t>(min(n0 + r, N - 1)) * K + static_cast<size_t>(g_begin) * 64 + (WIDE ? 16 : 8) * g;
+        const int x_lane = r * kSkPitch + (WIDE ? (g & 1) * 32 + (g >> 1) * 16 : g * 16);  // the x piece of this lane's codes
         const __half *d_ptr[4];  // scales of the four weight rows this lane accumulates: n0 + 4g + v
 #pragma unroll
         for (int v = 0; v < 4; ++v)
             d_ptr[v] = ds + static_cast<size_t>(min(n0 + 4 * g + v, N - 1)) * (K >> 5) + static_cast<size_t>(g_begin) * 2;
-        u32x2 a_reg[RING][2];
+        sk_u32x4 a_reg[RING];
         sk_u32x4 d_reg[RING / 4][4];
         auto load_a = [&](int u, int group) __attribute__((always_inline)) {
             int gg = min(group, n_groups - 1) + rot;
             if (gg >= n_groups) gg -= n_groups;
+            if constexpr (WIDE) {
+                a_reg[u] = *reinterpret_cast<const sk_u32x4 *>(a_ptr + static_cast<size_t>(gg) * 64);
+            } else {
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
-                a_reg[u][b] = *reinterpret_cast<const u32x2 *>(a_ptr + static_cast<size_t>(gg) * 64 + 32 * b);
+                for (int b = 0; b < 2; ++b) {
+                    const u32x2 v = *reinterpret_cast<const u32x2 *>(a_ptr + static_cast<size_t>(gg) * 64 + 32 * b);
+                    a_reg[u][2 * b] = v[0];
+                    a_reg[u][2 * b + 1] = v[1];
+                }
+            }
         };
         auto load_d = [&](int set, int round) __attribute__((always_inline)) {
             int rr = min(round, n_rounds - 1) + rot / 4;
@@ -293,7 +309,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         auto b_read = [&](const unsigned char *xb, int i, int limb) __attribute__((always_inline)) {
             return *reinterpret_cast<const sk_bf16x8 *>(xb + limb * S::PLANE + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
         };
-        const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
+        const unsigned char *xb_cur = sk_lds + x_lane;
         __syncthreads();  // tiles 0 and 1 are staged
         // The x operands of a unit are requested two units ahead (into the next group's tile too, which is staged
         // by then) in four rotating register sets, three of them live at a time; the fence keeps the request where
@@ -312,15 +328,25 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                 constexpr bool tile_ends = (u + 1) % G == 0;
                 const int gl = R * 4 + u;
                 const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
-                const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
+                const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + x_lane;
                 // the eight codes of each block as bf16
-                asm volatile("" : "+v"(a_reg[u][0]), "+v"(a_reg[u][1]));
+                asm volatile("" : "+v"(a_reg[u]));
+                u32x2 a_blk[2];  // after the swap: dwords 0, 1 are codes of the group's first block, 2, 3 of its second
+                if constexpr (WIDE) {
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(a_reg[u][0], a_reg[u][2], false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(a_reg[u][1], a_reg[u][3], false, false);
+                    a_blk[0] = u32x2{s02[0], s13[0]};
+                    a_blk[1] = u32x2{s02[1], s13[1]};
+                } else {
+                    a_blk[0] = u32x2{a_reg[u][0], a_reg[u][1]};
+                    a_blk[1] = u32x2{a_reg[u][2], a_reg[u][3]};
+                }
                 sk_u32x4 a_bf[2];
 #pragma unroll
                 for (int b = 0; b < 2; ++b)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const uint32_t w = a_reg[u][b][e >> 1];
+                        const uint32_t w = a_blk[b][e >> 1];
                         const float lo = static_cast<float>(static_cast<signed char>(w >> (16 * (e & 1))));
                         const float hi = static_cast<float>(static_cast<signed char>(w >> (16 * (e & 1) + 8)));
                         a_bf[b][e] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
