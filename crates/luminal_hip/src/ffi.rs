@@ -17,7 +17,7 @@ extern "C" {
     pub fn lhip_q8_0_raw_nbytes(n: i64, k: i64) -> usize;
     pub fn lhip_q8_0_planar_nbytes(n: i64, k: i64) -> usize;
     pub fn lhip_q8_0_repack(raw: *const c_void, planar: *mut c_void, n: i64, k: i64, s: Stream) -> Status;
-    // with m >= 6 rows (a prompt) both matmuls run on the matrix cores by themselves, at f32 accuracy, streaming the
+    // with more than a few rows (a prompt) both matmuls run on the matrix cores by themselves, at f32 accuracy, streaming the
     // weights once per 64 rows instead of once per row
     pub fn lhip_q8_0_matmul_f32(w: *const c_void, x: *const f32, y: *mut f32, m: i64, n: i64, k: i64, s: Stream) -> Status;
     pub fn lhip_q8_0_gather_f32(w: *const c_void, idx: *const f32, out: *mut f32, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;

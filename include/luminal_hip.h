@@ -102,7 +102,8 @@ lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, flo
  * order of the f32 additions (measured 5e-7 to 9e-7 of the rms for both), and products of small integers stay
  * exact.  The f16 form is the f32 form on the widened inputs, rounded once.  Any m >= 1.
  * LHIP_ERR_UNSUPPORTED unless K % 512 == 0, N % 4 == 0, x 16-byte and y 16-byte (f16: 8-byte) aligned.
- * lhip_q8_0_matmul_f32 and lhip_q8_0_matmul_f16 take this form by themselves from six rows on where those
+ * lhip_q8_0_matmul_f32 and lhip_q8_0_matmul_f16 take this form by themselves from a few rows on (two for N*K >=
+ * 2^28 codes, three from 2^25, four from 2^23, six below: the measured crossovers with the matvec form) where those
  * conditions hold (the _cfg entry never does).  May keep partial sums in the library's scratch array, see the
  * note on overlapping calls at lhip_q8_0_matmul_bf16. */
 lhip_status lhip_q8_0_matmul_f32_gemm(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,

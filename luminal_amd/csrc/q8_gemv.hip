@@ -29,9 +29,14 @@ bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16
 lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void *x, void *y, int64_t m, int n, int k,
                                  bool f16, int splits, hipStream_t s);
 // From this many activation rows on the plain operators take that form where the shape allows it: the weights are
-// then streamed once per 64 rows instead of once per group of at most four (measured crossover: 14336 x 4096
-// 34 us either way at four rows, 4096 x 4096 at five to six).
-constexpr int kSplitMinRows = 6;
+// then streamed once per 64 rows instead of once per row.  The matrix-core form has a fixed cost (its launch, a
+// reduce launch where K is sliced, staging) that a matvec pass over a small matrix stays under.  Measured, matvec
+// against matrix cores, us: 1024 x 4096 at five rows 6.0 / 10.7; 4096 x 4096 at three rows 12.4 / 12.7, at four
+// 15.8 / 12.4; 14336 x 4096 at two rows 20.6 / 21.5, at three 31.7 / 22.0; 128256 x 4096 at two rows 168 / 130.
+static int split_min_rows(int64_t n, int64_t k) {
+    const int64_t codes = n * k;
+    return codes >= (int64_t{256} << 20) ? 2 : codes >= (int64_t{32} << 20) ? 3 : codes >= (int64_t{8} << 20) ? 4 : 6;
+}
 
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -712,7 +717,7 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
 lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
                                  int64_t k, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
-    if (m >= kSplitMinRows && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_dev, y_dev, false))
+    if (m >= split_min_rows(n, k) && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_dev, y_dev, false))
         return lhip_q8_0_matmul_f32_gemm(planar_dev, x_dev, y_dev, m, n, k, stream);
     int r, u, b, w;
     choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
@@ -726,7 +731,7 @@ lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, 
     if (m <= 0 || m > 65535) return LHIP_ERR_INVALID_SHAPE;
     // Rows of x start at multiples of K halves; K % 32 == 0 keeps them 8-byte aligned.
     if (!aligned(planar_dev, 256) || !aligned(x_f16_dev, 8) || !aligned(y_f16_dev, 2)) return LHIP_ERR_MISALIGNED;
-    if (m >= kSplitMinRows && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_f16_dev, y_f16_dev, true))
+    if (m >= split_min_rows(n, k) && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_f16_dev, y_f16_dev, true))
         return lhip_q8_0_matmul_f16_gemm(planar_dev, x_f16_dev, y_f16_dev, m, n, k, stream);
     auto *base = static_cast<const uint8_t *>(planar_dev);
     int r, u, b, w;

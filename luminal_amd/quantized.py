@@ -74,7 +74,7 @@ class Q8Weight:
 class QuantizedMatmul:
     """(.., M, K) x Q8_0 (N, K) -> (.., M, N) in the activation type T = f32 or f16, f32 accumulation either way
     (QuantizedMatmul<T>::process, crates/luminal_cuda/src/quantized.rs:116-168).  The library runs one matvec per
-    group of activation rows, as the reference does per row, or from six rows on (where the shape allows it) the
+    group of activation rows, as the reference does per row, or from two to six rows on, by matrix size (where the shape allows it), the
     matrix-core form with exact products (x as three bf16 limbs, an f16 x as two), which streams the weights once per 64 rows.  A launch shape
     can be chosen for f32 only and always means the matvec form."""
 

@@ -112,7 +112,7 @@ def test_rows_gemm_full_size_one_hot(oracle):
 
 
 def test_plain_operator_takes_the_matrix_core_form(oracle):
-    """lhip_q8_0_matmul_f32 / _f16 (and so QuantizedMatmul.process): from six rows on the matrix-core form where
+    """lhip_q8_0_matmul_f32 / _f16 (and so QuantizedMatmul.process): from six rows on (small matrices; large ones earlier) the matrix-core form where
     the shape allows it, the matvec form below that, for other shapes, and whenever a launch shape is given."""
     lib = capi.load_library()
     qs, d = synth.q8_0_random(512, 1024, seed=21)
@@ -139,6 +139,24 @@ def test_plain_operator_takes_the_matrix_core_form(oracle):
                                          stream()) == capi.LHIP_ERR_UNSUPPORTED
     wf2 = oracle.q8_0_dequant(synth.q8_0_raw_blocks(q2, d2), q2.size).reshape(q2.shape)
     assert rel_err(QuantizedMatmul().process(x2, w2).cpu().numpy(), oracle.matmul_f64(x2.cpu().numpy(), wf2)) < 2e-3
+
+
+def test_large_matrices_take_the_matrix_core_form_earlier(oracle):
+    """4096 x 4096 (2^24 codes): the plain operator is the matvec form at three rows and the matrix-core form at
+    four (bit-equal to the _gemm entry), both within the operator's bar."""
+    lib = capi.load_library()
+    n = k = 4096
+    qs, d = synth.q8_0_random(n, k, seed=31)
+    w = upload(qs, d)
+    wf = oracle.q8_0_dequant(synth.q8_0_raw_blocks(qs, d), qs.size).reshape(qs.shape)
+    for m, same in ((3, False), (4, True)):
+        x = synth.activations(m, k, seed=40 + m)
+        xd = torch.from_numpy(x).to(DEV)
+        y = torch.empty(m, n, device=DEV)
+        capi.check(lib.lhip_q8_0_matmul_f32(w.planar.data_ptr(), xd.data_ptr(), y.data_ptr(), m, n, k, stream()), "plain")
+        y = y.cpu().numpy()
+        assert np.array_equal(y, gemm_f32(w, x)) == same
+        assert rel_err(y, oracle.matmul_f64(x, wf)) < 2e-3
 
 
 def test_rows_gemm_argument_errors():
