@@ -88,10 +88,11 @@ class Content:
 
         tensor_count = rd(size)
         kv_count = rd(size)
-        metadata = {}
+        metadata, value_types = {}, {}
         for _ in range(kv_count):
             key = rd_string()
-            metadata[key] = rd_value(rd("<I"))
+            value_types[key] = rd("<I")
+            metadata[key] = rd_value(value_types[key])
         infos = {}
         for _ in range(tensor_count):
             name = rd_string()
@@ -103,8 +104,10 @@ class Content:
             offset = rd("<Q")
             infos[name] = TensorInfo(int(np.prod(dims, dtype=np.int64)) if dims else 1, offset, GGML_DTYPES[code], dims)
         pos = f.tell()
+        # the reference takes general.alignment from the 8/16/32-bit integer types only, signed ones when they are not
+        # negative (gguf.rs:246-255); anything else means the default.  (Zero would divide by zero there: default here.)
         a = metadata.get("general.alignment")
-        alignment = a if isinstance(a, int) and not isinstance(a, bool) and a > 0 else DEFAULT_ALIGNMENT
+        alignment = a if value_types.get("general.alignment") in (0, 1, 2, 3, 4, 5) and a > 0 else DEFAULT_ALIGNMENT
         return Content(version, metadata, infos, -(-pos // alignment) * alignment)
 
 

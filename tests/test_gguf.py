@@ -60,3 +60,49 @@ def test_llama_tensor_names_follow_the_reference_paths():
     names = gguf.llama_tensor_names(2)
     assert names[:3] == ["token_embd.weight", "output_norm.weight", "output.weight"]
     assert "blk.1.attn_output.weight" in names and "blk.0.ffn_gate.weight" in names and len(names) == 3 + 2 * 9
+
+
+def literal_bytes():
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_v3_literal.hex")
+    with open(path) as f:
+        return b"".join(bytes.fromhex(line.split("#")[0]) for line in f)
+
+
+def test_hand_assembled_v3_file(oracle):
+    """A file written out byte by byte from examples/llama/src/gguf.rs:190-263 (not by write_gguf): one key of every
+    value type, nested arrays, a string with a trailing NUL, alignment 64, one F32 and one Q8_0 tensor."""
+    b = literal_bytes()
+    assert len(b) == 644
+    f = io.BytesIO(b)
+    c = gguf.Content.read(f)
+    assert c.version == 3 and len(c.metadata) == 15
+    md = c.metadata
+    assert (md["u8"], md["i8"], md["u16"], md["i16"], md["u32"], md["i32"]) == (254, -128, 65534, -2, 4000000000, -5)
+    assert md["f32"] == 1.5 and md["bool"] is True and md["str"] == "ab" and md["arr"] == ["x", "yz"]
+    assert md["u64"] == 2 ** 40 + 1 and md["i64"] == -1 and md["f64"] == 0.25 and md["nest"] == [[7, 8]]
+    assert md["general.alignment"] == 64 and c.tensor_data_offset == 512  # 477 header bytes rounded up to 64
+    a, q = c.tensor_infos["a.weight"], c.tensor_infos["blk.0.attn_q.weight"]
+    assert (a.n_elements, a.offset, a.dtype) == (3, 0, "F32")
+    assert (q.n_elements, q.offset, q.dtype, q.dims) == (64, 64, "Q8_0", (32, 2))
+    assert np.array_equal(gguf.read_tensor(f, c, "a.weight"), np.array([1.0, -2.0, 0.5], np.float32))
+    raw = gguf.read_tensor(f, c, "blk.0.attn_q.weight")
+    assert raw.size == 68
+    w = oracle.q8_0_dequant(raw, 64).reshape(2, 32)
+    assert np.array_equal(w[0], 0.5 * np.arange(32, dtype=np.float32))
+    assert np.array_equal(w[1], -2.0 * np.arange(-16, 16, dtype=np.float32))
+
+
+def test_alignment_key_types(tmp_path):
+    # only 8/16/32-bit integer types set the alignment (gguf.rs:246-255): a u64 value is ignored
+    b = bytearray(literal_bytes())
+    at = bytes(b).index(b"general.alignment") + 17
+    assert bytes(b[at:at + 8]) == struct.pack("<II", 4, 64)
+    head = bytes(b[:at]) + struct.pack("<IQ", 10, 64) + bytes(b[at + 8:477])
+    c = gguf.Content.read(io.BytesIO(head))
+    assert c.metadata["general.alignment"] == 64 and c.tensor_data_offset == -(-len(head) // 32) * 32
+    head = bytes(b[:at]) + struct.pack("<Ii", 5, -64) + bytes(b[at + 8:477])  # negative i32: default
+    assert gguf.Content.read(io.BytesIO(head)).tensor_data_offset == -(-len(head) // 32) * 32
+    head = bytes(b[:at]) + struct.pack("<IB", 0, 16) + bytes(b[at + 8:477])   # u8 16
+    assert gguf.Content.read(io.BytesIO(head)).tensor_data_offset == -(-len(head) // 16) * 16
