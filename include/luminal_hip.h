@@ -152,12 +152,15 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
  * (x (m, K) row-major, 16-byte aligned), f32 accumulation on the matrix cores
  * and bf16 output (y (m, N) row-major).  The reference has no bf16 type and no
  * Q8_0 GEMM on CUDA (crates/luminal_cuda/src/quantized.rs:146-164 re-runs the
- * matvec per row); the counterpart is the Metal GEMM, which also rounds q*d to
- * the activation type before the matrix unit
- * (crates/luminal_metal/src/quantized.rs:54-61,63-199,353-376).  Weights are
- * rounded to bf16 after dequantisation, so results are within 1e-2 of the f32
- * semantics, not bit-equal.  K must be a multiple of 64 (LHIP_ERR_UNSUPPORTED
- * otherwise).
+ * matvec per row); the counterpart is the Metal GEMM
+ * (crates/luminal_metal/src/quantized.rs:54-61,63-199,353-376), which rounds
+ * q*d to the activation type before its matrix unit.  Here the weights stay
+ * exact: the int8 codes go to the matrix cores as they are (exact in bf16) and
+ * every Q8_0 block's f32 sum is multiplied by the block's scale in f32, the
+ * arithmetic of the reference's matvec kernel (quantized.rs:93-96).  With bf16
+ * activations every product is exact, so the f32 result differs from the exact
+ * one only by the roundings of the f32 additions, and the bf16 result by one
+ * more rounding.  K must be a multiple of 64 (LHIP_ERR_UNSUPPORTED otherwise).
  *
  * With m <= 128 (and K % 512 == 0, N % 4 == 0, y aligned to 8 bytes; 16 for the f32
  * form below) the three entry points take a kernel that is bound by streaming the
@@ -181,9 +184,9 @@ lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_d
 lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_dev, void *out_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
- * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each), 4 = 256x256 (8 waves;
- * K % 128 == 0, else LHIP_ERR_UNSUPPORTED), 5 = the weight-streaming kernel for
- * m <= 128 described above (LHIP_ERR_UNSUPPORTED for shapes it does not cover),
+ * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each),
+ * 5 = the weight-streaming kernel for m <= 128 described above
+ * (LHIP_ERR_UNSUPPORTED for shapes it does not cover),
  * 50 + S = the same with S slices of K (S clamped to K / 512), 120 + S = the 256x128
  * tile over S slices of K with the partial sums in the same scratch array (2 <= S <= 16,
  * K / 64 / S a whole multiple of 4, S * m * N <= 8 Mi; what the plain entry

@@ -4,24 +4,37 @@
 // The reference has no such kernel on CUDA (its QuantizedMatmul re-runs the
 // matvec once per activation row, crates/luminal_cuda/src/quantized.rs:146-164);
 // the design precedent is the Metal backend's GEMM, which dequantises a weight
-// tile into threadgroup memory (q * d rounded to the activation type) and feeds
-// the matrix unit (crates/luminal_metal/src/quantized.rs:54-61,63-199).  This
-// kernel does the same for gfx950:
+// tile into threadgroup memory and feeds the matrix unit
+// (crates/luminal_metal/src/quantized.rs:54-61,63-199).  That kernel rounds
+// q * d to the activation type first; this one keeps the weights exact:
 //   * a workgroup owns a BM x BN output tile and walks K in steps of 64 (two
 //     Q8_0 blocks);
-//   * activations go global -> registers -> LDS as bf16; weights go global
-//     (planar int8, 16-byte loads) -> registers -> dequantised q*d, rounded to
-//     bf16 (v_cvt_pk_bf16_f32, round-to-nearest-even) -> LDS;
-//   * LDS is double-buffered and the global loads run D = 4 tiles ahead in
-//     rotating register sets, so HBM/L2 latency is covered by three tiles of
-//     MFMA work; one barrier per tile separates LDS writers from readers;
-//   * each wavefront computes a (BM/WM) x (BN/WN) sub-tile with
-//     v_mfma_f32_32x32x16_bf16; LDS rows are padded by 16 bytes so the 16-byte
-//     operand reads of 8 consecutive lanes hit all banks once;
+//   * activations go global -> registers -> LDS as bf16; weight codes go global
+//     (planar int8, 16-byte loads) -> registers -> bf16 (an int8 is exact in
+//     bf16: one sign-extending byte conversion and a pack) -> LDS, and the two
+//     block scales of the K tile go to LDS as f32;
+//   * LDS is double-buffered and the global loads run D tiles ahead in
+//     rotating register sets; one barrier per tile separates LDS writers from
+//     readers;
+//   * each wavefront computes a 64 x 64 sub-tile with v_mfma_f32_32x32x16_bf16:
+//     a Q8_0 block is two chained steps into a zeroed accumulator, and the
+//     block's scale multiplies that f32 block sum, acc += d * sum, the
+//     arithmetic of the matvec kernels (quantized.rs:93-96: sumf += sumq * d);
+//     LDS rows are padded by 16 bytes so the 16-byte operand reads of 8
+//     consecutive lanes hit all banks once;
 //   * workgroups that share a weight tile (same N tile, different M tiles) get
 //     consecutive slots on the same XCD (block id modulo 8), so the weight tile
 //     is fetched from HBM once and re-read from that XCD's L2.
+// With bf16 activations every product is exact, so the only roundings are those
+// of the f32 additions (and the one of the bf16 store).  Rounding q * d to bf16
+// instead leaves a relative error of 2^-9 per weight, proportional to the sum
+// of |w x| and therefore large on every output that cancels: measured 3.5 to
+// 5.1 under max |y - t| / max(|t|, 1e-3 rms(t)) on the Llama-3-8B shapes, where
+// this kernel scores 3.9e-3 (the bf16 store alone) and 1e-4 to 5e-4 on its f32 output.
 #include <hip/hip_fp16.h>
+
+#include <type_traits>
+#include <utility>
 
 #include "common.h"
 
@@ -31,41 +44,45 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t gu32x4 __attribute__((ext_vector_type(4)));
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), expanded at compile time (register arrays
+// indexed at run time land in scratch memory).
+template <class F, int... Is>
+__device__ __forceinline__ void gm_static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void gm_static_for(F &&f) {
+    gm_static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
+}
+
 constexpr int kBK = 64;             // K per tile: two Q8_0 blocks
 constexpr int kRowBytes = 144;      // 64 bf16 + 16 bytes of padding
 
-__device__ __forceinline__ float sbyte(uint32_t w, int i) {
-    return static_cast<float>(static_cast<int8_t>((w >> (8 * i)) & 0xff));
-}
-
-// 4 packed int8 -> 4 bf16 (q * d, rounded to nearest even), as two dwords.
-__device__ __forceinline__ uint2 dequant4_bf16(uint32_t q4, float d) {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    bf16x2 lo = {static_cast<__bf16>(sbyte(q4, 0) * d), static_cast<__bf16>(sbyte(q4, 1) * d)};
-    bf16x2 hi = {static_cast<__bf16>(sbyte(q4, 2) * d), static_cast<__bf16>(sbyte(q4, 3) * d)};
-    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-}
-
+// Tile BM x BN by WM x WN waves of at most 64 x 64 each.  LDS per buffer: activations BM x 64 bf16, codes BN x 64 as
+// bf16 (rows of 144 bytes), and the BN x 2 block scales of the K tile as f32.  The lane that owns column n of a
+// 32 x 32 accumulator tile needs one scale per block: it reads both scales of the K tile with one 8-byte LDS read.
+// The per-block fma costs one v_fma per output element and block on the vector ALU, the same number of cycles the
+// block's two MFMAs take on the matrix pipe.
 // D = register prefetch depth in K tiles (D > 1 needs K % (64*D) == 0 and D even).
 // OutT = __bf16 (rounded to nearest even) or float (the accumulators as they are).
-template <int BM, int BN, int WM, int WN, int D, bool PIPE = false, typename OutT = __bf16>
+template <int BM, int BN, int WM, int WN, int D, typename OutT>
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
-                                                                   const __half *__restrict__ ds,
-                                                                   const __bf16 *__restrict__ x,
-                                                                   OutT *__restrict__ y_all, int M, int N, int K,
-                                                                   int m_tiles, int n_tiles, int swiglu, int kt_slice) {
+                                                                 const __half *__restrict__ ds,
+                                                                 const __bf16 *__restrict__ x, OutT *__restrict__ y_all,
+                                                                 int M, int N, int K, int m_tiles, int n_tiles,
+                                                                 int swiglu, int kt_slice) {
     constexpr int T = WM * WN * 64;
-    constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
-    constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 MFMA tiles per wave
-    constexpr int A_CHUNKS = BM * 8 / T;       // 16-byte chunks (8 bf16) per thread per tile
-    constexpr int B_CHUNKS = BN * 4 / T;       // 16-byte chunks (16 int8) per thread per tile
+    constexpr int TM = BM / WM, TN = BN / WN;
+    constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 accumulator tiles per wave
+    static_assert(FM >= 1 && FN >= 1 && FM <= 2 && FN <= 2, "wave tiles of at most 64 x 64");
+    constexpr int A_CHUNKS = BM * 8 / T;
+    constexpr int B_CHUNKS = BN * 4 / T;
     static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * 8 % T == 0 && BN * 4 % T == 0, "tile/thread mismatch");
-    constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
+    constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, S_BYTES = BN * 8;
+    constexpr int BUF = A_BYTES + B_BYTES + S_BYTES;
 
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x (A tile, B tile)
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 x (A tile, B tile, scales)
 
-    // Block id -> (m tile, n tile): ids that differ by 8 run on the same XCD;
-    // the m tiles of one n tile take consecutive such ids.
     int mt, nt;
     {
         const int id = blockIdx.x;
@@ -73,7 +90,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         const int n_hi = slot / m_tiles;
         mt = slot - n_hi * m_tiles;
         nt = n_hi * 8 + xcd;
-        if (nt >= n_tiles) return;  // grid is padded to a multiple of 8 n tiles
+        if (nt >= n_tiles) return;
     }
     const int m0 = mt * BM, n0 = nt * BN;
     const int tid = threadIdx.x;
@@ -81,13 +98,10 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int nblk = K >> 5;
-    // kt_slice > 0: blockIdx.y takes K tiles [kt0, kt0 + KT) and writes its f32 partial result to plane blockIdx.y
-    // of y (the caller adds the planes); 0: all of K.
     const int kt0 = kt_slice > 0 ? static_cast<int>(blockIdx.y) * kt_slice : 0;
     const int KT = kt_slice > 0 ? min(kt_slice, K / kBK - kt0) : K / kBK;
     OutT *__restrict__ y = y_all + (kt_slice > 0 ? static_cast<size_t>(blockIdx.y) * M * N : 0);
 
-    // Per-thread global sources (rows past the edge re-read the last row; their results are not stored).
     const __bf16 *a_src[A_CHUNKS];
     int a_dst[A_CHUNKS];
 #pragma unroll
@@ -99,8 +113,8 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     }
     const int8_t *b_src[B_CHUNKS];
     const uint32_t *d_src[B_CHUNKS];  // the two scales of a K tile are one aligned dword (K/32 is even)
-    int d_shift[B_CHUNKS];
     int b_dst[B_CHUNKS];
+    int s_dst[B_CHUNKS];              // where this thread leaves the row's scales, or -1: one thread in four does
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
         const int c = tid + i * T;
@@ -108,14 +122,12 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         const int grow = min(n0 + row, N - 1);
         b_src[i] = qs + static_cast<size_t>(grow) * K + q16 * 16 + kt0 * kBK;
         d_src[i] = reinterpret_cast<const uint32_t *>(ds + static_cast<size_t>(grow) * nblk) + kt0;
-        d_shift[i] = (q16 >> 1) * 16;
         b_dst[i] = row * kRowBytes + q16 * 32;
+        s_dst[i] = q16 == 0 ? row * 8 : -1;
     }
 
-    // D register sets: tile t lives in set t % D from its load until it is written to LDS.
     gu32x4 a_reg[D][A_CHUNKS], b_reg[D][B_CHUNKS];
-    uint32_t d_reg[D][B_CHUNKS];  // both f16 scale codes of the tile
-    // part p of P: the p-th share of the thread's chunks (P = 1: everything), the same split as store_tile's.
+    uint32_t d_reg[D][B_CHUNKS];
     auto load_tile = [&](int set, int kt, int p = 0, int P = 1) {
         const int k0 = min(kt, KT - 1) * kBK;  // tiles past the end re-read the last one (never used)
 #pragma unroll
@@ -128,11 +140,17 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
             d_reg[set][i] = d_src[i][k0 >> 6];
         }
     };
-    // part p of P: the p-th share of the thread's chunks (P = 1: everything).  A weight chunk (16 quants -> two
-    // 16-byte halves of bf16) counts as two units, so its unpacking can be spread over two parts.
+    // two int8 of a dword (bytes 2h, 2h+1) -> two bf16, exactly: the sign-extending byte conversion gives an f32
+    // whose upper half is the bf16 code
+    auto codes2 = [](uint32_t w, int h) {
+        const float lo = static_cast<float>(static_cast<signed char>(w >> (16 * h)));
+        const float hi = static_cast<float>(static_cast<signed char>(w >> (16 * h + 8)));
+        return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+    };
     auto store_tile = [&](int set, int buf, int p = 0, int P = 1) {
-        unsigned char *A = lds + buf * (A_BYTES + B_BYTES);
+        unsigned char *A = lds + buf * BUF;
         unsigned char *B = A + A_BYTES;
+        unsigned char *S = B + B_BYTES;
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i)
             if (i * P / A_CHUNKS == p) *reinterpret_cast<gu32x4 *>(A + a_dst[i]) = a_reg[set][i];
@@ -140,17 +158,20 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
         for (int u = 0; u < 2 * B_CHUNKS; ++u) {
             if (u * P / (2 * B_CHUNKS) != p) continue;
             const int i = u >> 1;
-            // Opaque to the optimiser: keeps the unpacking of this set here, at its use,
-            // instead of next to its loads (where it would wait for data just requested).
+            // Opaque to the optimiser: keeps the unpacking of this set here, at its use, instead of next to its loads
             asm volatile("" : "+v"(b_reg[set][i]), "+v"(d_reg[set][i]));
-            const float d = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[set][i] >> d_shift[i])));
             if ((u & 1) == 0) {
-                const uint2 w0 = dequant4_bf16(b_reg[set][i].x, d), w1 = dequant4_bf16(b_reg[set][i].y, d);
-                gu32x4 lo = {w0.x, w0.y, w1.x, w1.y};
+                const gu32x4 lo = {codes2(b_reg[set][i].x, 0), codes2(b_reg[set][i].x, 1), codes2(b_reg[set][i].y, 0),
+                                   codes2(b_reg[set][i].y, 1)};
                 *reinterpret_cast<gu32x4 *>(B + b_dst[i]) = lo;
+                if (s_dst[i] >= 0) {
+                    const float d0 = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[set][i] & 0xffffu)));
+                    const float d1 = __half2float(__ushort_as_half(static_cast<unsigned short>(d_reg[set][i] >> 16)));
+                    *reinterpret_cast<float2 *>(S + s_dst[i]) = make_float2(d0, d1);
+                }
             } else {
-                const uint2 w2 = dequant4_bf16(b_reg[set][i].z, d), w3 = dequant4_bf16(b_reg[set][i].w, d);
-                gu32x4 hi = {w2.x, w2.y, w3.x, w3.y};
+                const gu32x4 hi = {codes2(b_reg[set][i].z, 0), codes2(b_reg[set][i].z, 1), codes2(b_reg[set][i].w, 0),
+                                   codes2(b_reg[set][i].w, 1)};
                 *reinterpret_cast<gu32x4 *>(B + b_dst[i] + 16) = hi;
             }
         }
@@ -164,55 +185,75 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // MFMA operand addresses inside a tile: lane l reads 8 consecutive k of row (l % 32), k group (l / 32).
     const int frag_off = (lane & 31) * kRowBytes + (lane >> 5) * 16;
-    auto compute_tile = [&](int buf) {
-        const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
-        const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
+    // One K tile: two blocks of FM x FN slots; a slot is the two chained MFMAs of one accumulator tile's block sum.
+    // The scheduler, left alone, issues every MFMA of the K tile first and every fma after (eight block sums live:
+    // spills), so the order is fixed with scheduling fences: the sixteen fmas of the previous slot's block sum are
+    // issued in two halves behind the two MFMAs of this slot and run on the vector ALU while the matrix pipe
+    // works; the last slot's sum of a K tile is carried into the next tile (`pend`, zero before the first).  With STAGE the
+    // dequantise-and-store of the next tile and the global loads of the tile after that are dealt out over the
+    // slots.  The operand fragments of block 1 are requested during block 0 as their registers fall free (row i's
+    // A fragments after its last column, column j's B fragments after its last row).
+    f32x16 pend = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // block sum whose fmas are still to be issued
+    float pend_d = 0.f;                                                                              // and its scale
+    // Opaque to the optimiser, or it peels the first K tile off the loop (its fmas fold away) and schedules that
+    // copy with all eight block sums live.
+    asm volatile("" : "+v"(pend), "+v"(pend_d));
+    auto k_tile = [&](int buf, bool stage, int set, int next_buf, int load_set, int load_kt) {
+        const unsigned char *A = lds + buf * BUF + (wm * TM) * kRowBytes + frag_off;
+        const unsigned char *B = lds + buf * BUF + A_BYTES + (wn * TN) * kRowBytes + frag_off;
+        const unsigned char *S = lds + buf * BUF + A_BYTES + B_BYTES + (wn * TN + (lane & 31)) * 8;
+        bf16x8 af[2][2][FM], bfr[2][2][FN];  // [block][k step][tile]
+        auto load_a = [&](int b, int i) {
 #pragma unroll
-        for (int kk = 0; kk < kBK / 16; ++kk) {
-            bf16x8 af[FM], bfr[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const bf16x8 *>(A + i * 32 * kRowBytes + kk * 32);
-#pragma unroll
-            for (int j = 0; j < FN; ++j) bfr[j] = *reinterpret_cast<const bf16x8 *>(B + j * 32 * kRowBytes + kk * 32);
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
-    };
-
-    // Pipelined form of compute_tile + store_tile: the operand fragments of step kk+1 are requested before the
-    // MFMAs of step kk, and the dequantise-and-store of the next tile is dealt out over the four steps so its VALU
-    // and LDS-write work sits between the MFMAs instead of after them (measured: +10 % on the large shapes).
-    // The global loads of the tile after next are dealt out the same way: issued all at once at the top of a step
-    // by all eight waves, they fill the memory pipeline's queue (48 KiB per K tile at 64 B/clk is ~770 cycles) and
-    // the later waves sit in their load instructions for ~1000 cycles while the first wave of each SIMD runs its
-    // MFMAs alone; the two waves of a SIMD then work one after the other instead of side by side.
-    auto compute_and_store = [&](int buf, int set, int next_buf, int load_set, int load_kt) {
-        const unsigned char *A = lds + buf * (A_BYTES + B_BYTES) + (wm * TM) * kRowBytes + frag_off;
-        const unsigned char *B = lds + buf * (A_BYTES + B_BYTES) + A_BYTES + (wn * TN) * kRowBytes + frag_off;
-        bf16x8 af[2][FM], bfr[2][FN];
-        auto load_frags = [&](int kk, int to) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i) af[to][i] = *reinterpret_cast<const bf16x8 *>(A + i * 32 * kRowBytes + kk * 32);
-#pragma unroll
-            for (int j = 0; j < FN; ++j) bfr[to][j] = *reinterpret_cast<const bf16x8 *>(B + j * 32 * kRowBytes + kk * 32);
+            for (int s = 0; s < 2; ++s)
+                af[b][s][i] = *reinterpret_cast<const bf16x8 *>(A + i * 32 * kRowBytes + (2 * b + s) * 32);
         };
-        load_frags(0, 0);
+        auto load_b = [&](int b, int j) {
 #pragma unroll
-        for (int kk = 0; kk < kBK / 16; ++kk) {
-            if (kk + 1 < kBK / 16) load_frags(kk + 1, (kk + 1) & 1);
-            store_tile(set, next_buf, kk, kBK / 16);
-            load_tile(load_set, load_kt, kk, kBK / 16);
+            for (int s = 0; s < 2; ++s)
+                bfr[b][s][j] = *reinterpret_cast<const bf16x8 *>(B + j * 32 * kRowBytes + (2 * b + s) * 32);
+        };
+        float2 sc[FN];
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+        for (int j = 0; j < FN; ++j) sc[j] = *reinterpret_cast<const float2 *>(S + j * 32 * 8);
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
-        }
+        for (int i = 0; i < FM; ++i) load_a(0, i);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) load_b(0, j);
+        gm_static_for<2 * FM * FN>([&](auto qc) __attribute__((always_inline)) {
+            constexpr int q = decltype(qc)::value;
+            constexpr int b = q / (FM * FN), r = q % (FM * FN), i = r / FN, j = r % FN;
+            constexpr int rp = (r + FM * FN - 1) % (FM * FN), ip = rp / FN, jp = rp % FN;  // the slot before this one
+            if (stage) {
+                store_tile(set, next_buf, q, 2 * FM * FN);
+                load_tile(load_set, load_kt, q, 2 * FM * FN);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 sum = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[b][0][i], bfr[b][0][j], sum, 0, 0, 0);
+            // (the empty asm statements tie each result to its place between the fences: the fences hold the machine
+            // scheduler, but arithmetic without side effects is moved past them before it ever gets there)
+            asm volatile("" : "+v"(sum));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < 8; ++v) acc[ip][jp][v] = fmaf(pend_d, pend[v], acc[ip][jp][v]);
+            asm volatile("" : "+v"(acc[ip][jp]));
+            __builtin_amdgcn_sched_barrier(0);
+            sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[b][1][i], bfr[b][1][j], sum, 0, 0, 0);
+            asm volatile("" : "+v"(sum));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 8; v < 16; ++v) acc[ip][jp][v] = fmaf(pend_d, pend[v], acc[ip][jp][v]);
+            asm volatile("" : "+v"(acc[ip][jp]));
+            if constexpr (b == 0) {  // this slot's MFMAs are issued: block 1's fragments into the registers that fell free
+                if constexpr (j == FN - 1) load_a(1, i);
+                if constexpr (i == FM - 1) load_b(1, j);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            pend = sum;
+            pend_d = b ? sc[j].y : sc[j].x;
+        });
     };
 
 #pragma unroll
@@ -223,7 +264,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
     if constexpr (D == 1) {
         for (int kt = 0; kt < KT; ++kt) {
             load_tile(0, kt + 1);
-            compute_tile(kt & 1);
+            k_tile(kt & 1, false, 0, 0, 0, 0);
             store_tile(0, (kt + 1) & 1);
             __syncthreads();
         }
@@ -233,27 +274,18 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int j = 0; j < D; ++j) {
                 // set j held tile kt+j, already in LDS: refill it with tile kt+j+D
-                if constexpr (PIPE) {
-                    compute_and_store(j & 1, (j + 1) % D, (j + 1) & 1, j, kt + j + D);
-                } else {
-                    load_tile(j, kt + j + D);
-                    // Keep the loads here, at the top of the step: if they sink towards the
-                    // LDS stores below, the wait for the tile loaded D-1 steps ago also
-                    // waits for them and the prefetch distance collapses.
-                    __builtin_amdgcn_sched_barrier(0);
-                    compute_tile(j & 1);
-                    store_tile((j + 1) % D, (j + 1) & 1);  // tile kt+j+1, loaded D-1 iterations ago
-                }
+                k_tile(j & 1, true, (j + 1) % D, (j + 1) & 1, j, kt + j + D);
                 __syncthreads();
             }
         }
     }
 
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[FM - 1][FN - 1][v] = fmaf(pend_d, pend[v], acc[FM - 1][FN - 1][v]);
+
     // Epilogue: acc element v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile.
     if constexpr (sizeof(OutT) == 2) {
         if (swiglu) {
-            // Columns are (gate, up) pairs (weight rows interleaved at load): y[row][c/2] = up * swish(gate), N/2
-            // columns of bf16.  A pair sits in neighbouring lanes; two pairs are packed into one 4-byte store.
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -302,15 +334,15 @@ constexpr int kTileSkinny = 5;        // K slices chosen by the library
 constexpr int kTileSkinnySplit = 50;  // + number of K slices
 constexpr int kTileSliced = 120;      // + number of K slices: the 256x128 tile over slices of K, then a reduction
 
-template <int BM, int BN, int WM, int WN, int D, bool PIPE, typename OutT>
+template <int BM, int BN, int WM, int WN, int D, typename OutT>
 static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
-                                 int swiglu, hipStream_t s, int slices = 1) {
+                               int swiglu, hipStream_t s, int slices = 1) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
-    const size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
-    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, PIPE, OutT>;
+    if (static_cast<int64_t>(m_tiles) * n_tiles_pad > 0x7fffffff) return LHIP_ERR_INVALID_SHAPE;  // the grid's x extent
+    const size_t lds_bytes = 2 * (static_cast<size_t>(BM + BN) * kRowBytes + static_cast<size_t>(BN) * 8);
+    auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, OutT>;
     if (lds_bytes > 64 * 1024) {
-        // Opting in to more than 64 KiB of dynamic LDS is a per-function attribute.
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     }
@@ -322,11 +354,11 @@ static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void 
     return LHIP_OK;
 }
 
-template <int BM, int BN, int WM, int WN, int D, bool PIPE = false>
-static lhip_status launch_gemm(int out, const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n,
-                               int k, hipStream_t s) {
-    return out == kOutF32 ? launch_gemm_t<BM, BN, WM, WN, D, PIPE, float>(qs, ds, x, y, m, n, k, 0, s)
-                          : launch_gemm_t<BM, BN, WM, WN, D, PIPE, __bf16>(qs, ds, x, y, m, n, k, out == kOutSwiglu, s);
+template <int BM, int BN, int WM, int WN, int D>
+static lhip_status launch_gemm(int out, const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
+                             hipStream_t s) {
+    return out == kOutF32 ? launch_gemm_t<BM, BN, WM, WN, D, float>(qs, ds, x, y, m, n, k, 0, s)
+                          : launch_gemm_t<BM, BN, WM, WN, D, __bf16>(qs, ds, x, y, m, n, k, out == kOutSwiglu, s);
 }
 
 static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
@@ -342,11 +374,6 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
     auto *ds = reinterpret_cast<const __half *>(base + q8_scale_offset(n, k));
     const int mi = static_cast<int>(m), ni = static_cast<int>(n), ki = static_cast<int>(k);
     hipStream_t s = as_stream(stream);
-    // Deep register prefetch (4 K tiles ahead) needs K to be a whole number of 4-tile rounds.
-    const bool deep = (k % (kBK * 4)) == 0;
-#define LHIP_TILE(BM, BN, WM, WN)                                                                  \
-    return deep ? launch_gemm<BM, BN, WM, WN, 4, true>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s) \
-                : launch_gemm<BM, BN, WM, WN, 1>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
     if (tile == kTileSkinny || (tile > kTileSkinnySplit && tile <= kTileSkinnySplit + 64)) {
         if (!q8_gemm_skinny_supports(mi, ni, ki, out, y_dev)) return LHIP_ERR_UNSUPPORTED;
         return q8_gemm_skinny_launch(qs, ds, x_dev, y_dev, mi, ni, ki, out, tile == kTileSkinny ? 0 : tile - kTileSkinnySplit, s);
@@ -362,19 +389,21 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
         if (slices < 2 || kt % slices != 0 || (kt / slices) % 4 != 0 || static_cast<size_t>(slices) * mi * ni > cap ||
             ni % 4 != 0 || !aligned(y_dev, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4)))
             return LHIP_ERR_UNSUPPORTED;
-        if (lhip_status st = launch_gemm_t<256, 128, 4, 2, 4, true, float>(qs, ds, x_dev, part, mi, ni, ki, 0, s, slices))
+        if (lhip_status st = launch_gemm_t<256, 128, 4, 2, 4, float>(qs, ds, x_dev, part, mi, ni, ki, 0, s, slices))
             return st;
         return q8_gemm_reduce_launch(part, y_dev, mi, ni, slices, out, s);
     }
+    // Register prefetch four (two) K tiles ahead needs K to be a whole number of 4-tile (2-tile) rounds.
+    const int depth = (k % (kBK * 4)) == 0 ? 4 : ((k % (kBK * 2)) == 0 ? 2 : 1);
+#define LHIP_TILE(BM, BN, WM, WN)                                                                          \
+    return depth == 4   ? launch_gemm<BM, BN, WM, WN, 4>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)      \
+           : depth == 2 ? launch_gemm<BM, BN, WM, WN, 2>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)      \
+                        : launch_gemm<BM, BN, WM, WN, 1>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s)
     switch (tile) {
         case 0: LHIP_TILE(256, 128, 4, 2);
         case 1: LHIP_TILE(128, 128, 2, 2);
         case 2: LHIP_TILE(128, 64, 2, 2);
         case 3: LHIP_TILE(64, 64, 2, 2);
-        case 4:  // 256x256 by eight 64x128 waves: 0.75 KiB of LDS operand reads per MFMA instead of 1; both
-                 // LDS buffers together are 144 KiB, which leaves registers for a prefetch depth of two K tiles
-            if (k % (kBK * 2) != 0) return LHIP_ERR_UNSUPPORTED;
-            return launch_gemm<256, 256, 4, 2, 2, true>(out, qs, ds, x_dev, y_dev, mi, ni, ki, s);
         default: return LHIP_ERR_UNSUPPORTED;
     }
 #undef LHIP_TILE
@@ -400,8 +429,7 @@ static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *
                 return kTileSliced + slices;
     }
     int tile = 3;
-    if (m > 128 && k % (kBK * 2) == 0 && blocks(256, 256) >= 192) tile = 4;
-    else if (m > 128 && blocks(256, 128) >= 192) tile = 0;
+    if (m > 128 && blocks(256, 128) >= 192) tile = 0;
     else if (blocks(128, 128) >= 192) tile = 1;
     else if (blocks(128, 64) >= 192) tile = 2;
     return tile;

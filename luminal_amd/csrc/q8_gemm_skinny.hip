@@ -1,29 +1,27 @@
-// Q8_0 weights x activations for up to 128 activation rows per pass (short prompts, small batches).
+// Q8_0 weights x activations for few activation rows (short prompts, small batches; up to 128 rows per pass).
 //
 // With so few activation rows the product is bound by streaming the weights, not by the matrix cores, and the
 // 128/256-row tiles of q8_gemm.hip leave most of the chip idle.  Here a workgroup owns a strip of 128 weight rows
 // (and, when the strips alone would not fill the chip, a slice of K) and streams it from HBM straight into
 // registers in matrix-core operand order:
 //
-//   * the compute waves (four of 32 weight rows, or eight of 16 for at most 64 activation rows) work in blocks of
-//     16 weight rows.  Lane (r, g) = (lane % 16, lane / 16) loads the 16 codes k = 64*group + 16*g .. +16 of row r with one 16-byte load: the A operands of two
-//     v_mfma_f32_16x16x32_bf16 steps, whose k slots (g, e) are taken to mean k = 16*g + 8*step + e.  Eight groups
-//     (512 k) per row block are in flight per wave, reloaded in place as they are consumed; the codes are
-//     dequantised (q * d rounded to bf16, as in q8_gemm.hip) one group ahead of their MFMAs, in between them.
+//   * eight compute waves of 16 weight rows each.  The int8 codes go to the matrix cores as they are (an int8 is
+//     exact in bf16); an MFMA step (v_mfma_f32_16x16x32_bf16) is one Q8_0 block, a lane supplies eight of its
+//     codes, and the block's scale multiplies the f32 block sum: acc += d * sum, the arithmetic of the matvec
+//     kernels (crates/luminal_cuda/src/quantized.rs:93-96).  Eight groups of 64 k per row block are in flight per
+//     wave, reloaded in place as they are consumed.
 //   * four more waves ("loaders") stage the activations for all the compute waves: (16*MT) x (64*G) tiles of x go
 //     through their registers into one of three LDS buffers, two tiles ahead, one barrier per tile.  The compute
 //     waves never wait for an activation load, so their in-order load counter only ever sees the weight stream.
 //     In LDS a tile is G panels of 64 k, a row of a panel 128 bytes at pitch 160 (free of bank conflicts for the
-//     16-lane x 4-group operand reads), with its eight 16-byte pieces permuted so that piece g + 4*step holds
-//     k = 16*g + 8*step .. +8: the B operand of a step is one 16-byte read.
+//     16-lane x 4-group operand reads).
+//   * activations are bf16 (the prefill GEMM: one plane per tile), or f32 / f16 held as three / two bf16 limbs
+//     whose sum is the value exactly (the f32 / f16 matmul operators for several rows: one plane and one chained
+//     MFMA per limb).  Every product is exact; the only roundings are those of the f32 additions.
 //
 // K slices write f32 partial tiles to a scratch array owned by the library (one per device, shared by every
 // call on it) and a second kernel adds them in slice order and applies the output form, so results do not depend
 // on timing.
-//
-// The same kernel with f32 or f16 activations is the f32-exact form of the f32 / f16 matmul operators for several
-// activation rows: the codes as exact bf16, x as three bf16 limbs (two for f16), the block scales applied in f32
-// (see the kernel's comment).
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
@@ -58,34 +56,19 @@ __device__ __forceinline__ void sk_static_for(F &&f) {
     sk_static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
 }
 
-// NL > 0 ("split"): f32 / f16 activations held as NL bf16 planes (see q8_gemm_skinny_kernel), at most 64 rows,
-// 64 k per panel row as before but fewer panels per tile.
-template <int MT, int NL = 0>
+// NL = bf16 planes of an activation tile (1: bf16 activations, 2: f16, 3: f32).  64 k per panel row.
+template <int MT, int NL>
 struct SkShape {
-    static constexpr bool SPLIT = NL > 0;
-    static_assert(!SPLIT || MT <= 4, "the split form takes at most 64 activation rows");
-    static constexpr int G = SPLIT ? (MT >= 4 ? 1 : (MT == 2 ? 2 : 4))
-                                   : (MT >= 8 ? 2 : 4);  // groups per activation tile; a slice is an even number of tiles
+    static_assert(NL >= 1 && NL <= 3 && (MT <= 4 || NL == 1), "three or two planes per tile: at most 64 activation rows");
+    static constexpr int G = MT >= 4 ? 1 : (MT == 2 ? 2 : 4);  // groups per activation tile; a slice is an even number of tiles
     static constexpr int PANEL = 16 * MT * kSkPitch;
     static constexpr int PLANE = G * PANEL;
-    static constexpr int STAGE = (SPLIT ? NL : 1) * PLANE;
+    static constexpr int STAGE = NL * PLANE;
     static constexpr int CHUNKS = 16 * MT * G * 8;             // pieces of 8 k per tile
     static constexpr int CH = CHUNKS / 256;                    // per loader thread
     static_assert(CHUNKS % 256 == 0 && 8 % G == 0, "tile split");
     static constexpr size_t LDS = static_cast<size_t>(kSkStages) * STAGE;
 };
-
-// Two packed int8 (half `h` of a dword) -> two bf16 of q * d, packed.  A byte is converted as unsigned (one
-// instruction), so the dword arrives biased by 128 per byte (w = q ^ 0x80808080) and the fma takes the bias out
-// again: for a finite scale (q + 128) * d - 128 * d is exact in an fma because q * d has at most 19 significant bits,
-// and the value rounded to bf16 is that of q * d itself (an infinite scale gives NaN here, not +-inf).
-__device__ __forceinline__ uint32_t sk_dequant2(uint32_t w, int h, float d, float off) {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    const float lo = fmaf(static_cast<float>((w >> (16 * h)) & 0xffu), d, off);
-    const float hi = fmaf(static_cast<float>((w >> (16 * h + 8)) & 0xffu), d, off);
-    const bf16x2 pk = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
-    return __builtin_bit_cast(uint32_t, pk);
-}
 
 // Two f32 -> NL packed bf16 pairs whose sums are the two values exactly: limb[0] the bf16 roundings, limb[1]
 // the roundings of what that left, limb[2] of what is left then (8 + 8 + 8 significant bits cover an f32, 8 + 8 the
@@ -126,26 +109,21 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
     }
 }
 
-// grid (strips of 128 weight rows, K slices); 8 / RB compute waves of RB row blocks each and four loader waves.
-// K % 512 == 0, N % 4 == 0, M <= 16 * MT.
+// grid (strips of 128 weight rows, K slices, passes of 16 * MT activation rows); eight compute waves of 16 weight
+// rows and four loader waves.  K % 512 == 0, N % 4 == 0.
 // A slice is `slice_groups` groups of 64 k (a multiple of 8); the last may be shorter (also a multiple of 8).
-// RING = groups in flight per wave and row block; a slice is a multiple of RING groups.
-//
-// XT = __bf16: the product as described above.  XT = float or __half ("split"): the f32-exact form behind the
-// f32 / f16 matmul operators for more than a few activation rows (at most 64 per pass, MT <= 4, RB = 1); its
-// compute path is the `if constexpr (SPLIT)` block below, its loaders write x as bf16 limbs whose sum is the value
-// exactly (three planes per tile for f32, two for f16, whose 11 significant bits two limbs hold; pieces in natural
-// order).
-template <int MT, int OUT, int RING, int RB, typename XT = __bf16>
-__global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
+// RING = groups in flight per wave; a slice is a multiple of RING groups.
+// XT = __bf16, __half or float: the loaders write x as NL = 1, 2 or 3 bf16 planes per tile whose sum is the value
+// exactly (an f16 has 11 significant bits, which two limbs hold; an f32's 24 take three).
+template <int MT, int OUT, int RING, typename XT>
+__global__ __launch_bounds__(12 * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
                                                              const XT *__restrict__ x, void *__restrict__ y,
                                                              float *__restrict__ part, int M, int N, int K,
                                                              int slice_groups) {
-    constexpr bool SPLIT = !std::is_same<XT, __bf16>::value;
-    constexpr int NL = SPLIT ? (sizeof(XT) == 4 ? 3 : 2) : 0;  // bf16 limbs of an activation
+    constexpr int NL = sizeof(XT) == 4 ? 3 : (std::is_same<XT, __bf16>::value ? 1 : 2);  // bf16 limbs of an activation
     using S = SkShape<MT, NL>;
     constexpr int G = S::G;
-    constexpr int CW = 8 / RB;  // compute waves, RB blocks of 16 weight rows each
+    constexpr int CW = 8;  // compute waves
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -154,8 +132,8 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
     const int g_begin = split * slice_groups;
     const int n_groups = min(slice_groups, (K >> 6) - g_begin);
     const int n_tiles = n_groups / G;
-    // split form: blockIdx.z takes 64 activation rows of the M in all (one launch streams the weights once per pass)
-    const int m_base = SPLIT ? static_cast<int>(blockIdx.z) * 64 : 0;
+    // blockIdx.z takes 16 * MT activation rows of the M in all (one launch streams the weights once per pass)
+    const int m_base = static_cast<int>(blockIdx.z) * (16 * MT);
     // With few activation rows every strip starts its walk over K at a different place (a whole number of rings):
     // the strips advance at the same pace and would otherwise all ask the same memory channels for the same k at
     // the same time (measured: 39 -> 36 us for 28672 x 4096 at 16 rows).  With many rows the strips reading the
@@ -173,8 +151,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             const int m = c / (G * 8), j = c % (G * 8);
             const int panel = j >> 3, jj = j & 7;
             src[i] = x + static_cast<size_t>(min(m_base + m, M - 1)) * K + (static_cast<size_t>(g_begin) + panel) * 64 + jj * 8;
-            // plain form: pieces permuted to its operand order; split form: natural order (a step is one Q8_0 block)
-            dst[i] = panel * S::PANEL + m * kSkPitch + (SPLIT ? jj : (jj >> 1) + 4 * (jj & 1)) * 16;
+            dst[i] = panel * S::PANEL + m * kSkPitch + jj * 16;  // pieces in natural order: an MFMA step is one Q8_0 block
         }
         constexpr int XL = sizeof(XT) == 4 ? 2 : 1;  // 16-byte loads per piece of 8 k
         sk_u32x4 xr[2][S::CH][XL];
@@ -192,7 +169,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
             unsigned char *base = sk_lds + stage * S::STAGE;
 #pragma unroll
             for (int i = 0; i < S::CH; ++i) {
-                if constexpr (!SPLIT) {
+                if constexpr (NL == 1) {
                     *reinterpret_cast<sk_u32x4 *>(base + dst[i]) = xr[slot][i][0];
                 } else {
                     float v[8];
@@ -204,7 +181,7 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
                         for (int e = 0; e < 8; ++e)
                             v[e] = __half2float(__ushort_as_half(static_cast<unsigned short>(xr[slot][i][0][e >> 1] >> (16 * (e & 1)))));
                     }
-                    constexpr int NLS = NL > 0 ? NL : 1;
+                    constexpr int NLS = NL;
                     sk_u32x4 limbs[NLS];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -246,12 +223,12 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
 
     // ---------------- compute waves
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = strip * kSkRows + wave * (16 * RB);
+    const int n0 = strip * kSkRows + wave * 16;
 
-    if constexpr (SPLIT) {
-        // ---- f32-exact form.  The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block
-        // scale is applied to the f32 sum of each block, as the matvec kernels do; only x is split, into NL bf16
-        // limbs.  An MFMA step is one Q8_0 block and a lane supplies eight of its codes; the x pieces lie in natural
+    {
+        // The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block scale is applied to
+        // the f32 sum of each block, as the matvec kernels do; only an f32 / f16 x is split, into NL bf16 limbs.
+        // An MFMA step is one Q8_0 block and a lane supplies eight of its codes; the x pieces lie in natural
         // order in LDS and a lane reads the one that matches its codes.  Two ways to get the codes:
         //  - WIDE (few activation rows, where the weight stream is what bounds the kernel): lane (r, g) requests the
         //    16 codes 16g .. 16g+15 of a group of two blocks (one 16-byte load: a row's 64 bytes are contiguous over
@@ -263,7 +240,6 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         // Per block and column block NL chained MFMAs (x2, x1, x0 for f32; exact products, 96 f32 additions; an
         // f16's x2 is zero and has no MFMA, which leaves every sum as it is) and four fmas acc += d * sum.
         constexpr bool WIDE = MT <= 2;
-        static_assert(RB == 1, "one row block per compute wave");
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         const int n_rounds = n_groups >> 2;
         const int8_t *a_ptr = qs + static_cast<size_t>(min(n0 + r, N - 1)) * K + static_cast<size_t>(g_begin) * 64 + (WIDE ? 16 : 8) * g;
@@ -395,139 +371,6 @@ __global__ __launch_bounds__((8 / RB + 4) * 64) void q8_gemm_skinny_kernel(const
         return;
     }
 
-    const int8_t *a_ptr[RB];
-    const __half *d_ptr[RB];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        const int row = min(n0 + rb * 16 + r, N - 1);
-        a_ptr[rb] = qs + static_cast<size_t>(row) * K + static_cast<size_t>(g_begin) * 64 + 16 * g;
-        d_ptr[rb] = ds + static_cast<size_t>(row) * (K >> 5) + static_cast<size_t>(g_begin) * 2;
-    }
-    const int d_shift = (g >> 1) * 16;  // a lane's 16 codes lie in block 2*group + g/2
-    const int n_rounds = n_groups >> 2;
-
-    sk_u32x4 a_reg[RING][RB], d_reg[RING / 4][RB];
-    auto load_a = [&](int u, int group) __attribute__((always_inline)) {
-        int gg = min(group, n_groups - 1) + rot;
-        if (gg >= n_groups) gg -= n_groups;
-        const size_t off = static_cast<size_t>(gg) * 64;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-            // plain, not non-temporal: an instruction takes half a 128-byte line of each of its 16 rows and the next
-            // group's takes the other half; kept in L1 the line is fetched once (30 -> 23 us for one 128 x 4096 strip)
-            a_reg[u][rb] = *reinterpret_cast<const sk_u32x4 *>(a_ptr[rb] + off);
-    };
-    auto load_d = [&](int set, int round) __attribute__((always_inline)) {
-        int rr = min(round, n_rounds - 1) + rot / 4;
-        if (rr >= n_rounds) rr -= n_rounds;
-        const size_t off = static_cast<size_t>(rr) * 8;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) d_reg[set][rb] = *reinterpret_cast<const sk_u32x4 *>(d_ptr[rb] + off);
-    };
-    // Dequantisation of ring slot `un` in sixteen pieces of two codes: piece p belongs to row block p / 8,
-    // step (p / 4) % 2, dword p / 2 of the lane's four, half p % 2.
-    float d_next[RB], off_next[RB];
-    auto dequant_piece = [&](sk_u32x4 (&to)[RB][2], int un, int p) __attribute__((always_inline)) {
-        const int rb = p >> 3, dw = (p >> 1) & 3;
-        // Opaque to the optimiser: keeps the unpacking here, at its use, instead of next to the load
-        asm volatile("" : "+v"(a_reg[un][rb]));
-        if ((p & 7) == 0) {
-            const uint32_t bits = (d_reg[un >> 2][rb][un & 3] >> d_shift) & 0xffffu;
-            d_next[rb] = __half2float(__ushort_as_half(static_cast<unsigned short>(bits)));
-            off_next[rb] = -128.f * d_next[rb];
-        }
-        if ((p & 1) == 0) a_reg[un][rb][dw] ^= 0x80808080u;
-        to[rb][(p >> 2) & 1][(p >> 1) & 1 ? 2 + (p & 1) : (p & 1)] = sk_dequant2(a_reg[un][rb][dw], p & 1, d_next[rb], off_next[rb]);
-    };
-
-    // the loop reloads in the order a0 a1 a2 a3 d0 a4 a5 a6 a7 d1: the same order here, so the counted waits of the
-    // first trip are those of the steady state
-#pragma unroll
-    for (int u = 0; u < RING; ++u) {
-        load_a(u, u);
-        if ((u & 3) == 3) load_d(u >> 2, u >> 2);
-    }
-
-    sk_f32x4 acc[RB][MT];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int cb = 0; cb < MT; ++cb) acc[rb][cb] = sk_f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // A group is UNITS = 2 * MT units (step, column block): one B operand read and two MFMAs each.  W reads are
-    // kept in flight, running ahead into the next group (whose tile was complete in LDS a barrier ago), and the
-    // next group's dequantisation is dealt out over the units, so that LDS latency and VALU work sit under MFMAs.
-    constexpr int UNITS = 2 * MT;
-    constexpr int W = UNITS < 4 ? UNITS : 4;
-    auto b_read = [&](const unsigned char *xb, int i) __attribute__((always_inline)) {
-        return *reinterpret_cast<const sk_bf16x8 *>(xb + (i % MT) * 16 * kSkPitch + (i / MT) * 64);
-    };
-    sk_u32x4 af[RB][2];  // [row block][step] of the group being multiplied, as packed bf16
-    sk_bf16x8 bw[W];
-#pragma unroll
-    for (int p = 0; p < 8 * RB; ++p) dequant_piece(af, 0, p);
-    const unsigned char *xb_cur = sk_lds + r * kSkPitch + g * 16;
-    __syncthreads();  // tiles 0 and 1 are staged
-#pragma unroll
-    for (int i = 0; i < W; ++i) bw[i] = b_read(xb_cur, i);
-    int stage = 0;
-    for (int R = 0; R < n_rounds; R += RING / 4) {
-        sk_static_for<RING>([&](auto uc) __attribute__((always_inline)) {
-            constexpr int u = decltype(uc)::value;
-            constexpr int un = (u + 1) % RING;  // ring slot of the next group
-            constexpr bool tile_ends = (u + 1) % G == 0;
-            const int gl = R * 4 + u;
-            const int stage_next = tile_ends ? (stage == 2 ? 0 : stage + 1) : stage;
-            const unsigned char *xb_next = sk_lds + stage_next * S::STAGE + ((u + 1) % G) * S::PANEL + r * kSkPitch + g * 16;
-            sk_u32x4 af_next[RB][2];
-            sk_static_for<UNITS>([&](auto ic) __attribute__((always_inline)) {
-                constexpr int i = decltype(ic)::value;
-                const sk_bf16x8 b = bw[i % W];
-                bw[i % W] = i + W < UNITS ? b_read(xb_cur, i + W) : b_read(xb_next, i + W - UNITS);
-                sk_static_for<8 * RB>([&](auto pc) __attribute__((always_inline)) {
-                    constexpr int p = decltype(pc)::value;
-                    if constexpr (p * UNITS / (8 * RB) == i) {
-                        dequant_piece(af_next, un, p);
-                        if constexpr (p == 8 * RB - 1 && (un & 3) == 3) {
-                            // the four groups of this round are unpacked: request the round after next, 256
-                            // consecutive bytes of every row back to back
-                            sk_static_for<4>([&](auto qc) __attribute__((always_inline)) {
-                                constexpr int q = decltype(qc)::value;
-                                load_a(un - 3 + q, gl + 1 - 3 + q + RING);
-                            });
-                            load_d(un >> 2, R + RING / 4 + (un >> 2));
-                        }
-                    }
-                });
-#pragma unroll
-                for (int rb = 0; rb < RB; ++rb)
-                    acc[rb][i % MT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, af[rb][i / MT]), b,
-                                                                              acc[rb][i % MT], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            });
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-                for (int st = 0; st < 2; ++st) af[rb][st] = af_next[rb][st];
-            xb_cur = xb_next;
-            if constexpr (tile_ends) {
-                stage = stage_next;
-                __syncthreads();
-            }
-        });
-    }
-
-    // ---------------- lane (r, g) holds activation row 16*cb + r and weight rows n0 + 16*rb + 4*g .. +4
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        const int n = n0 + rb * 16 + 4 * g;
-        if (n >= N) continue;  // N % 4 == 0: the four rows are in or out together
-#pragma unroll
-        for (int cb = 0; cb < MT; ++cb) {
-            const int m = cb * 16 + r;
-            if (m < M) sk_store4<OUT>(y, part, split, M, N, m, n, acc[rb][cb]);
-        }
-    }
 }
 
 // Sum of the K slices in slice order, then the output form.  One thread per four weight rows.
@@ -592,38 +435,35 @@ bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y) {
     return m >= 1 && m <= 128 && k % kSkUnit == 0 && n % 4 == 0 && aligned(y, out == kSkOutF32 ? 16 : (out == kSkOutBf16 ? 8 : 4));
 }
 
-template <int MT, int OUT, int RING, int RB>
-static lhip_status sk_launch_r(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
-                               int k, int splits, int slice_groups, hipStream_t s) {
-    auto kern = q8_gemm_skinny_kernel<MT, OUT, RING, RB>;
-    constexpr size_t lds_bytes = SkShape<MT>::LDS;
+template <typename XT>
+constexpr int sk_limbs() { return sizeof(XT) == 4 ? 3 : (std::is_same<XT, __bf16>::value ? 1 : 2); }
+
+template <int MT, int OUT, typename XT>
+static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
+                               int k, int splits, int passes, hipStream_t s) {
+    auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, XT>;
+    constexpr size_t lds_bytes = SkShape<MT, sk_limbs<XT>()>::LDS;
     if (lds_bytes > 64 * 1024)  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)));
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits)),
-                       dim3((8 / RB + 4) * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, slice_groups);
+    const int units = k / kSkUnit, per = (units + splits - 1) / splits;
+    hipLaunchKernelGGL(kern,
+                       dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits),
+                            static_cast<unsigned>(passes)),
+                       dim3(12 * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
-template <int MT, int OUT>
-static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m, int n,
-                               int k, int splits, hipStream_t s) {
-    const int units = k / kSkUnit, per = (units + splits - 1) / splits;
-    // Up to 64 activation rows: eight compute waves of 16 weight rows, two per SIMD, so that one's waits sit under
-    // the other's instructions (36.5 -> 34 us on 28672 x 4096 at 16 rows, 173 -> 156 us on lm_head).  At 128 rows the
-    // B operand reads per MFMA double that way and four waves of 32 rows are faster (58 against 62 us).
-    return sk_launch_r<MT, OUT, 8, (MT >= 8 ? 2 : 1)>(qs, ds, x, y, part, m, n, k, splits, per * 8, s);
-}
-
+// bf16 activations, at most 128 rows in one pass (one plane per tile leaves room for 128-row tiles)
 template <int MT>
 static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m,
                                 int n, int k, int splits, hipStream_t s) {
-    if (splits > 1) return sk_launch_t<MT, kSkOutPartial>(qs, ds, x, y, part, m, n, k, splits, s);
+    if (splits > 1) return sk_launch_t<MT, kSkOutPartial, __bf16>(qs, ds, x, y, part, m, n, k, splits, 1, s);
     switch (out) {
-        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16>(qs, ds, x, y, part, m, n, k, 1, s);
-        case kSkOutF32: return sk_launch_t<MT, kSkOutF32>(qs, ds, x, y, part, m, n, k, 1, s);
-        default: return sk_launch_t<MT, kSkOutSwiglu>(qs, ds, x, y, part, m, n, k, 1, s);
+        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+        case kSkOutF32: return sk_launch_t<MT, kSkOutF32, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+        default: return sk_launch_t<MT, kSkOutSwiglu, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
     }
 }
 
@@ -655,35 +495,18 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
 
 // ---- the f32-accurate ("split") form behind the f32 / f16 operators
 
-template <int MT, int OUT, typename XT>
-static lhip_status sk_launch_split_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
-                                     int k, int splits, int passes, hipStream_t s) {
-    auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, 1, XT>;
-    constexpr size_t lds_bytes = SkShape<MT, sizeof(XT) == 4 ? 3 : 2>::LDS;
-    if (lds_bytes > 64 * 1024)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds_bytes)));
-    const int units = k / kSkUnit, per = (units + splits - 1) / splits;
-    hipLaunchKernelGGL(kern,
-                       dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits),
-                            static_cast<unsigned>(passes)),
-                       dim3(12 * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
-    LHIP_CHECK_LAUNCH();
-    return LHIP_OK;
-}
-
 // m rows in all; passes of 64 rows (one: the tile height follows m).
 template <typename XT, int OUT>
 static lhip_status sk_launch_split_rows(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
                                         int k, int splits, int passes, hipStream_t s) {
     if (splits > 1) {
-        if (passes == 1 && m <= 16) return sk_launch_split_t<1, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
-        if (passes == 1 && m <= 32) return sk_launch_split_t<2, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
-        return sk_launch_split_t<4, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, passes, s);
+        if (passes == 1 && m <= 16) return sk_launch_t<1, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
+        if (passes == 1 && m <= 32) return sk_launch_t<2, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, 1, s);
+        return sk_launch_t<4, kSkOutPartial, XT>(qs, ds, x, y, part, m, n, k, splits, passes, s);
     }
-    if (passes == 1 && m <= 16) return sk_launch_split_t<1, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
-    if (passes == 1 && m <= 32) return sk_launch_split_t<2, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
-    return sk_launch_split_t<4, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+    if (passes == 1 && m <= 16) return sk_launch_t<1, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+    if (passes == 1 && m <= 32) return sk_launch_t<2, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+    return sk_launch_t<4, OUT, XT>(qs, ds, x, y, part, m, n, k, 1, passes, s);
 }
 
 bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16) {

@@ -1,32 +1,32 @@
 """Parity of the Q8_0 prefill GEMM (bf16 activations, f32 accumulate on MFMA,
 bf16 out) with the CPU oracle, through the C ABI.
 
-Bar for bf16-output paths: max |y - t| / max(|t|, rms(t)) <= 1e-2 against the f64
-truth computed from the same bf16 activations and the exactly dequantised
-weights.  (The kernel rounds q*d to bf16, an error proportional to the size of
-the whole dot product, not of its possibly cancelled result; hence rms(t) in the
-denominator.)  The norm-wise error ||y - t|| / ||t|| is held to 4e-3.
+Bar: max |y - t| / max(|t|, 1e-3 rms(t)) (conftest.rel_err, the metric of the f32
+operators) <= 1e-2 for the bf16 output and <= 2e-3 for the f32 output, against the
+f64 truth computed from the same bf16 activations and the exactly dequantised
+weights.  The kernels keep the weights exact (codes on the matrix cores, block
+scales applied in f32), so the bf16 figure is the rounding of the store alone.
 """
 import numpy as np
 import pytest
 
 torch = pytest.importorskip("torch")
 
+from conftest import rel_err  # noqa: E402
 from luminal_amd import capi, synth  # noqa: E402
 from luminal_amd.quantized import Q8Weight, QuantizedMatmulBf16  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-TOL = 1e-2
+TOL = 1e-2      # bf16 output
+TOL_F32 = 2e-3  # f32 output
 
 
 def bf16_err(y, truth):
+    """(element-wise error with the 1e-3 rms floor, norm-wise error)"""
     y = np.asarray(y, np.float64)
     t = np.asarray(truth, np.float64)
-    rms = float(np.sqrt(np.mean(t * t))) + 1e-300
-    elem = float(np.max(np.abs(y - t) / np.maximum(np.abs(t), rms)))
-    norm = float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300))
-    return elem, norm
+    return rel_err(y, t), float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300))
 
 
 def upload(qs, d):
@@ -52,17 +52,13 @@ def truth_for(oracle, qs, d, xf):
     return oracle.matmul_f64(xf, wf)
 
 
-@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3])
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (16, 512, 1024), (33, 67, 128), (130, 200, 256), (257, 129, 4096),
-                                   (128, 1024, 4096), (300, 96, 14336), (513, 600, 2048)])
+                                   (128, 1024, 4096), (300, 96, 14336), (513, 600, 2048), (70, 130, 192)])
 def test_gemm_vs_oracle_all_tiles_ragged(oracle, tile, m, n, k):
+    # K = 64 / 192: one-tile register prefetch; 128: two tiles; multiples of 256: four
     qs, d = synth.q8_0_random(n, k, seed=m + n + k)
     xf, bits = bf16_activations(oracle, m, k, seed=m * n)
-    if tile == 4 and k % 128 != 0:  # the 256x256 tile prefetches two K tiles at a time
-        with pytest.raises(capi.LhipError) as e:
-            run(upload(qs, d), bits, tile)
-        assert e.value.status == capi.LHIP_ERR_UNSUPPORTED
-        return
     y = run(upload(qs, d), bits, tile)
     assert y.shape == (m, n)
     elem, norm = bf16_err(y, truth_for(oracle, qs, d, xf))
@@ -81,7 +77,7 @@ def test_gemm_integer_exact():
     want = x.astype(np.float64) @ (qs.astype(np.float64) * np.repeat(d.astype(np.float64), 32, axis=1)).T
     want_bf16 = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).float().numpy()
     w = upload(qs, d)
-    for tile in (None, 0, 1, 2, 3, 4):
+    for tile in (None, 0, 1, 2, 3):
         assert np.array_equal(run(w, bits, tile), want_bf16), tile
 
 
@@ -100,27 +96,43 @@ def test_reference_metal_matmul_case(oracle):
     assert np.max(np.abs(y - truth) / np.maximum(np.abs(truth), 1.0)) < 2.0 ** -8
 
 
-@pytest.mark.parametrize("name,m", [("q", 128), ("k", 512), ("down", 128), ("gate", 2048), ("gate", 40), ("lm_head", 100),
-                                    ("down", 512)])
+FULL_CELLS = [(name, m) for name in ("q", "k", "v", "o", "gate", "up", "down", "lm_head") for m in (128, 512, 2048)
+              if not (name in ("v", "up") and m != 512)]  # v / up have the shapes of k / gate: one cell each
+FULL_CELLS += [("gate", 40), ("lm_head", 100), ("down", 300)]
+
+
+@pytest.mark.parametrize("name,m", FULL_CELLS)
 def test_full_size_prefill_shapes(oracle, name, m):
-    """The Llama-3-8B prefill shapes (M in {128, 512, 2048}); the oracle runs on a sample of weight rows."""
+    """Every Llama-3-8B prefill shape at M in {128, 512, 2048} (and three off-grid M); the oracle runs on a sample
+    of weight rows, the first and last forty among them."""
     n, k = synth.LLAMA3_8B_PROJ[name]
     qs, d = synth.q8_0_random(n, k, seed=300 + m)
     xf, bits = bf16_activations(oracle, m, k, seed=301)
-    y = run(upload(qs, d), bits)
+    w = upload(qs, d)
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y = QuantizedMatmulBf16().process(x, w)
     rows = np.unique(np.concatenate([np.arange(40), np.arange(n - 40, n),
-                                     np.random.default_rng(7).integers(0, n, 176)]))
+                                     np.random.default_rng(7).integers(0, n, 112)]))
+    got = y[:, torch.from_numpy(rows).to(DEV)].float().cpu().numpy()
     truth = truth_for(oracle, qs[rows], d[rows], xf)
-    elem, norm = bf16_err(y[:, rows], truth)
+    elem, norm = bf16_err(got, truth)
     assert elem < TOL and norm < 4e-3, (elem, norm)
+    # the f32 output of the same product
+    y32 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    capi.check(capi.load_library().lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k,
+                                                                torch.cuda.current_stream().cuda_stream), "f32out")
+    assert rel_err(y32[:, torch.from_numpy(rows).to(DEV)].cpu().numpy(), truth) < TOL_F32
+    del y, y32
     # zero activations give exactly zero; one-hot activation row gives the bf16-rounded weight column
     e = np.zeros((m, k), np.float32)
     e[m // 2, 77] = 1.0
-    ye = run(upload(qs, d), (e.view(np.uint32) >> 16).astype(np.uint16))
+    xe = torch.from_numpy((e.view(np.uint32) >> 16).astype(np.uint16).view(np.int16)).to(DEV).view(torch.bfloat16)
+    ye = QuantizedMatmulBf16().process(xe, w)
     col = (qs[:, 77].astype(np.float32) * d[:, 77 // 32].astype(np.float32))
     want = torch.from_numpy(col).to(torch.bfloat16).float().numpy()
-    assert np.array_equal(ye[m // 2], want)
-    assert not ye[np.arange(m) != m // 2].any()
+    assert np.array_equal(ye[m // 2].float().cpu().numpy(), want)
+    ye[m // 2] = 0
+    assert not bool(ye.any())
 
 
 # ---- the weight-streaming kernel for at most 128 activation rows (K % 512 == 0, N % 4 == 0): tile id 5 lets
@@ -146,7 +158,7 @@ def test_weight_streaming_gemm_vs_oracle(oracle, m, n, k):
     y32 = torch.full((m, n), float("nan"), device=DEV)
     capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st), "f32out")
     elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
-    assert elem < TOL and norm < 4e-3, (elem, norm)
+    assert elem < TOL_F32 and norm < 1e-5, (elem, norm)
     auto = run(w, bits, SKINNY_AUTO)
     assert np.array_equal(auto, y32.to(torch.bfloat16).float().cpu().numpy())
     for slices in (1, 2, 3, 8):
@@ -229,7 +241,7 @@ def test_k_sliced_tiled_gemm(oracle):
     y32 = torch.full((m, n), float("nan"), device=DEV)
     capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st), "f32out")
     elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
-    assert elem < TOL and norm < 4e-3, (elem, norm)
+    assert elem < TOL_F32 and norm < 1e-5, (elem, norm)
     auto = run(w, bits)
     assert np.array_equal(auto, y32.to(torch.bfloat16).float().cpu().numpy())
     assert np.array_equal(auto, run(w, bits, 120 + 8)) and np.array_equal(auto, run(w, bits))
@@ -271,7 +283,7 @@ def test_gemm_argument_errors():
 @pytest.mark.parametrize("m,n,k", [(70, 150, 512), (300, 700, 1024), (513, 600, 2048)])
 def test_f32_output_is_the_unrounded_accumulator(oracle, m, n, k):
     """lhip_q8_0_matmul_bf16_f32out: same kernel, accumulators stored as f32 — rounding them gives the bf16 form bit
-    for bit, and they sit within the bf16-path bar of the f64 truth."""
+    for bit, and they sit within the f32 bar of the f64 truth."""
     lib = capi.load_library()
     qs, d = synth.q8_0_random(n, k, seed=m + n)
     xf, bits = bf16_activations(oracle, m, k, seed=3)
@@ -284,7 +296,7 @@ def test_f32_output_is_the_unrounded_accumulator(oracle, m, n, k):
     assert lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st) == 0
     assert torch.equal(y32.to(torch.bfloat16), y16)
     elem, norm = bf16_err(y32.cpu().numpy(), truth_for(oracle, qs, d, xf))
-    assert elem < TOL and norm < 4e-3, (elem, norm)
+    assert elem < TOL_F32 and norm < 1e-5, (elem, norm)
     assert lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr() + 2, m, n, k,
                                             st) == capi.LHIP_ERR_MISALIGNED
 
