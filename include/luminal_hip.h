@@ -246,6 +246,15 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
                                 const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                 int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream);
 
+/* The intermediates of the last lhip_mxfp4_moe_bf16 call that used this workspace with the same (t, h, i, e, topk),
+ * per routed entry r = t*topk + s: act_dev (t*topk, i) f32 = up * swish(gate) as the down projection consumed it
+ * (a bf16 value, held in the workspace as two fp8 numbers and a block scale: decoded exactly), down_dev (t*topk, h)
+ * f32 = that entry's down projection before the weighted sum.  Either pointer may be NULL.  No counterpart in the
+ * reference; it lets a caller check each of the layer's two matmuls against its own inputs, since the rounding of
+ * the activations to bf16 between them makes the end-to-end result a discontinuous function of the first one. */
+lhip_status lhip_mxfp4_moe_read_intermediates(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
+                                              int64_t h, int64_t i, int64_t e, int64_t topk, void *stream);
+
 /* ---- the operators around the matmuls in the Llama-3 decode loop (f32) --------
  * What the reference assembles from primitive ops in examples/llama/src/model.rs,
  * as single kernels.  Positions live in device memory (pos_dev) so that a decode

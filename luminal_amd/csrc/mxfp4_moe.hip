@@ -19,10 +19,14 @@
 // bf16 activations are not an MFMA input format here, so each activation is
 // split exactly into two fp8 numbers: per 32-block, scale 2^s with
 // max|x|/2^s in [128, 256); hi = fp8(x/2^s) keeps the top 4 significant bits,
-// lo = fp8(x/2^s - hi) the remaining 4 of bf16's 8 (exact down to 2^-10 of the
-// block maximum).  Two MFMAs (hi, lo) per weight fragment then give the exact
-// sum of exact products in f32, which is closer to the f32 semantics than a
-// bf16 MFMA over rounded weights would be.
+// lo = fp8(32 (x/2^s - hi)) the remaining 4 of bf16's 8, multiplied with the
+// block scale 2^(s-5): the residual is at most 8, so 32 times it stays inside
+// fp8's range while its last bit stays above fp8's smallest step for every
+// element down to 2^-14 of the block maximum (smaller ones are off by at most
+// 2^-22 of the maximum; without the gain of 32 the bounds were 2^-9 and 2^-17,
+// which shows on elements far below the block's scale).  Two MFMAs (hi, lo) per
+// weight fragment then give the exact sum of exact products in f32, which is
+// closer to the f32 semantics than a bf16 MFMA over rounded weights would be.
 #include "common.h"
 
 #include <type_traits>
@@ -35,6 +39,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t mu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kChunk = 128;      // K elements per MFMA
+constexpr int kLoShift = 5;      // the lo plane of an activation is held times 2^5 and multiplied with block scale - 5
+constexpr float kLoGain = 32.f;
 constexpr int kARow = 160;       // LDS bytes per activation row of a chunk: 128 fp8 + 32 padding (with 16 the fragment reads,
                                  // lane (r, g) at r * pitch + 16 g, take twice as long: measured 8.0 against 4.3 cycles per read)
 
@@ -211,7 +217,7 @@ __device__ __forceinline__ void mx_quantize_act_item(size_t idx, const __bf16 *_
     float inv = 1.0f;
     if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
         const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);  // biased exponent (0 = subnormal)
-        e = max(ex - 7, 1);                                                       // e8m0 code of 2^s
+        e = max(ex - 7, kLoShift + 1);                                                       // e8m0 code of 2^s
         inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);              // 2^-s, exact
     }
     uint32_t ph[2], pl[2];
@@ -222,8 +228,8 @@ __device__ __forceinline__ void mx_quantize_act_item(size_t idx, const __bf16 *_
         h = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, h, true);
         const float r0 = a0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), r1 = a1 - __builtin_amdgcn_cvt_f32_fp8(h, 1);
         const float r2 = a2 - __builtin_amdgcn_cvt_f32_fp8(h, 2), r3 = a3 - __builtin_amdgcn_cvt_f32_fp8(h, 3);
-        int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, 0, false);
-        l = __builtin_amdgcn_cvt_pk_fp8_f32(r2, r3, l, true);
+        int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0 * kLoGain, r1 * kLoGain, 0, false);
+        l = __builtin_amdgcn_cvt_pk_fp8_f32(r2 * kLoGain, r3 * kLoGain, l, true);
         ph[j] = static_cast<uint32_t>(h);
         pl[j] = static_cast<uint32_t>(l);
     }
@@ -449,7 +455,7 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
             const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
             const int sb = static_cast<int>(bs[set].s[f]);
             acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[i][f], 0, 4, 0, sa, 0, sb);
-            acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa, 0, sb);
+            acc[i][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[i][f], 0, 4, 0, sa - kLoShift, 0, sb);
             // Pin the accumulation here: nothing else reads acc until the epilogue, and
             // without this the optimiser sinks every MFMA of the unrolled pipeline to its
             // end, keeping the fragments of all its steps alive.
@@ -552,13 +558,13 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
                     float inv = 1.0f;
                     if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
                         const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);
-                        e = max(ex - 7, 1);
+                        e = max(ex - 7, kLoShift + 1);
                         inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);
                     }
                     const float s0 = a[0] * inv, s1 = a[1] * inv;
                     const int h = __builtin_amdgcn_cvt_pk_fp8_f32(s0, s1, 0, false);
                     const float r0 = s0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), r1 = s1 - __builtin_amdgcn_cvt_f32_fp8(h, 1);
-                    const int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, 0, false);
+                    const int l = __builtin_amdgcn_cvt_pk_fp8_f32(r0 * kLoGain, r1 * kLoGain, 0, false);
                     const size_t at = static_cast<size_t>(row0 + m) * g.q_kp + b * 32 + r;
                     g.q_hi[at] = static_cast<uint8_t>(h);
                     g.q_hi[at + 16] = static_cast<uint8_t>(h >> 8);
@@ -710,7 +716,7 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
             const int sb = bs[set].valid ? static_cast<int>(bs[set].s[f] >> s_shift) : 127;  // the matrix core reads byte 0
             const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
             acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc[f], 0, 4, 0, sa, 0, sb);
-            acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[f], 0, 4, 0, sa, 0, sb);
+            acc[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc[f], 0, 4, 0, sa - kLoShift, 0, sb);
             asm volatile("" : "+a"(acc[f]));
         }
     };
@@ -752,12 +758,12 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
                 float inv = 1.0f;
                 if (amax > 0.f && amax < __uint_as_float(0x7f800000u)) {
                     const int ex = static_cast<int>((__float_as_uint(amax) >> 23) & 0xff);
-                    e = max(ex - 7, 1);
+                    e = max(ex - 7, kLoShift + 1);
                     inv = __uint_as_float(static_cast<uint32_t>(254 - e) << 23);
                 }
                 const float s0 = a[v] * inv;
                 const int h = __builtin_amdgcn_cvt_pk_fp8_f32(s0, 0.f, 0, false);
-                const int l = __builtin_amdgcn_cvt_pk_fp8_f32(s0 - __builtin_amdgcn_cvt_f32_fp8(h, 0), 0.f, 0, false);
+                const int l = __builtin_amdgcn_cvt_pk_fp8_f32((s0 - __builtin_amdgcn_cvt_f32_fp8(h, 0)) * kLoGain, 0.f, 0, false);
                 const size_t at = static_cast<size_t>(row0 + m) * g.q_kp + b * 32 + half + r;
                 g.q_hi[at] = static_cast<uint8_t>(h);
                 g.q_lo[at] = static_cast<uint8_t>(l);
@@ -822,6 +828,35 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     o[1] = static_cast<__bf16>(a.y);
     o[2] = static_cast<__bf16>(a.z);
     o[3] = static_cast<__bf16>(a.w);
+}
+
+// What the two GEMMs of the last layer pass left in the workspace, per routed entry r = t*topk + s (not per slot):
+// act[r][k] = the SwiGLU activation as the down GEMM consumed it, (hi + lo) * 2^(scale - 127) of its two fp8
+// planes, and down[r][h] = the down projection's f32 row.  Entries whose expert id was invalid give zeros.
+__global__ __launch_bounds__(256) void moe_read_intermediates_kernel(const int *__restrict__ slot_of,
+                                                                     const uint8_t *__restrict__ a_hi,
+                                                                     const uint8_t *__restrict__ a_lo,
+                                                                     const uint8_t *__restrict__ a_sc,
+                                                                     const float *__restrict__ out, float *__restrict__ act,
+                                                                     float *__restrict__ down, int R, int I, int Ip, int H) {
+    const int r = blockIdx.x;
+    if (r >= R) return;
+    const int slot = slot_of[r];
+    if (act) {
+        for (int k = threadIdx.x; k < I; k += 256) {
+            float v = 0.f;
+            if (slot >= 0) {
+                const size_t at = static_cast<size_t>(slot) * Ip + k;
+                const float hi = __builtin_amdgcn_cvt_f32_fp8(a_hi[at], 0), lo = __builtin_amdgcn_cvt_f32_fp8(a_lo[at], 0);
+                const uint32_t e = a_sc[static_cast<size_t>(slot) * (Ip / 32) + (k >> 5)];
+                v = (hi + lo * (1.0f / kLoGain)) * __uint_as_float(e << 23);  // e > kLoShift: the quantiser's floor
+            }
+            act[static_cast<size_t>(r) * I + k] = v;
+        }
+    }
+    if (down)
+        for (int h = threadIdx.x; h < H; h += 256)
+            down[static_cast<size_t>(r) * H + h] = slot >= 0 ? out[static_cast<size_t>(slot) * H + h] : 0.f;
 }
 
 // ---------------------------------------------------------------------------
@@ -1018,6 +1053,21 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
                            w.plan.slot_of, wts_dev, static_cast<__bf16 *>(y_dev), T, H, topk_i);
         LHIP_CHECK_LAUNCH();
     }
+    return LHIP_OK;
+}
+
+lhip_status lhip_mxfp4_moe_read_intermediates(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
+                                              int64_t h, int64_t i, int64_t e, int64_t topk, void *stream) {
+    if (!workspace_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_moe_shape(t, h, i, e, topk)) return s;
+    if (!aligned(workspace_dev, 256) || !aligned(act_dev, 4) || !aligned(down_dev, 4)) return LHIP_ERR_MISALIGNED;
+    if (!act_dev && !down_dev) return LHIP_OK;
+    MoeWorkspace w = carve(const_cast<void *>(workspace_dev), t, h, i, e, topk);
+    const int R = static_cast<int>(t * topk);
+    hipLaunchKernelGGL(moe_read_intermediates_kernel, dim3(static_cast<unsigned>(R)), dim3(256), 0, as_stream(stream),
+                       w.plan.slot_of, w.a_hi, w.a_lo, w.a_sc, w.out, act_dev, down_dev, R, static_cast<int>(i),
+                       static_cast<int>(pad128(i)), static_cast<int>(h));
+    LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 

@@ -94,4 +94,19 @@ class MoEExperts:
                                          sel.contiguous().data_ptr(), wts.contiguous().data_ptr(), y.data_ptr(), t,
                                          self.h, self.i, self.e, topk, self._ws.data_ptr(), _stream())
         capi.check(st, "lhip_mxfp4_moe_bf16")
+        self._last = (t, topk)
         return y
+
+    def intermediates(self):
+        """(act (T*topk, I) f32, down (T*topk, H) f32) of the last `process` call: the SwiGLU activations as the down
+        projection consumed them and every routed entry's down projection (lhip_mxfp4_moe_read_intermediates)."""
+        lib = capi.load_library()
+        t, topk = self._last
+        dev = self._ws.device
+        act = torch.empty((t * topk, self.i), dtype=torch.float32, device=dev)
+        down = torch.empty((t * topk, self.h), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            st = lib.lhip_mxfp4_moe_read_intermediates(self._ws.data_ptr(), act.data_ptr(), down.data_ptr(), t, self.h,
+                                                       self.i, self.e, topk, _stream())
+        capi.check(st, "lhip_mxfp4_moe_read_intermediates")
+        return act, down

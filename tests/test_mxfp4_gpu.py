@@ -2,16 +2,38 @@
 
 MXFP4 and MoE do not exist in the reference, so its tests hold nothing for
 them: parity here is against the oracle only (pinned by the OCP MX value table
-and closed forms, see tests/test_oracle.py).  Bars: storage and dequantised
-weights bit-exact; the bf16-output layer within 1e-2 (max |y-t| / max(|t|,
-rms(t))) and 4e-3 norm-wise of the f64 truth that rounds the SwiGLU activations
-to bf16 like the kernel pipeline does.
+and closed forms, see tests/test_oracle.py).  Storage and dequantised weights
+are bit-exact.
+
+The layer's two matmuls are checked one by one, each against the f64 product of
+ITS OWN inputs (lhip_mxfp4_moe_read_intermediates hands back what the first one
+produced and the second consumed).  End to end the layer is a discontinuous
+function of its first matmul, because the SwiGLU activations are rounded to bf16
+in between: where the GPU's f32 value and the oracle's fall on different sides of
+a rounding boundary, that token's outputs move by a bf16 step of one activation.
+
+What bounds each matmul is the matrix instruction itself.
+v_mfma_scale_f32_16x16x128_f8f6f4 does not add its 128 products exactly: it
+aligns them to the largest and keeps about 19 bits below it (measured with a
+one-instruction probe: exact while the operands span at most seven binades, off
+by up to 2^-13 of the largest product when one operand is 2^12 times the rest).
+So every output carries an absolute error of up to 2^-12 * (largest |product| of
+each 128-wide chunk, summed over the chunks), whatever its own size, and outputs
+that cancel to far below that fail any purely relative bar: under
+max |y-t| / max(|t|, 1e-3 rms) the benchmark layer scores 3e-2 to 4e-2 (bf16
+output) where the bar for bf16 outputs is 1e-2; with the floor at 1e-2 rms it
+scores 7e-3.  The tests therefore hold every output to
+    |y - t| <= tol * |t| + 2^-11 * sum_chunks max_k |a_k w_k|
+with tol = 2^-8 for bf16 results (one rounding) and 1e-5 for the f32 rows of the
+down projection, i.e. exactness up to what the instruction drops, and the
+end-to-end result to 4e-3 norm-wise.
 """
 import numpy as np
 import pytest
 
 torch = pytest.importorskip("torch")
 
+from conftest import rel_err  # noqa: E402
 from luminal_amd import capi, synth  # noqa: E402
 from luminal_amd.moe import Mxfp4Weight, MoEExperts, route_topk  # noqa: E402
 
@@ -19,12 +41,60 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def bf16_err(y, truth):
+def norm_err(y, truth):
     y = np.asarray(y, np.float64)
     t = np.asarray(truth, np.float64)
-    rms = float(np.sqrt(np.mean(t * t))) + 1e-300
-    return (float(np.max(np.abs(y - t) / np.maximum(np.abs(t), rms))),
-            float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300)))
+    return float(np.linalg.norm(y - t) / (np.linalg.norm(t) + 1e-300))
+
+
+def chunk_bound(a, w):
+    """2^-11 * sum over 128-wide chunks of k of max_k |a_k w[:, k]|, per row of w: what the block-scaled matrix
+    instructions of a chunk (one for each fp8 half of the activations) may drop from each output (see the module
+    docstring; measured: up to 0.8 of this bound on these layers, 0.25 on the benchmark layer)."""
+    a = np.abs(np.asarray(a, np.float64))
+    w = np.abs(np.asarray(w, np.float64))
+    k = a.size
+    pad = (-k) % 128
+    terms = np.pad(w * a[None, :], ((0, 0), (0, pad)))
+    return 2.0 ** -11 * terms.reshape(w.shape[0], -1, 128).max(axis=2).sum(axis=1)
+
+
+def check_stages(oracle, layer, xf, w_gu, w_dn, sel, wts, y, tokens=None):
+    """Every matmul of the layer against the f64 product of its own inputs (see the module docstring).
+    Returns the three errors under conftest.rel_err, for the record."""
+    t_all, topk = sel.shape
+    tokens = np.arange(t_all) if tokens is None else np.asarray(tokens)
+    act_d, down_d = layer.intermediates()
+    torch.cuda.synchronize()
+    i_dim = w_dn.shape[2]
+    rows = (tokens[:, None] * topk + np.arange(topk)[None, :]).reshape(-1)
+    idx = torch.from_numpy(rows).to(act_d.device)
+    act = act_d[idx].cpu().numpy()
+    down = down_d[idx].cpu().numpy()
+    assert not (act.view(np.uint32) & 0xffff).any()  # bf16 values: the two-fp8 form held them exactly
+    want_act = np.empty((len(rows), i_dim))
+    want_down = np.empty((len(rows), w_dn.shape[1]))
+    for j, r in enumerate(rows):
+        tok, e = r // topk, sel[r // topk, r % topk]
+        x64 = xf[tok].astype(np.float64)
+        wg, wu = w_gu[e, :i_dim].astype(np.float64), w_gu[e, i_dim:].astype(np.float64)
+        g, u = wg @ x64, wu @ x64
+        sw = g / (1.0 + np.exp(-g))
+        want_act[j] = u * sw
+        # d(act) <= |swish(g)| d(u) + |u| |swish'(g)| d(g) + d(u) |swish'| d(g), |swish'| <= 1.1; then one bf16 rounding
+        bu, bg = chunk_bound(x64, wu), chunk_bound(x64, wg)
+        slack = np.abs(sw) * bu + 1.1 * np.abs(u) * bg + 1.1 * bu * bg
+        # the two-fp8 form of the result: exact down to 2^-14 of its 32-column block's maximum, 2^-21 of it below that
+        blk_max = np.abs(np.pad(want_act[j], (0, (-i_dim) % 32))).reshape(-1, 32).max(axis=1)
+        slack = slack + 2.0 ** -21 * np.repeat(blk_max, 32)[:i_dim]
+        assert np.all(np.abs(act[j] - want_act[j]) <= 2.0 ** -8 * (np.abs(want_act[j]) + slack) + slack + 1e-30), ("act", r)
+        a64 = act[j].astype(np.float64)
+        want_down[j] = w_dn[e].astype(np.float64) @ a64
+        assert np.all(np.abs(down[j] - want_down[j]) <= 1e-5 * np.abs(want_down[j]) + chunk_bound(a64, w_dn[e]) + 1e-30), ("down", r)
+    # the weighted sum of the GPU's own down rows, rounded once to bf16
+    want_y = (wts[tokens].astype(np.float64)[:, :, None] * down.reshape(len(tokens), topk, -1).astype(np.float64)).sum(axis=1)
+    assert rel_err(y[tokens], want_y) < 1e-2
+    return rel_err(act, want_act), rel_err(down, want_down), rel_err(y[tokens], want_y)
 
 
 @pytest.mark.parametrize("n,k", [(1, 32), (5, 96), (64, 2880), (300, 128)])
@@ -111,8 +181,8 @@ def test_moe_small_layers_vs_oracle(oracle, t, e, h, i, topk):
     layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=t + e + h)
     xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t * 7 + 1, scale=0.05)
     truth = oracle.moe_forward(xf, w_gu, w_dn, sel, wts, act_bf16=True)
-    elem, norm = bf16_err(y, truth)
-    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+    assert norm_err(y, truth) < 4e-3
+    check_stages(oracle, layer, xf, w_gu, w_dn, sel, wts, y)
 
 
 def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
@@ -127,8 +197,8 @@ def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
     sel, wts = route_topk(torch.from_numpy(logits).to(DEV), topk)
     y = layer.process(torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16), sel, wts)
     truth = oracle.moe_forward(xf, w_gu, w_dn, sel.cpu().numpy(), wts.cpu().numpy(), act_bf16=True)
-    elem, norm = bf16_err(y.float().cpu().numpy(), truth)
-    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+    assert norm_err(y.float().cpu().numpy(), truth) < 4e-3
+    check_stages(oracle, layer, xf, w_gu, w_dn, sel.cpu().numpy(), wts.cpu().numpy(), y.float().cpu().numpy())
 
 
 @pytest.mark.parametrize("t", [1, 64, 1024])
@@ -139,8 +209,8 @@ def test_moe_benchmark_layer(oracle, t):
     xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t, scale=1.0)
     pick = np.unique(np.concatenate([[0, t - 1], np.random.default_rng(1).integers(0, t, 4)]))
     truth = oracle.moe_forward(xf[pick], w_gu, w_dn, sel[pick], wts[pick], act_bf16=True)
-    elem, norm = bf16_err(y[pick], truth)
-    assert elem < 1e-2 and norm < 4e-3, (elem, norm)
+    assert norm_err(y[pick], truth) < 4e-3
+    check_stages(oracle, layer, xf, w_gu, w_dn, sel, wts, y, tokens=pick)
     assert np.isfinite(y).all()
 
 
@@ -154,3 +224,6 @@ def test_moe_argument_errors():
     assert lib.lhip_mxfp4_moe_bf16(p, p, p, p, p, p, 4, 64, 48, 4, 2, p, None) == capi.LHIP_ERR_INVALID_SHAPE
     assert lib.lhip_mxfp4_moe_bf16(p + 64, p, p, p, p, p, 4, 64, 64, 4, 2, p, None) == capi.LHIP_ERR_MISALIGNED
     assert lib.lhip_moe_route_topk(p, p, p, 4, 4, 5, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_mxfp4_moe_read_intermediates(None, p, p, 4, 64, 64, 4, 2, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_mxfp4_moe_read_intermediates(p, p, p, 4, 64, 48, 4, 2, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_mxfp4_moe_read_intermediates(p, None, None, 4, 64, 64, 4, 2, None) == capi.LHIP_OK
