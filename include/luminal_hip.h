@@ -246,6 +246,19 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
                                 const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                 int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream);
 
+/* lhip_mxfp4_moe_bf16 for callers that cannot allocate a workspace (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc): no counterpart in the reference.  The workspace is a scratch array inside the
+ * library (a __device__ array of 8 MiB per device, held until the process ends); the call allocates and frees
+ * nothing.  LHIP_ERR_UNSUPPORTED when lhip_mxfp4_moe_workspace_nbytes(t, h, i, e, topk) exceeds 8 MiB (the
+ * benchmark layer, h = i = 2880 with 32 experts and top-4, fits up to t = 84).  Every call on a device shares
+ * that device's array: calls that overlap in time on one device (two streams, two host threads) race for it and must
+ * be ordered by the caller; the array keeps the last call's contents, and no call depends on them.  Same results,
+ * bit for bit, as lhip_mxfp4_moe_bf16.  lhip_init looks the array's address up for its device; otherwise the first
+ * call on a device does. */
+lhip_status lhip_mxfp4_moe_bf16_static(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                       const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                       int64_t i, int64_t e, int64_t topk, void *stream);
+
 /* The intermediates of the last lhip_mxfp4_moe_bf16 call that used this workspace with the same (t, h, i, e, topk),
  * per routed entry r = t*topk + s: act_dev (t*topk, i) f32 = up * swish(gate) as the down projection consumed it
  * (a bf16 value, held in the workspace as two fp8 numbers and a block scale: decoded exactly), down_dev (t*topk, h)

@@ -56,6 +56,7 @@ SIGNATURES = {
     "lhip_moe_route_topk": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_mxfp4_moe_workspace_nbytes": (_sz, [_i64] * 5),
     "lhip_mxfp4_moe_bf16": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp, _vp]),
+    "lhip_mxfp4_moe_bf16_static": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp]),
     "lhip_mxfp4_moe_read_intermediates": (C.c_int32, [_vp] * 3 + [_i64] * 5 + [_vp]),
     "lhip_gather_rows_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_rms_norm_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),

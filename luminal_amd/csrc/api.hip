@@ -12,6 +12,8 @@ lhip_status hip_failed(hipError_t e) {
     return LHIP_ERR_HIP;
 }
 
+lhip_status moe_static_setup();  // mxfp4_moe.hip
+
 }  // namespace lhip
 
 extern "C" {
@@ -37,7 +39,7 @@ lhip_status lhip_init(int device) {
     LHIP_HIP_TRY(hipGetDeviceCount(&count));
     if (device < 0 || device >= count) return LHIP_ERR_INVALID_SHAPE;
     LHIP_HIP_TRY(hipSetDevice(device));
-    return LHIP_OK;
+    return lhip::moe_static_setup();  // the address of the per-device scratch array behind lhip_mxfp4_moe_bf16_static
 }
 
 lhip_status lhip_malloc(void **dptr, size_t nbytes) {

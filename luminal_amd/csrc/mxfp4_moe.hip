@@ -930,6 +930,34 @@ static lhip_status launch_moe_gemm_small(const MoeGemmArgs &a, int col_blocks, i
     return LHIP_OK;
 }
 
+// Scratch memory of lhip_mxfp4_moe_bf16_static: the layer's workspace for callers that cannot allocate one.  One copy
+// per device, held until the process ends; every call of that entry point on a device shares it.
+constexpr size_t kMoeStaticBytes = size_t{8} << 20;
+static __device__ __align__(256) unsigned char scratch[kMoeStaticBytes];
+
+// Device address of `scratch` on the current device (in host code the array's name is not a device address): asked
+// for once per device, with that device current, and kept.
+static lhip_status moe_scratch_address(unsigned char **out) {
+    static unsigned char *ptrs[64] = {};
+    int dev = 0;
+    LHIP_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return LHIP_ERR_UNSUPPORTED;
+    unsigned char *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        LHIP_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+        if (!p) return LHIP_ERR_HIP;
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+    }
+    *out = p;
+    return LHIP_OK;
+}
+
+// Called by lhip_init for the device it selects, so that the first lhip_mxfp4_moe_bf16_static call finds the address.
+lhip_status moe_static_setup() {
+    unsigned char *p = nullptr;
+    return moe_scratch_address(&p);
+}
+
 static lhip_status check_moe_shape(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
     if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return LHIP_ERR_INVALID_SHAPE;
     if (E > 1024 || topk > E || T * topk > (int64_t{1} << 24)) return LHIP_ERR_INVALID_SHAPE;
@@ -1054,6 +1082,17 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         LHIP_CHECK_LAUNCH();
     }
     return LHIP_OK;
+}
+
+lhip_status lhip_mxfp4_moe_bf16_static(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                       const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                       int64_t i, int64_t e, int64_t topk, void *stream) {
+    if (lhip_status s = check_moe_shape(t, h, i, e, topk)) return s;
+    if (carve(nullptr, t, h, i, e, topk).total > kMoeStaticBytes) return LHIP_ERR_UNSUPPORTED;  // beyond the scratch array
+    unsigned char *ws = nullptr;
+    if (lhip_status s = moe_scratch_address(&ws)) return s;
+    // Nothing in the workspace has to start at zero: every piece a pass reads is written earlier in the same pass.
+    return lhip_mxfp4_moe_bf16(w_gate_up_planar, w_down_planar, x_dev, sel_dev, wts_dev, y_dev, t, h, i, e, topk, ws, stream);
 }
 
 lhip_status lhip_mxfp4_moe_read_intermediates(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
