@@ -287,7 +287,9 @@ lhip_status lhip_rms_norm_f32(const float *x_dev, const float *residual_dev, flo
                               float *y_dev, int64_t rows, int64_t dim, float eps, void *stream);
 /* Rotary embedding (adjacent pairs, model.rs:52-72) applied in place to the q and k heads
  * of fused rows qkv[tokens][(q_heads + 2*kv_heads)*head_dim] at positions *pos_dev + t, then
- * k and v appended to the caches [kv_heads][max_seq][head_dim] (model.rs:108-110). */
+ * k and v appended to the caches [kv_heads][max_seq][head_dim] (model.rs:108-110).  The caches do not grow: a
+ * position at or beyond max_seq is not appended (and the attention operators read at most max_seq rows), so the
+ * caller keeps *pos_dev + tokens <= max_seq. */
 lhip_status lhip_rope_kv_append_f32(float *qkv_dev, float *k_cache_dev, float *v_cache_dev, const int32_t *pos_dev,
                                     int64_t tokens, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
                                     int64_t max_seq, float theta, void *stream);

@@ -193,7 +193,7 @@ def llama_tensor_names(layers: int):
 
 
 def q8_load(path, cfg, device="cuda:0") -> dict:
-    """Reads a Llama GGUF (linears Q8_0, norms and embedding F32) into the weight dict of luminal_amd.llama.LlamaQ8.
+    """Reads a Llama GGUF (linears Q8_0, norms F32, embedding F32 or Q8_0) into the weight dict of luminal_amd.llama.LlamaQ8.
     Q8_0 bytes are uploaded raw and re-arranged on the device; q|k|v are row-concatenated, gate and up rows interleaved."""
     import torch
 
@@ -219,7 +219,13 @@ def q8_load(path, cfg, device="cuda:0") -> dict:
                 raise GgufError(f"{name}: expected {n}x{k} Q8_0, found {info.n_elements} {info.dtype}")
             return read_tensor(f, c, name)
 
-        w = {"embed": f32("token_embd.weight", cfg.vocab * cfg.dim).reshape(cfg.vocab, cfg.dim),
+        # the embedding table in whatever dtype the file holds it, as the reference's loader takes each tensor
+        # (loader.rs:124-131): f32 rows, or Q8_0 blocks gathered by lhip_q8_0_gather_f32 (QuantizedGather)
+        if c.tensor_infos["token_embd.weight"].dtype == "Q8_0":
+            embed = Q8Weight.from_raw(raw("token_embd.weight", cfg.vocab, cfg.dim), cfg.vocab, cfg.dim, device)
+        else:
+            embed = f32("token_embd.weight", cfg.vocab * cfg.dim).reshape(cfg.vocab, cfg.dim)
+        w = {"embed": embed,
              "out_norm": f32("output_norm.weight", cfg.dim),
              "lm_head": Q8Weight.from_raw(raw("output.weight", cfg.vocab, cfg.dim), cfg.vocab, cfg.dim, device)}
         for i in range(cfg.layers):

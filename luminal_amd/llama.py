@@ -51,7 +51,7 @@ def _s() -> int:
 
 class LlamaQ8:
     def __init__(self, cfg: LlamaConfig, weights: dict, max_seq: int, device="cuda:0"):
-        """weights: 'embed' f32 (vocab, dim); 'out_norm' f32 (dim); 'lm_head' Q8Weight (vocab, dim); and per
+        """weights: 'embed' f32 (vocab, dim) or Q8Weight (vocab, dim); 'out_norm' f32 (dim); 'lm_head' Q8Weight (vocab, dim); and per
         layer i: f'{i}.attn_norm', f'{i}.ffn_norm' f32 (dim); f'{i}.qkv' Q8Weight (qkv_rows, dim);
         f'{i}.o' (dim, dim); f'{i}.gate_up' (2*ffn, dim), gate and up rows interleaved; f'{i}.down' (dim, ffn)."""
         self.cfg, self.w, self.max_seq, self.dev = cfg, weights, max_seq, torch.device(device)
@@ -60,6 +60,7 @@ class LlamaQ8:
         self.k_cache = [torch.zeros(kv, dtype=torch.float32, device=self.dev) for _ in range(cfg.layers)]
         self.v_cache = [torch.zeros(kv, dtype=torch.float32, device=self.dev) for _ in range(cfg.layers)]
         self.pos = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        self._pos_host = 0  # host copy of the position, for the max_seq check
         self.tok = torch.zeros(1, dtype=torch.float32, device=self.dev)      # next token id, as f32
         self.tok_i = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self._bufs = {}
@@ -79,6 +80,25 @@ class LlamaQ8:
 
     def reset(self):
         self.pos.zero_()
+        self._pos_host = 0
+
+    def _room(self, n: int):
+        """The KV caches hold max_seq positions (the reference's caches grow instead, model.rs:108-110): a pass that
+        would run past them is refused here, on the host, before anything is launched."""
+        if self._pos_host + n > self.max_seq:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "LlamaQ8",
+                                 f"position {self._pos_host} + {n} tokens exceeds max_seq {self.max_seq}")
+
+    def _embed(self, tokens_f32, out, n):
+        """Embedding rows of n token ids (f32, on the device): an f32 table (crates/luminal_nn/src/embedding.rs:40-58) or
+        a Q8_0 one (QuantizedGather, crates/luminal_cuda/src/quantized.rs:170-233)."""
+        cfg, lib, e = self.cfg, self.lib, self.w["embed"]
+        if isinstance(e, Q8Weight):
+            capi.check(lib.lhip_q8_0_gather_f32(e.planar.data_ptr(), tokens_f32.data_ptr(), out.data_ptr(), n, cfg.vocab,
+                                                cfg.dim, _s()), "lhip_q8_0_gather_f32")
+        else:
+            capi.check(lib.lhip_gather_rows_f32(e.data_ptr(), tokens_f32.data_ptr(), out.data_ptr(), n, cfg.vocab,
+                                                cfg.dim, _s()), "lhip_gather_rows_f32")
 
     # ---- ops ---------------------------------------------------------------
     def _matmul(self, w: Q8Weight, x, y, m, bf16):
@@ -103,6 +123,7 @@ class LlamaQ8:
         """Runs s tokens (ids as f32 on the device) at positions pos .. pos+s-1, appends to the KV cache and
         returns the logits of the last position ((vocab,)), or of all positions ((s, vocab)).
         Does not advance the position."""
+        self._room(s)
         if bf16 and s > 1:
             return self._forward_prompt_bf16(tokens_f32, s, all_logits)
         cfg, lib, w = self.cfg, self.lib, self.w
@@ -115,8 +136,7 @@ class LlamaQ8:
         gu = self._buf("gu", (s, 2 * cfg.ffn))
         act = self._buf("act", (s, cfg.ffn))
         dn = self._buf("dn", (s, d))
-        capi.check(lib.lhip_gather_rows_f32(w["embed"].data_ptr(), tokens_f32.data_ptr(), h.data_ptr(), s, cfg.vocab,
-                                            d, _s()), "lhip_gather_rows_f32")
+        self._embed(tokens_f32, h, s)
         for i in range(cfg.layers):
             if i == 0:
                 self._norm(h, None, None, w["0.attn_norm"], n, s)
@@ -172,8 +192,7 @@ class LlamaQ8:
             capi.check(lib.lhip_q8_0_matmul_bf16_f32out(wq.planar.data_ptr(), x.data_ptr(), y.data_ptr(), m, wq.n, wq.k,
                                                         _s()), "lhip_q8_0_matmul_bf16_f32out")
 
-        capi.check(lib.lhip_gather_rows_f32(w["embed"].data_ptr(), tokens_f32.data_ptr(), h.data_ptr(), s, cfg.vocab,
-                                            d, _s()), "lhip_gather_rows_f32")
+        self._embed(tokens_f32, h, s)
         for i in range(cfg.layers):
             norm(None if i == 0 else dn, w[f"{i}.attn_norm"])       # h += previous MLP out; nb = norm(h)
             gemm(w[f"{i}.qkv"], nb, qkv, s)
@@ -230,13 +249,13 @@ class LlamaQ8:
     def forward_decode(self, token_f32: torch.Tensor):
         """One token at position pos through the fused batch-1 path; returns the logits (vocab,)."""
         cfg, lib = self.cfg, self.lib
+        self._room(1)
         if not self.fused_decode:
             return self.forward(token_f32, 1)
         if self._plans is None:
             self._build_plans()
         plans, head, h, qkv, att, act, logits = self._plans
-        capi.check(lib.lhip_gather_rows_f32(self.w["embed"].data_ptr(), token_f32.data_ptr(), h.data_ptr(), 1,
-                                            cfg.vocab, cfg.dim, _s()), "lhip_gather_rows_f32")
+        self._embed(token_f32, h, 1)
         for i, (p_qkv, p_o, p_gu, p_down) in enumerate(plans):
             p_qkv.run(h)                                   # qkv = Wqkv norm(h)
             self._attend_one(i, qkv, att)
@@ -271,15 +290,18 @@ class LlamaQ8:
         t = torch.as_tensor(np.asarray(tokens, dtype=np.float32)).to(self.dev)
         logits = self.forward(t, t.numel(), bf16=bf16)
         self._pick(logits, t.numel())
+        self._pos_host += t.numel()
         return logits
 
     def decode_step(self):
         logits = self.forward_decode(self.tok)
         self._pick(logits, 1)
+        self._pos_host += 1
         return logits
 
     def decode(self, steps: int, use_graph: bool = True):
         """Greedy decode of `steps` tokens after a prefill; returns the token ids (first = the prefill's pick)."""
+        self._room(steps)
         out = torch.empty(steps, dtype=torch.int32, device=self.dev)
         if not use_graph:
             for i in range(steps):
@@ -287,7 +309,8 @@ class LlamaQ8:
                 self.decode_step()
             return out
         if self._graph is None:
-            pos0, tok0, toki0 = self.pos.clone(), self.tok.clone(), self.tok_i.clone()
+            self._room(2)  # the warm-up step and the captured one
+            pos0, tok0, toki0, host0 = self.pos.clone(), self.tok.clone(), self.tok_i.clone(), self._pos_host
             st = torch.cuda.Stream(device=self.dev)
             st.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(st):
@@ -302,9 +325,11 @@ class LlamaQ8:
             self.pos.copy_(pos0)
             self.tok.copy_(tok0)
             self.tok_i.copy_(toki0)
+            self._pos_host = host0
         for i in range(steps):
             out[i:i + 1].copy_(self.tok_i)
             self._graph.replay()
+        self._pos_host += steps
         return out
 
 

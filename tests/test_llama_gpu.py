@@ -134,6 +134,33 @@ def test_rope_attention_swiglu_gather_argmax():
     assert int(idi.item()) == 4021 == lo.argmax_last(v) and idf.item() == 4021.0 and int(pos.item()) == pos0 + 3
 
 
+def test_attention_over_the_longest_cache():
+    """max_seq = 12000 (the operator's limit): 48 000 bytes of scores on top of the kernel's static arrays is more
+    LDS than a kernel gets without asking; three tokens at positions 11 990 .. 11 992 against a direct softmax."""
+    lib = capi.load_library()
+    rng = np.random.default_rng(8)
+    hq, hkv, hd, max_seq, S, pos0 = 4, 2, 64, 12000, 3, 11990
+    qkv = rng.standard_normal((S, (hq + 2 * hkv) * hd)).astype(np.float32)
+    kc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    vc = rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)
+    qd, kd, vd = (torch.from_numpy(a).to(DEV) for a in (qkv, kc, vc))
+    pos = torch.tensor([pos0], dtype=torch.int32, device=DEV)
+    out = torch.full((S, hq * hd), float("nan"), dtype=torch.float32, device=DEV)
+    assert lib.lhip_attention_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), pos.data_ptr(), S, hq,
+                                  hkv, hd, max_seq, s()) == 0
+    torch.cuda.synchronize()
+    q = qkv.reshape(S, hq + 2 * hkv, hd)[:, :hq].astype(np.float64)
+    want = np.empty((S, hq, hd))
+    for t in range(S):
+        for h in range(hq):
+            sc = kc[h // (hq // hkv), :pos0 + t + 1].astype(np.float64) @ q[t, h] / np.sqrt(hd)
+            p = np.exp(sc - sc.max())
+            want[t, h] = (p / p.sum()) @ vc[h // (hq // hkv), :pos0 + t + 1].astype(np.float64)
+    assert rel_err(out.cpu().numpy(), want.reshape(S, -1)) < 1e-3
+    assert lib.lhip_attention_f32(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), pos.data_ptr(), S, hq,
+                                  hkv, hd, max_seq + 1, s()) == capi.LHIP_ERR_INVALID_SHAPE
+
+
 @pytest.mark.parametrize("n", [16384, 16387, 128256, 128259, 1 << 20])
 def test_argmax_of_long_rows(n):
     """Rows long enough for the two-launch pick (partial picks over 64 workgroups, then one wave): ties in several
@@ -389,6 +416,42 @@ def test_prefill_and_decode_logits_vs_oracle(oracle, cfg):
         eng.tok_i.fill_(tok)
 
 
+def test_llama3_8b_layer_dimensions_vs_oracle(oracle):
+    """Two layers with the real Llama-3-8B dimensions (examples/llama/src/model.rs:5-14: dim 4096, 32 query and 8 KV
+    heads of 128, FFN 14336; a small vocabulary keeps the oracle's lm_head cheap): the f32 prompt pass, the bf16
+    prompt pass and fused-matvec decode steps (eager and replayed from a graph) against the numpy oracle."""
+    cfg = LlamaConfig(vocab=2048, dim=4096, layers=2, q_heads=32, kv_heads=8, ffn=14336)
+    eng, wf = build_model(oracle, cfg, seed=31, max_seq=64)
+    assert eng.fused_decode
+    rng = np.random.default_rng(5)
+    prompt = [int(t) for t in rng.integers(0, cfg.vocab, 16)]
+    kc, vc = empty_cache(cfg), empty_cache(cfg)
+    want = lo.forward(cfg, wf, prompt, kc, vc, 0)
+    got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
+    assert rel_err(got.cpu().numpy(), want) < 2e-3
+    rms = float(np.sqrt(np.mean(want * want)))
+    gotb = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True, all_logits=True)
+    assert np.max(np.abs(gotb.cpu().numpy() - want)) / rms < 5e-2  # bf16 activations through the whole stack
+    eng.reset()
+    eng.prefill(prompt)
+    tok = lo.argmax_last(want[-1])
+    assert int(eng.tok_i.item()) == tok and int(eng.pos.item()) == len(prompt)
+    for step in range(3):
+        want_step = lo.forward(cfg, wf, [tok], kc, vc, len(prompt) + step)[0]
+        logits = eng.decode_step()
+        assert rel_err(logits.cpu().numpy(), want_step) < 2e-3, step
+        tok = lo.argmax_last(want_step)
+        eng.tok.fill_(float(tok))
+        eng.tok_i.fill_(tok)
+    # greedy decode replayed from a graph picks the tokens eager stepping picks
+    eng.reset()
+    eng.prefill(prompt)
+    eager = eng.decode(6, use_graph=False).cpu().numpy()
+    eng.reset()
+    eng.prefill(prompt)
+    assert np.array_equal(eng.decode(6, use_graph=True).cpu().numpy(), eager)
+
+
 @pytest.mark.parametrize("cfg", [LlamaConfig(vocab=512, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512),
                                  LlamaConfig(vocab=700, dim=1024, layers=2, q_heads=8, kv_heads=4, ffn=1024)])
 def test_graph_replay_equals_eager_decode(oracle, cfg):
@@ -511,9 +574,11 @@ def test_prompt_pass_replays_from_a_graph():
         assert not torch.equal(other, ref)
 
 
-def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
+@pytest.mark.parametrize("embed_dtype", ["F32", "Q8_0"])
+def test_gguf_loader_gives_the_same_model(oracle, tmp_path, embed_dtype):
     """A synthetic GGUF with the reference's tensor names, read back through the loader
-    (examples/llama/src/loader.rs:99-165), must produce exactly the engine built from the same blocks."""
+    (examples/llama/src/loader.rs:99-165), must produce exactly the engine built from the same blocks; with the
+    embedding table in f32 or, as quantised checkpoints hold it, in Q8_0 (then gathered by lhip_q8_0_gather_f32)."""
     from luminal_amd import gguf
 
     cfg = LlamaConfig(vocab=256, dim=256, layers=2, q_heads=4, kv_heads=2, ffn=512)  # head_dim 64
@@ -521,6 +586,9 @@ def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
     hd = cfg.head_dim
     tensors = {"token_embd.weight": ("F32", (cfg.dim, cfg.vocab), rng.standard_normal((cfg.vocab, cfg.dim)).astype("<f4").tobytes()),
                "output_norm.weight": ("F32", (cfg.dim,), (1 + 0.05 * rng.standard_normal(cfg.dim)).astype("<f4").tobytes())}
+    if embed_dtype == "Q8_0":
+        eq, ed = synth.q8_0_random(cfg.vocab, cfg.dim, seed=499, scale_sigma=1.0)
+        tensors["token_embd.weight"] = ("Q8_0", (cfg.dim, cfg.vocab), synth.q8_0_raw_blocks(eq, ed).tobytes())
 
     def q8(name, n, k, i):
         qs, d = synth.q8_0_random(n, k, seed=500 + i, scale_sigma=float(np.sqrt(3.0 / k) / 0.8))
@@ -555,7 +623,36 @@ def test_gguf_loader_gives_the_same_model(oracle, tmp_path):
         ow[f"{i}.gate"] = wf[b + "ffn_gate.weight"].reshape(cfg.ffn, cfg.dim)
         ow[f"{i}.up"] = wf[b + "ffn_up.weight"].reshape(cfg.ffn, cfg.dim)
         ow[f"{i}.down"] = wf[b + "ffn_down.weight"].reshape(cfg.dim, cfg.ffn)
+    assert isinstance(eng.w["embed"], Q8Weight) == (embed_dtype == "Q8_0")
     prompt = [3, 200, 17, 5]
-    want = lo.forward(cfg, ow, prompt, empty_cache(cfg), empty_cache(cfg), 0)
+    kc, vc = empty_cache(cfg), empty_cache(cfg)
+    want = lo.forward(cfg, ow, prompt, kc, vc, 0)
     got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
     assert rel_err(got.cpu().numpy(), want) < 2e-3
+    gotb = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True, all_logits=True)
+    assert np.max(np.abs(gotb.cpu().numpy() - want)) / np.sqrt(np.mean(want * want)) < 5e-2
+    eng.prefill(prompt)
+    tok = lo.argmax_last(want[-1])
+    assert int(eng.tok_i.item()) == tok
+    step = lo.forward(cfg, ow, [tok], kc, vc, len(prompt))[0]
+    assert rel_err(eng.decode_step().cpu().numpy(), step) < 2e-3
+
+
+def test_running_past_max_seq_is_refused_on_the_host(oracle):
+    cfg = LlamaConfig(vocab=64, dim=128, layers=1, q_heads=2, kv_heads=1, ffn=128)
+    eng, _ = build_model(oracle, cfg, seed=3, max_seq=8)
+    with pytest.raises(capi.LhipError) as e:
+        eng.prefill(list(range(9)))
+    assert e.value.status == capi.LHIP_ERR_INVALID_SHAPE
+    eng.prefill([1, 2, 3, 4, 5, 6])
+    eng.decode_step()
+    eng.decode_step()  # position 8 = max_seq reached
+    with pytest.raises(capi.LhipError):
+        eng.decode_step()
+    with pytest.raises(capi.LhipError):
+        eng.decode(1, use_graph=False)
+    eng.reset()
+    eng.prefill([1, 2, 3])
+    with pytest.raises(capi.LhipError):
+        eng.decode(6, use_graph=False)
+    assert eng.decode(5, use_graph=False).numel() == 5

@@ -59,6 +59,24 @@ def test_every_launch_shape_grouped(oracle, cfg):
         assert rel_err(y.cpu().numpy(), truth) < TOL
 
 
+def test_longest_staged_k(oracle):
+    """K = 16384: 64 KiB of staged activations plus the reduction array is more LDS than a kernel gets without
+    asking; with and without the norm prologue, and the plain operator's kernel at the same K."""
+    k, n = 16384, 520
+    w, raw = make(n, k, 3)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(k).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    wd = dense(oracle, raw, n, k)
+    y = torch.full((n,), float("nan"), device=DEV)
+    FusedMatvec([w], [y]).run(torch.from_numpy(x).to(DEV))
+    assert rel_err(y.cpu().numpy(), oracle.matmul_f64(x[None, :], wd).reshape(-1)) < TOL
+    assert torch.equal(y, QuantizedMatmul().process(torch.from_numpy(x).to(DEV).reshape(1, k), w).reshape(-1))
+    y.fill_(float("nan"))
+    FusedMatvec([w], [y], norm_weight=torch.from_numpy(g).to(DEV), eps=1e-5).run(torch.from_numpy(x).to(DEV))
+    assert rel_err(y.cpu().numpy(), lo.rms_norm(x[None, :], g, 1e-5) @ wd.astype(np.float64).T) < TOL
+
+
 @pytest.mark.parametrize("k,n", [(4096, 6144), (1024, 200), (2048, 4096), (4096, 32768)])
 def test_rms_norm_prologue(oracle, k, n):
     w, raw = make(n, k, 5)
