@@ -30,15 +30,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# Average HBM bytes per launch of the dominant kernel over one step, from the
-# committed rocprofv3 counter runs (FETCH_SIZE scaled by the copy-kernel factor
-# 2.0, plus WRITE_SIZE); None until measured.
-TRAFFIC_PER_LAUNCH = 138310222
-# The same for the dominant kernel of the prefill GEMM set (gate/up 14336 x 4096 at M = 2048: FETCH_SIZE
-# 173 100 KiB x 2.0 + WRITE_SIZE 60 045 KiB) and for the two grouped GEMMs of the MoE layer at T = 64
-# (FETCH_SIZE 158 755 + 82 880 KiB, x 2.0; the layer's other kernels move under 2 MiB).
-GEMM_TRAFFIC_PER_LAUNCH = (2 * 173100 + 60045) * 1024
-MOE_T64_TRAFFIC = 2 * (158755 + 82880) * 1024
+# HBM bytes per launch (FETCH_SIZE scaled by the copy-kernel factor 2.0, plus WRITE_SIZE) of each section's dominant
+# kernel, copied from the committed rocprofv3 counter summaries named beside them; printed with the figure so a
+# reader can tell where it came from (they go stale when a kernel changes and the profile is not refreshed).
+TRAFFIC = {
+    "gemv": (138310222, "profiles/q8_gemv_decode_projection_set.md"),
+    "gemm": (None, "profiles/q8_gemm_prefill_set.md"),
+    "moe_t64": (2 * (158755 + 82880) * 1024, "profiles/mxfp4_moe_layer.md"),
+}
 
 
 def parse():
@@ -53,6 +52,7 @@ def parse():
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end Llama-3-8B decode section")
+    ap.add_argument("--no-sections", action="store_true", help="skip the prefill-GEMM and MoE sections of the default line")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
 
@@ -202,16 +202,52 @@ def bench_rows_f32(args):
         "dtype": "int8 codes as bf16 x f32 activations as three bf16 limbs, three products per step, block scales and sums in f32, f32 out",
         "data": "synthetic", "config": {"workload": "llama3_8b_q8_0_f32_rows_set", "m": list(ms_list)},
         "per_shape": per, "matvec_form_gate_m128_us": round(mv_us, 1),
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, 1, float> (gate/up, M=128: two passes of 64 rows in one launch)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_skinny_kernel<4, *, 8, float> (gate/up, M=128: two passes of 64 rows in one launch)",
                      "achieved": round(3 * g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(3 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "note": "achieved counts the three bf16 products issued per useful multiply-add"}}))
 
 
-def bench_prefill_gemm(args):
+def cpu_baseline_gemm(seconds: float):
+    """The reference's CPU path for the prefill GEMM at M = 128 (the only M the plan of record times on the host):
+    dequantise once, then the f32 matmul of the q/o shape (4096 x 4096), single-threaded like the reference's
+    matrixmultiply configuration, and on all host cores."""
+    import numpy as np
+
+    from luminal_amd import synth
+    from oracle import cpu_oracle
+
+    n, k, m = 4096, 4096, 128
+    qs, d = synth.q8_0_random(n, k, seed=910)
+    w = cpu_oracle.q8_0_dequant(synth.q8_0_raw_blocks(qs, d), n * k).reshape(n, k)
+    x = synth.activations(m, k, seed=911)
+    out = np.empty((m, n), np.float32)
+
+    def timed(threads, budget):
+        cpu_oracle.matmul_fast_f32(x, w, threads=threads, out=out)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            cpu_oracle.matmul_fast_f32(x, w, threads=threads, out=out)
+            reps += 1
+            if time.perf_counter() - t0 >= budget:
+                break
+        return (time.perf_counter() - t0) / reps, reps
+
+    fl = 2.0 * m * n * k
+    t1, r1 = timed(1, seconds * 0.7)
+    ncpu = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    tn, rn = timed(ncpu, seconds * 0.3)
+    return {"value": round(fl / t1 / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"q/o shape 4096 x 4096 at M = 128, f32 weights after load-time dequant, {r1} passes, "
+                      f"{t1 * 1e3:.1f} ms/pass single-threaded",
+            "all_cores": {"value": round(fl / tn / 1e12, 5), "cores": ncpu, "passes": rn, "ms_per_pass": round(tn * 1e3, 2)}}
+
+
+def bench_prefill_gemm(args, cpu_seconds=None):
     """Prefill GEMM set: the seven Llama-3-8B weight shapes in Q8_0 against bf16 activations,
     M in {128, 512, 2048}, f32 accumulation, bf16 output.  A step is one pass over all shapes at
-    all three M; weights rotate over distinct buffers."""
+    all three M; weights rotate over distinct buffers.  Returns the section (a dict)."""
     import torch
 
     from luminal_amd import capi, synth
@@ -264,28 +300,89 @@ def bench_prefill_gemm(args):
             per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
                                   "frac_mfma_bf16": round(fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                   "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
-    # dominant kernel: q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true> on the M = 2048 gate/up shape
+    # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> on the M = 2048 gate/up shape
     n, k, m = 14336, 4096, 2048
     us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5) / len(bufs["gate/up"])
     ach = 2.0 * m * n * k / us / 1e6
     value = flops_step / (wall / args.steps) / 1e12
-    print(json.dumps({
+    g128 = per["gate/up M=128"]
+    out = {
         "metric": "Q8_0 prefill GEMM TFLOP/s (MFMA utilisation), 1 GPU", "value": round(value, 1), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 weights dequantised to bf16 x bf16 activations, f32 accumulate, bf16 out", "data": "synthetic",
+        "dtype": "int8 codes as exact bf16 x bf16 activations on the matrix cores, block scales and sums in f32, bf16 out",
+        "data": "synthetic",
         "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list)},
         "per_shape": per,
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 256, 4, 2, 2, true, __bf16> (gate/up, M=2048)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> (gate/up, M=2048)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_TRAFFIC_PER_LAUNCH,
-                     "avg_launch_us": round(us, 1)}}))
+                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": TRAFFIC["gemm"][0],
+                     "traffic_source": TRAFFIC["gemm"][1], "avg_launch_us": round(us, 1)},
+        "roofline_m128": {"bound": "hbm", "kernel": "lhip::q8_gemm_skinny_kernel<8, *, 8, __bf16> (gate/up, M=128)",
+                          "achieved": g128["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g128["frac_hbm"],
+                          "traffic": None}}
+    if cpu_seconds:
+        out["cpu_baseline"] = cpu_baseline_gemm(cpu_seconds)
+    del bufs, xs, ys
+    torch.cuda.empty_cache()
+    return out
 
 
-def bench_moe(args):
+def cpu_baseline_moe(seconds: float):
+    """The oracle's expert layer (exact dequantisation, then f32-input matmuls accumulated in f64) at T = 1 and on a
+    sample of the T = 64 batch, one thread and all host cores (tokens dealt out over threads).  Eight experts are
+    built (the work per token does not depend on which experts it is routed to)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    import numpy as np
+
+    from luminal_amd import synth
+    from oracle import cpu_oracle
+
+    e, h, i, topk = 8, synth.MOE_HIDDEN, synth.MOE_INTER, synth.MOE_TOPK
+    gu_c, gu_s = synth.mxfp4_random(e * 2 * i, h, seed=920)
+    dn_c, dn_s = synth.mxfp4_random(e * h, i, seed=921)
+    w_gu = cpu_oracle.mxfp4_dequant(synth.mxfp4_raw_blocks(gu_c, gu_s), gu_c.size).reshape(e, 2 * i, h)
+    w_dn = cpu_oracle.mxfp4_dequant(synth.mxfp4_raw_blocks(dn_c, dn_s), dn_c.size).reshape(e, h, i)
+    del gu_c, gu_s, dn_c, dn_s
+    rng = np.random.default_rng(922)
+    ncpu = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    t_sample = ncpu  # tokens of the T = 64 batch that are run: one per thread in the all-cores leg
+    x = cpu_oracle.bf16_bits_to_f32(cpu_oracle.f32_to_bf16_bits(rng.standard_normal((t_sample, h)).astype(np.float32)))
+    sel, wts = cpu_oracle.moe_route(rng.standard_normal((t_sample, e)).astype(np.float32), topk)
+
+    def run(rows, threads):
+        if threads == 1:
+            cpu_oracle.moe_forward(x[rows], w_gu, w_dn, sel[rows], wts[rows], act_bf16=True)
+            return
+        with ThreadPoolExecutor(threads) as ex:
+            list(ex.map(lambda r: cpu_oracle.moe_forward(x[r:r + 1], w_gu, w_dn, sel[r:r + 1], wts[r:r + 1], act_bf16=True), rows))
+
+    def timed(rows, threads, budget):
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            run(rows, threads)
+            reps += 1
+            if time.perf_counter() - t0 >= budget:
+                break
+        return (time.perf_counter() - t0) / reps
+
+    fl_tok = 199065600.0
+    one = timed(np.arange(1), 1, seconds * 0.4)                  # T = 1, one thread
+    allc = timed(np.arange(t_sample), ncpu, seconds * 0.6)       # t_sample tokens, one per thread
+    return {"value": round(fl_tok / one / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"T = 1: one token through its 4 experts, {one * 1e3:.0f} ms single-threaded (f64 accumulation); "
+                      f"T = 64: {t_sample} of the 64 tokens, one per thread",
+            "t1_us": round(one * 1e6, 0),
+            "t64_all_cores": {"value": round(t_sample * fl_tok / allc / 1e12, 6), "cores": ncpu,
+                              "us_for_64_tokens_extrapolated": round(allc * 64 / t_sample * 1e6, 0)}}
+
+
+def bench_moe(args, cpu_seconds=None):
     """MoE workload: gpt-oss-style MXFP4 expert layer, H = I = 2880, 32 experts, top-4,
     T in {1, 64, 1024}; a step is one layer pass at each T (routing rotates so T = 1 streams
-    different experts from HBM every pass)."""
+    different experts from HBM every pass).  Returns the section (a dict)."""
     import torch
 
     from luminal_amd import capi, synth
@@ -351,8 +448,8 @@ def bench_moe(args):
         per[f"T={T}"] = {"us": round(us, 1), "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
                          "tflops": round(fl / us / 1e6, 1), "frac_mfma_fp4": round(fl / us / 1e6 / MFMA_FP4_PEAK_TFLOPS, 5),
                          "frac_mfma_fp8_two_pass": round(2 * fl / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 5)}
-    t64 = per["T=64"]
-    print(json.dumps({
+    t64, t1024 = per["T=64"], per["T=1024"]
+    out = {
         "metric": "MXFP4 MoE expert layer (H=I=2880, 32 experts, top-4): GB/s and TFLOP/s, 1 GPU",
         "value": round(flops_step / (wall / args.steps) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3), "higher_is_better": True,
@@ -361,9 +458,18 @@ def bench_moe(args):
                  "f32 accumulate on v_mfma_scale_f32_16x16x128_f8f6f4, bf16 out",
         "data": "synthetic", "config": {"workload": "gpt_oss_style_mxfp4_moe_layer", "tokens": [1, 64, 1024]},
         "per_tokens": per,
-        "roofline": {"bound": "hbm", "kernel": "whole layer at T=64 (plan, quantise, 2 grouped GEMMs, combine)",
+        "roofline": {"bound": "hbm", "kernel": "whole layer at T=64 (plan + quantise, 2 grouped GEMMs, combine)",
                      "achieved": t64["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": t64["frac_hbm"],
-                     "traffic": MOE_T64_TRAFFIC}}))
+                     "traffic": TRAFFIC["moe_t64"][0], "traffic_source": TRAFFIC["moe_t64"][1]},
+        "roofline_t1024_mfma": {"bound": "mfma", "kernel": "whole layer at T=1024",
+                                "achieved": t1024["tflops"], "peak": MFMA_FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                "frac": t1024["frac_mfma_fp4"], "frac_of_fp8_two_pass": t1024["frac_mfma_fp8_two_pass"],
+                                "traffic": None}}
+    if cpu_seconds:
+        out["cpu_baseline"] = cpu_baseline_moe(cpu_seconds)
+    del layer, cases
+    torch.cuda.empty_cache()
+    return out
 
 
 def llama_decode(torch):
@@ -379,7 +485,12 @@ def llama_decode(torch):
     eng = LlamaQ8(cfg, w, max_seq=1024)
     prompt = np.random.default_rng(0).integers(0, cfg.vocab, 512)
     eng.prefill(prompt, bf16=True)          # warm-up (allocates buffers)
-    eng.decode(4, use_graph=True)           # captures the decode graph
+    eager = eng.decode(8, use_graph=False).tolist()
+    eng.reset()
+    eng.prefill(prompt, bf16=True)
+    replayed = eng.decode(8, use_graph=True).tolist()   # captures the decode graph
+    if eager != replayed:
+        raise SystemExit(f"bench.py: graph replay picked {replayed}, eager stepping {eager}")
     eng.reset()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -400,7 +511,8 @@ def llama_decode(torch):
             "q8_0_weight_bytes_per_token": weight_bytes,
             "weight_stream_gbs": round(weight_bytes / (t_decode / 256) / 1e9, 1),
             "frac_hbm_peak": round(weight_bytes / (t_decode / 256) / 1e9 / HBM_PEAK_GBS, 4),
-            "first_tokens": [int(t) for t in toks[:4].tolist()]}
+            "first_tokens": [int(t) for t in toks[:8].tolist()],
+            "graph_replay_equals_eager_first_8": toks[:8].tolist() == eager}
 
 
 def synth_bytes(n, k):
@@ -414,9 +526,9 @@ def main():
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     if args.workload == "prefill_gemm":
-        return bench_prefill_gemm(args)
+        return print(json.dumps(bench_prefill_gemm(args, None if args.no_cpu_baseline else args.cpu_seconds)))
     if args.workload == "moe":
-        return bench_moe(args)
+        return print(json.dumps(bench_moe(args, None if args.no_cpu_baseline else args.cpu_seconds)))
     if args.workload == "rows_f32":
         return bench_rows_f32(args)
 
@@ -622,7 +734,8 @@ def main():
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/): within 1 % of algorithmic
-        "traffic": TRAFFIC_PER_LAUNCH if layers == 32 else None,
+        "traffic": TRAFFIC["gemv"][0] if layers == 32 else None,
+        "traffic_source": TRAFFIC["gemv"][1],
         "launches_per_step": dom_launches,
         "bytes_per_launch": round(dom_bytes / dom_launches),
         "avg_launch_us": round(dom_us, 3),
@@ -663,6 +776,12 @@ def main():
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    if not args.no_sections and layers == 32:
+        # configs 2 and 3 of the benchmark plan ride in the same line, each with its own roofline and CPU baseline
+        sec = argparse.Namespace(steps=max(2, args.steps // 4), warmup=1)
+        cpu_s = None if args.no_cpu_baseline else min(args.cpu_seconds, 8.0)
+        out["prefill_gemm"] = bench_prefill_gemm(sec, cpu_s)
+        out["moe"] = bench_moe(sec, cpu_s)
     print(json.dumps(out))
 
 

@@ -185,7 +185,7 @@ lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_d
                                          int64_t k, void *stream);
 /* Same with the output tile chosen by the caller: tile 0 = 256x128 (8 waves),
  * 1 = 128x128, 2 = 128x64, 3 = 64x64 (4 waves each),
- * 5 = the weight-streaming kernel for m <= 128 described above
+ * 5 = the weight-streaming kernel described above, here for any m <= 8192 in passes of 128 rows
  * (LHIP_ERR_UNSUPPORTED for shapes it does not cover),
  * 50 + S = the same with S slices of K (S clamped to K / 512), 120 + S = the 256x128
  * tile over S slices of K with the partial sums in the same scratch array (2 <= S <= 16,

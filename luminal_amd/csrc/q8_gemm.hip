@@ -414,25 +414,23 @@ static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *
     if (m <= 128 && n <= kMaxDim && k <= kMaxDim &&
         q8_gemm_skinny_supports(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), out, y))
         return kTileSkinny;
-    // Largest tile that still gives at least three quarters of the 256 CUs a
-    // workgroup (measured: 224 workgroups of 256x256 beat 448 of 256x128, which
-    // beat 896 of 128x128); a 256-row tile is skipped when it would be half padding.
     auto blocks = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    // Long K and few 256x128 tiles: slices of K until the chip is full, when the partial planes (written and read
-    // once more: 4 * slices / K bytes per flop) stay small next to the product.  Measured for 4096 x 14336: 102 -> 55 us
-    // at 256 rows (8 slices), 115 -> 83 us at 512 (4), 236 -> 142 us at 1024 (2); no gain for K = 4096.
-    if (m > 128 && k >= 8192 && n % 4 == 0 && aligned(y, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4))) {
+    // Few 256x128 tiles: slices of K until the chip is full, when the partial planes (written and read once more:
+    // 4 * slices / K bytes per flop) fit the scratch array.  A workgroup walks K at about 1.2 us per 64-wide tile
+    // whatever M is, so with fewer workgroups than CUs the K loop is the critical path and slicing it pays at every K
+    // (measured, us, whole K -> sliced: 4096 x 4096 at 256 / 512 / 1024 rows 75 -> 30 / 75 -> 38 / 78 -> 58;
+    // 1024 x 4096 at 512 rows 72 -> 23; 4096 x 14336 at 256 / 512 / 1024 rows 237 -> 56 / 240 -> 89 / 249 -> 163).
+    if (m > 128 && n % 4 == 0 && aligned(y, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4))) {
         const int64_t b0 = blocks(256, 128), kt = k / kBK;
         for (int slices = 8; slices >= 2; slices >>= 1)
             if (b0 * slices <= 256 && kt % slices == 0 && (kt / slices) % 4 == 0 &&
                 static_cast<size_t>(slices) * m * n <= (size_t{8} << 20))
                 return kTileSliced + slices;
     }
-    int tile = 3;
-    if (m > 128 && blocks(256, 128) >= 192) tile = 0;
-    else if (blocks(128, 128) >= 192) tile = 1;
-    else if (blocks(128, 64) >= 192) tile = 2;
-    return tile;
+    // Otherwise the 256x128 tile from 64 workgroups on (measured faster than the smaller tiles there even with a
+    // quarter of the CUs busy: its K loop is the shortest per flop), smaller tiles for small products.
+    if (m > 128 && blocks(256, 128) >= 64) return 0;
+    return blocks(128, 64) >= 64 ? 2 : 3;
 }
 
 }  // namespace lhip

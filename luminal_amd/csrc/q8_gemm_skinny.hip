@@ -422,8 +422,8 @@ lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int 
 // K slices for a product: enough workgroups for the 256 CUs, slices of whole 512-k units, partial sums within the
 // scratch array.
 int q8_gemm_skinny_splits(int m, int n, int k) {
-    const int strips = (n + kSkRows - 1) / kSkRows, units = k / kSkUnit;
-    int s = 256 / strips;
+    const int strips = (n + kSkRows - 1) / kSkRows, units = k / kSkUnit, passes = (m + 127) / 128;
+    int s = 256 / (strips * passes);
     if (s < 1) s = 1;
     if (s > units) s = units;
     while (s > 1 && static_cast<size_t>(s) * m * n > kSkScratchFloats) --s;
@@ -431,8 +431,10 @@ int q8_gemm_skinny_splits(int m, int n, int k) {
     return (units + per - 1) / per;
 }
 
+constexpr int kSkMaxRows = 128 * 64;  // passes are the grid's z extent
+
 bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y) {
-    return m >= 1 && m <= 128 && k % kSkUnit == 0 && n % 4 == 0 && aligned(y, out == kSkOutF32 ? 16 : (out == kSkOutBf16 ? 8 : 4));
+    return m >= 1 && m <= kSkMaxRows && k % kSkUnit == 0 && n % 4 == 0 && aligned(y, out == kSkOutF32 ? 16 : (out == kSkOutBf16 ? 8 : 4));
 }
 
 template <typename XT>
@@ -455,15 +457,16 @@ static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const XT *x, 
     return LHIP_OK;
 }
 
-// bf16 activations, at most 128 rows in one pass (one plane per tile leaves room for 128-row tiles)
+// bf16 activations: passes of 16 * MT rows (one plane per tile leaves room for 128-row tiles)
 template <int MT>
 static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m,
                                 int n, int k, int splits, hipStream_t s) {
-    if (splits > 1) return sk_launch_t<MT, kSkOutPartial, __bf16>(qs, ds, x, y, part, m, n, k, splits, 1, s);
+    const int passes = (m + 16 * MT - 1) / (16 * MT);
+    if (splits > 1) return sk_launch_t<MT, kSkOutPartial, __bf16>(qs, ds, x, y, part, m, n, k, splits, passes, s);
     switch (out) {
-        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
-        case kSkOutF32: return sk_launch_t<MT, kSkOutF32, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
-        default: return sk_launch_t<MT, kSkOutSwiglu, __bf16>(qs, ds, x, y, part, m, n, k, 1, 1, s);
+        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+        case kSkOutF32: return sk_launch_t<MT, kSkOutF32, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+        default: return sk_launch_t<MT, kSkOutSwiglu, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
     }
 }
 

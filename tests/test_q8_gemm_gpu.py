@@ -168,6 +168,16 @@ def test_weight_streaming_gemm_vs_oracle(oracle, m, n, k):
         assert np.all(np.abs(y - auto) <= step) and np.mean(y == auto) > 0.98, slices
 
 
+@pytest.mark.parametrize("m,n,k", [(129, 260, 1024), (300, 128, 512), (512, 1024, 4096)])
+def test_weight_streaming_gemm_in_passes(oracle, m, n, k):
+    """More than 128 rows through the weight-streaming kernel (tile id 5): passes of 128 rows in one launch."""
+    qs, d = synth.q8_0_random(n, k, seed=m + n)
+    xf, bits = bf16_activations(oracle, m, k, seed=5)
+    y = run(upload(qs, d), bits, SKINNY_AUTO)
+    elem, norm = bf16_err(y, truth_for(oracle, qs, d, xf))
+    assert elem < TOL and norm < 4e-3, (elem, norm)
+
+
 def test_weight_streaming_gemm_is_the_one_chosen_and_is_repeatable(oracle):
     """For m <= 128 the plain entry point takes the weight-streaming kernel (same bits as asking for it), K slices
     are added in a fixed order (two runs agree bit for bit, and a product that is exact in f32 is the same for
@@ -193,15 +203,16 @@ def test_weight_streaming_gemm_is_the_one_chosen_and_is_repeatable(oracle):
     wi = upload(qi, di)
     for tile in (None, SKINNY_AUTO, SKINNY_SLICES + 1, SKINNY_SLICES + 2, SKINNY_SLICES + 4):
         assert np.array_equal(run(wi, xb, tile), want_bf16), tile
-    # not covered: K not a multiple of 512, N not a multiple of 4, more than 128 rows
+    # not covered: K not a multiple of 512, N not a multiple of 4, more than 64 passes of 128 rows
     xd = torch.zeros((129, 4096), dtype=torch.bfloat16, device=DEV)
     yd = torch.zeros((129, 4096), dtype=torch.bfloat16, device=DEV)
 
     def cfg(mm, nn, kk):
         return lib.lhip_q8_0_matmul_bf16_cfg(w.planar.data_ptr(), xd.data_ptr(), yd.data_ptr(), mm, nn, kk, SKINNY_AUTO, s)
 
-    assert cfg(129, 64, 512) == capi.LHIP_ERR_UNSUPPORTED and cfg(8, 64, 576) == capi.LHIP_ERR_UNSUPPORTED
+    assert cfg(128 * 64 + 1, 64, 512) == capi.LHIP_ERR_UNSUPPORTED and cfg(8, 64, 576) == capi.LHIP_ERR_UNSUPPORTED
     assert cfg(8, 66, 512) == capi.LHIP_ERR_UNSUPPORTED and cfg(8, 64, 512) == capi.LHIP_OK
+    assert cfg(129, 64, 512) == capi.LHIP_OK  # asked for by name it takes more rows, in passes of 128
     torch.cuda.synchronize()
 
 
