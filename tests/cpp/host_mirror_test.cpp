@@ -1,10 +1,13 @@
 // Tests of the C++ host mirror (luminal_amd/host/luminal_hip.hpp), written after the reference's own tests of the
-// quantized path:
+// quantized path and of the matmul it replaces:
 //   test_quantized_matvec / test_quantized_matmul   crates/luminal_metal/src/quantized.rs:888-986
 //                                                   (same, commented out, crates/luminal_cuda/src/quantized.rs:307-451)
+//   the literal matmul case                         crates/luminal_cpu/src/lib.rs:177-192
 //   the compiler pass' two panics                   crates/luminal_cuda/src/quantized.rs:256-267
 //   the "column-major" assert                       crates/luminal_cuda/src/quantized.rs:118-121
-// Usage: host_mirror_test cpu   (graph rewrite and error paths, no device)
+// The graphs are built the way luminal's high-level ops spell them (src/hl_ops/matmul.rs:4-33, src/hl_ops/other.rs:114-123):
+// primitive Mul / SumReduce / LessThan / Add nodes over fake-expanded views, which the pass has to recognise by itself.
+// Usage: host_mirror_test cpu   (primitives, graph rewrite and error paths, no device)
 //        host_mirror_test gpu   (everything)
 #include <cmath>
 #include <cstdio>
@@ -34,249 +37,351 @@ static std::string panic_message(F f) {
     return "";
 }
 
-// f32 -> IEEE binary16 code, round to nearest even (normal range and zero are all these tests need).
-static uint16_t f16_code(float f) {
-    uint32_t x;
-    std::memcpy(&x, &f, 4);
-    const uint32_t sign = (x >> 16) & 0x8000u;
-    int e = static_cast<int>((x >> 23) & 0xff) - 127 + 15;
-    uint32_t m = x & 0x7fffffu;
-    if ((x & 0x7fffffffu) == 0) return static_cast<uint16_t>(sign);
-    if (e <= 0 || e >= 31) throw std::runtime_error("f16_code: out of the range these tests use");
-    uint32_t h = (static_cast<uint32_t>(e) << 10) | (m >> 13);
-    const uint32_t rest = m & 0x1fffu;
-    if (rest > 0x1000u || (rest == 0x1000u && (h & 1u))) ++h;
-    return static_cast<uint16_t>(sign | h);
-}
-static float f16_value(uint16_t c) {
-    const int e = (c >> 10) & 31, m = c & 1023;
-    const float v = e == 0 ? std::ldexp(static_cast<float>(m), -24) : std::ldexp(1.0f + m / 1024.0f, e - 15);
-    return (c & 0x8000) ? -v : v;
-}
-
 // (n, k) quants + per-block scales -> raw GGUF Q8_0 blocks {f16 d; i8 qs[32]}.
 static std::vector<uint8_t> q8_0_blocks(const std::vector<int8_t> &q, const std::vector<float> &d) {
     std::vector<uint8_t> raw(q.size() / 32 * 34);
     for (size_t b = 0; b < q.size() / 32; ++b) {
-        const uint16_t c = f16_code(d[b]);
+        const uint16_t c = f32_to_f16_code(d[b]);
         std::memcpy(&raw[b * 34], &c, 2);
         std::memcpy(&raw[b * 34 + 2], &q[b * 32], 32);
     }
     return raw;
 }
-
-static double max_abs_diff(const std::vector<float> &got, const std::vector<double> &want) {
-    double m = 0;
-    for (size_t i = 0; i < want.size(); ++i) m = std::max(m, std::fabs(got[i] - want[i]));
-    return m;
+static std::vector<uint8_t> f32_bytes(const std::vector<float> &v) {
+    std::vector<uint8_t> b(v.size() * 4);
+    std::memcpy(b.data(), v.data(), b.size());
+    return b;
 }
 
-// ---------------------------------------------------------------- graph rewrite, no device
+static double max_abs_diff(const std::vector<float> &got, const std::vector<float> &want) {
+    double m = got.size() == want.size() ? 0 : 1e30;
+    for (size_t i = 0; i < want.size() && i < got.size(); ++i) m = std::max(m, std::fabs(static_cast<double>(got[i]) - want[i]));
+    return m;
+}
+static double rms(const std::vector<float> &v) {
+    double s = 0;
+    for (float x : v) s += static_cast<double>(x) * x;
+    return std::sqrt(s / std::max<size_t>(v.size(), 1));
+}
+
+static Function *fn(Graph &g, NodeIndex n) { return dynamic_cast<Function *>(g.nodes[n].get()); }
+static int count_nodes(const Graph &g, const std::string &name) {
+    int c = 0;
+    for (auto &n : g.nodes) c += n && n->name() == name;
+    return c;
+}
+
+// ---- graph builders: what luminal's high-level ops put on the graph ------------------------------------------
+// x (.., m, k) . w^T with w stored (n, k): x.matmul(w.permute((1, 0))) as src/hl_ops/matmul.rs:4-33 expands it.
+static NodeIndex build_matmul(Graph &g, NodeIndex x, std::vector<int64_t> x_dims, NodeIndex w, int64_t n) {
+    const size_t r = x_dims.size();
+    const int64_t k = x_dims.back();
+    ShapeTracker xs = ShapeTracker(x_dims).expand_dim(r - 1, n);  // [.., m, n(fake), k]
+    ShapeTracker ws({n, k});
+    for (size_t i = 0; i + 1 < r; ++i) ws = ws.expand_dim(0, x_dims[r - 2 - i]);  // [..(fake), m(fake), n, k]
+    const NodeIndex mul = g.add(std::make_unique<Binary>(Binary::Mul));
+    g.connect(x, mul, 0, xs);
+    g.connect(w, mul, 1, ws);
+    const NodeIndex red = g.add(std::make_unique<SumReduce>(r));
+    std::vector<int64_t> prod = xs.dims;
+    g.connect(mul, red, 0, ShapeTracker(prod));
+    return red;
+}
+// table.gather(idx) as src/hl_ops/other.rs:114-123: one_hot = arange(V).expand(0, B).eq(idx.expand(1, V)) with
+// eq = -(a < b + b < a) + 1 (src/hl_ops/binary.rs:232-261); (one_hot.expand(2, D) * table.expand(0, B)).sum(1).
+static NodeIndex build_gather(Graph &g, NodeIndex idx, int64_t batch, NodeIndex table, int64_t vocab, int64_t dim) {
+    const NodeIndex ar = g.add(std::make_unique<ARange>(vocab));
+    const ShapeTracker ar_s = ShapeTracker({vocab}).expand_dim(0, batch), idx_s = ShapeTracker({batch}).expand_dim(1, vocab);
+    const ShapeTracker bv({batch, vocab}), scalar = ShapeTracker().expand_dim(0, batch).expand_dim(1, vocab);
+    auto binary = [&](Binary::Kind kind, NodeIndex a, ShapeTracker as, NodeIndex b, ShapeTracker bs) {
+        const NodeIndex n = g.add(std::make_unique<Binary>(kind));
+        g.connect(a, n, 0, as);
+        g.connect(b, n, 1, bs);
+        return n;
+    };
+    const NodeIndex lt = binary(Binary::LessThan, ar, ar_s, idx, idx_s), gt = binary(Binary::LessThan, idx, idx_s, ar, ar_s);
+    const NodeIndex ne = binary(Binary::Add, lt, bv, gt, bv);
+    const NodeIndex neg = binary(Binary::Mul, ne, bv, g.add(std::make_unique<Constant>(-1.f)), scalar);
+    const NodeIndex eq = binary(Binary::Add, neg, bv, g.add(std::make_unique<Constant>(1.f)), scalar);
+    const NodeIndex mul = binary(Binary::Mul, eq, bv.expand_dim(2, dim), table, ShapeTracker({vocab, dim}).expand_dim(0, batch));
+    const NodeIndex red = g.add(std::make_unique<SumReduce>(1));
+    g.connect(mul, red, 0, ShapeTracker({batch, vocab, dim}));
+    return red;
+}
+static NodeIndex build_relu(Graph &g, NodeIndex src, std::vector<int64_t> dims) {
+    const NodeIndex n = g.add(std::make_unique<Unary>("Relu", [](float v) { return v > 0 ? v : 0.f; }));
+    g.connect(src, n, 0, ShapeTracker(std::move(dims)));
+    return n;
+}
+
+// ---------------------------------------------------------------- primitives and graph rewrite, no device
+static void test_primitives_on_the_host() {
+    // crates/luminal_cpu/src/lib.rs:177-192: [[1,2,3],[1,2,3]] . [[1,2,3,1],[2,3,1,2],[3,1,2,3]] = [[14,11,11,14]] x 2;
+    // here the right operand is stored transposed, (n, k) = (4, 3), like a Linear's weight.
+    Graph g;
+    auto x = g.add(std::make_unique<Function>()), w = g.add(std::make_unique<Function>());
+    auto y = build_matmul(g, x, {2, 3}, w, 4);
+    g.to_retrieve.insert(y);
+    fn(g, x)->value = host_tensor({1, 2, 3, 1, 2, 3});
+    fn(g, w)->value = host_tensor({1, 2, 3, 2, 3, 1, 3, 1, 2, 1, 2, 3});
+    g.execute();
+    EXPECT((host_operand(g.results.at(y), "y") == std::vector<float>{14, 11, 11, 14, 14, 11, 11, 14}));
+    // gather on the host: rows 2, 0, 2 of a 3 x 2 table
+    Graph h;
+    auto idx = h.add(std::make_unique<Function>()), table = h.add(std::make_unique<Function>());
+    auto rows = build_gather(h, idx, 3, table, 3, 2);
+    fn(h, idx)->value = host_tensor({2, 0, 2});
+    fn(h, table)->value = host_tensor({10, 11, 20, 21, 30, 31});
+    h.execute();
+    EXPECT((host_operand(h.results.at(rows), "rows") == std::vector<float>{30, 31, 10, 11, 30, 31}));
+    // f16 codes: round to nearest even, subnormals, overflow
+    EXPECT(f32_to_f16_code(1.0f) == 0x3c00 && f32_to_f16_code(-2.0f) == 0xc000 && f32_to_f16_code(65504.f) == 0x7bff);
+    EXPECT(f32_to_f16_code(1.0f + 1.0f / 2048) == 0x3c00 && f32_to_f16_code(1.0f + 3.0f / 2048) == 0x3c02);  // ties to even
+    EXPECT(f32_to_f16_code(65520.f) == 0x7c00 && f32_to_f16_code(std::ldexp(1.0f, -24)) == 0x0001 &&
+           f32_to_f16_code(std::ldexp(1.0f, -25)) == 0x0000 && f32_to_f16_code(std::ldexp(3.0f, -25)) == 0x0002);
+    for (uint32_t c = 0; c < 0x7c00; c += 7) EXPECT(f32_to_f16_code(f16_code_to_f32(static_cast<uint16_t>(c))) == c);
+}
+
 static void test_compiler_pass_cpu() {
-    // tokens -> Gather(embed) -> ... ; x -> MatMul2D(w) ; a weight behind a unary copy ; the pass rewrites all three
+    // tokens -> gather(embed) -> matmul(w) -> relu (host) -> matmul(w2 behind a contiguous copy) -> retrieved
     Graph g;
     auto tok = g.add(std::make_unique<Function>());
     auto embed = g.add(std::make_unique<Function>());
     auto w = g.add(std::make_unique<Function>());
     auto w2 = g.add(std::make_unique<Function>());
     auto w2_copy = g.add(std::make_unique<Unary>("Contiguous"));
-    auto gather = g.add(std::make_unique<Gather>(64));
-    auto mm = g.add(std::make_unique<MatMul2D>());
-    auto mm2 = g.add(std::make_unique<MatMul2D>());
-    g.connect(tok, gather, 0, {{3}, true});
-    g.connect(embed, gather, 1, {{100, 64}, true});
-    g.connect(gather, mm, 0, {{3, 64}, true});
-    g.connect(w, mm, 1, {{64, 32}, false});
-    g.connect(w2, w2_copy, 0, {{32, 32}, true});
-    g.connect(mm, mm2, 0, {{3, 32}, true});
-    g.connect(w2_copy, mm2, 1, {{32, 32}, false});
+    g.connect(w2, w2_copy, 0, ShapeTracker({32, 32}));
+    auto rows = build_gather(g, tok, 3, embed, 100, 64);
+    auto h1 = build_matmul(g, rows, {3, 64}, w, 32);
+    auto act = build_relu(g, h1, {3, 32});
+    auto h2 = build_matmul(g, act, {3, 32}, w2_copy, 32);
+    g.to_retrieve.insert(h2);
+    const size_t before = g.nodes.size();
     EXPECT((downstream({embed, w, w2}, g) == std::vector<NodeIndex>{embed, w, w2_copy}));
     HipQuantizedCompiler({embed, w, w2}).compile(g, /*init_device=*/false);
-    EXPECT(g.nodes[gather]->name() == "QuantizedGather");
-    EXPECT(dynamic_cast<QuantizedGather *>(g.nodes[gather].get())->embed_dim == 64);
-    EXPECT(g.nodes[mm]->name() == "QuantizedMatmul" && g.nodes[mm2]->name() == "QuantizedMatmul");
-    EXPECT(g.nodes[w2_copy]->name() == "Contiguous");  // nodes on the way to the consumer are left alone
+    EXPECT(count_nodes(g, "QuantizedGather") == 1 && count_nodes(g, "QuantizedMatmul") == 2);
+    EXPECT(count_nodes(g, "Mul") == 0 && count_nodes(g, "SumReduce(1)") == 0 && count_nodes(g, "SumReduce(2)") == 0);
+    EXPECT(count_nodes(g, "LessThan") == 0 && count_nodes(g, "ARange") == 0 && count_nodes(g, "Add") == 0);  // the one-hot went
+    EXPECT(count_nodes(g, "Contiguous") == 1 && count_nodes(g, "Relu") == 1);  // nodes around the pattern are left alone
+    // gather -> matmul stays on the device; matmul -> relu -> matmul crosses to the host and back; the retrieved
+    // result is read from a copy
+    EXPECT(count_nodes(g, "HipCopyToDevice") == 1 && count_nodes(g, "HipCopyFromDevice") == 2);
+    EXPECT(g.to_retrieve.size() == 1 && g.nodes[*g.to_retrieve.begin()]->name() == "HipCopyFromDevice");
+    NodeIndex qg = -1, q1 = -1;
+    for (NodeIndex n = static_cast<NodeIndex>(before); n < static_cast<NodeIndex>(g.nodes.size()); ++n) {
+        if (g.nodes[n] && g.nodes[n]->name() == "QuantizedGather") qg = n;
+        if (g.nodes[n] && g.nodes[n]->name() == "QuantizedMatmul" && q1 < 0) q1 = n;
+    }
+    EXPECT(dynamic_cast<QuantizedGather *>(g.nodes[qg].get())->embed_dim == 64);
+    auto gi = g.incoming(qg);
+    EXPECT(gi.size() == 2 && gi[0]->src == tok && gi[0]->shape.dims == std::vector<int64_t>{3} && gi[1]->src == embed &&
+           (gi[1]->shape.dims == std::vector<int64_t>{100, 64}) && gi[1]->shape.is_contiguous());
+    auto mi = g.incoming(q1);
+    EXPECT(mi.size() == 2 && mi[0]->src == qg && (mi[0]->shape.dims == std::vector<int64_t>{3, 64}) && mi[1]->src == w &&
+           (mi[1]->shape.dims == std::vector<int64_t>{64, 32}) && !mi[1]->shape.is_contiguous());
+
+    // a batched matmul, (1, s, k) x (n, k): rank-4 product, SumReduce(3)
+    Graph b;
+    auto bx = b.add(std::make_unique<Function>()), bw = b.add(std::make_unique<Function>());
+    auto by = build_matmul(b, bx, {1, 5, 64}, bw, 96);
+    b.to_retrieve.insert(by);
+    HipQuantizedCompiler({bw}).compile(b, false);
+    EXPECT(count_nodes(b, "QuantizedMatmul") == 1 && count_nodes(b, "Mul") == 0 && count_nodes(b, "SumReduce(3)") == 0);
+    for (NodeIndex n = 0; n < static_cast<NodeIndex>(b.nodes.size()); ++n)
+        if (b.nodes[n] && b.nodes[n]->name() == "QuantizedMatmul") {
+            auto in = b.incoming(n);
+            EXPECT((in[0]->shape.dims == std::vector<int64_t>{1, 5, 64}) && (in[1]->shape.dims == std::vector<int64_t>{64, 96}) &&
+                   !in[1]->shape.is_contiguous());
+        }
 
     // weight as input 0: "Quantized weight .. is the wrong input!"
     Graph bad;
-    auto bw = bad.add(std::make_unique<Function>());
-    auto bx = bad.add(std::make_unique<Function>());
-    auto bmm = bad.add(std::make_unique<MatMul2D>());
-    bad.connect(bw, bmm, 0, {{8, 32}, false});
-    bad.connect(bx, bmm, 1, {{1, 32}, true});
-    EXPECT(panic_message([&] { HipQuantizedCompiler({bw}).compile(bad, false); }).find("is the wrong input!") != std::string::npos);
+    auto badw = bad.add(std::make_unique<Function>()), badx = bad.add(std::make_unique<Function>());
+    auto bmul = bad.add(std::make_unique<Binary>(Binary::Mul));
+    bad.connect(badw, bmul, 0, ShapeTracker({8, 32}).expand_dim(0, 1));
+    bad.connect(badx, bmul, 1, ShapeTracker({1, 32}).expand_dim(1, 8));
+    EXPECT(panic_message([&] { HipQuantizedCompiler({badw}).compile(bad, false); }).find("is the wrong input!") != std::string::npos);
 
-    // weight into something that is neither matmul nor gather
+    // weight into something that is neither matmul nor gather: another operator, or a Mul of another shape
     Graph odd;
-    auto ow = odd.add(std::make_unique<Function>());
-    auto ox = odd.add(std::make_unique<Function>());
-    auto oadd = odd.add(std::make_unique<Unary>("Add"));
-    odd.connect(ox, oadd, 0, {{32}, true});
-    odd.connect(ow, oadd, 1, {{32}, true});
-    const std::string msg = panic_message([&] { HipQuantizedCompiler({ow}).compile(odd, false); });
-    EXPECT(msg.find("isn't a matmul or gather (Add)") != std::string::npos);
+    auto ow = odd.add(std::make_unique<Function>()), ox = odd.add(std::make_unique<Function>());
+    auto oadd = odd.add(std::make_unique<Binary>(Binary::Add));
+    odd.connect(ox, oadd, 0, ShapeTracker({32}));
+    odd.connect(ow, oadd, 1, ShapeTracker({32}));
+    EXPECT(panic_message([&] { HipQuantizedCompiler({ow}).compile(odd, false); }).find("isn't a matmul or gather (Add)") !=
+           std::string::npos);
+    Graph odd2;
+    auto pw = odd2.add(std::make_unique<Function>()), px = odd2.add(std::make_unique<Function>());
+    auto pmul = odd2.add(std::make_unique<Binary>(Binary::Mul));  // element-wise product, no reduction behind it
+    odd2.connect(px, pmul, 0, ShapeTracker({4, 32}));
+    odd2.connect(pw, pmul, 1, ShapeTracker({4, 32}));
+    EXPECT(panic_message([&] { HipQuantizedCompiler({pw}).compile(odd2, false); }).find("isn't a matmul or gather (Mul)") !=
+           std::string::npos);
 
-    // operator-level asserts that need no device: contiguous weight view, mismatched K
+    // operator-level asserts that need no device: contiguous weight view, mismatched K, wrong byte count, host operand
     QuantizedMatmul op;
     Tensor dummy;
-    EXPECT(panic_message([&] { op.process({{&dummy, {{1, 32}, true}}, {&dummy, {{32, 8}, true}}}); }) ==
+    EXPECT(panic_message([&] { op.process({{&dummy, ShapeTracker({1, 32})}, {&dummy, ShapeTracker({32, 8})}}); }) ==
            "Weight matrix must be column-major");
-    EXPECT(panic_message([&] { op.process({{&dummy, {{1, 64}, true}}, {&dummy, {{32, 8}, false}}}); }).find("inner dimensions") !=
-           std::string::npos);
+    EXPECT(panic_message([&] {
+               op.process({{&dummy, ShapeTracker({1, 64})}, {&dummy, ShapeTracker({8, 32}).permute({1, 0})}});
+           }).find("inner dimensions") != std::string::npos);
+    Tensor host = host_tensor({1.f});
+    EXPECT(panic_message([&] {
+               op.process({{&host, ShapeTracker({1, 32})}, {&dummy, ShapeTracker({8, 32}).permute({1, 0})}});
+           }).find("activation is not a HIP buffer") != std::string::npos);
     EXPECT(panic_message([&] { HipData::q8_0_from_raw(std::vector<uint8_t>(33), 1, 32); }).find("n + n/16") != std::string::npos);
 }
 
 // ---------------------------------------------------------------- device
+struct Q8 {
+    std::vector<int8_t> q;
+    std::vector<float> d, dense;  // dense = the weights as luminal_cpu holds them after its load-time dequantisation
+    std::vector<uint8_t> raw;
+};
+static Q8 random_q8(std::mt19937 &rng, int rows, int cols, float floor_scale) {
+    Q8 w;
+    std::normal_distribution<float> gauss(0.f, 0.02f);
+    w.q.resize(static_cast<size_t>(rows) * cols);
+    w.d.resize(w.q.size() / 32);
+    for (auto &v : w.q) v = static_cast<int8_t>(static_cast<int>(rng() % 255) - 127);
+    for (auto &v : w.d) v = f16_code_to_f32(f32_to_f16_code(std::fabs(gauss(rng)) / 127.f + floor_scale));
+    w.raw = q8_0_blocks(w.q, w.d);
+    w.dense.resize(w.q.size());
+    for (size_t i = 0; i < w.q.size(); ++i) w.dense[i] = static_cast<float>(w.q[i]) * w.d[i / 32];
+    return w;
+}
+
 static void test_quantized_matvec_like_the_reference() {
-    // W 512 x 1024 of small non-negative ints with d = 1, x random: the reference compares with the f32 graph at 1e-3.
+    // W 512 x 1024 of small non-negative ints with d = 1, x random: the reference compares the quantized graph with
+    // the f32 graph at 1e-3 (crates/luminal_metal/src/quantized.rs:888-935).  Both graphs are built here: the f32 one
+    // runs on the host primitives, the other goes through the loader and the pass.
     std::mt19937 rng(1);
     const int n = 512, k = 1024;
-    std::vector<int8_t> q(static_cast<size_t>(n) * k);
-    for (auto &v : q) v = static_cast<int8_t>(rng() % 5);
-    std::vector<float> d(q.size() / 32, 1.0f), x(k);
+    Q8 w;
+    w.q.resize(static_cast<size_t>(n) * k);
+    for (auto &v : w.q) v = static_cast<int8_t>(rng() % 5);
+    w.d.assign(w.q.size() / 32, 1.0f);
+    w.raw = q8_0_blocks(w.q, w.d);
+    std::vector<float> dense(w.q.begin(), w.q.end()), x(k);
     std::uniform_real_distribution<float> u(-0.5f, 0.5f);
     for (auto &v : x) v = u(rng);
-    Tensor w{HipData::q8_0_from_raw(q8_0_blocks(q, d), n, k)};
-    Tensor xt{std::make_shared<std::vector<float>>(x)};
-    QuantizedMatmul op;
-    auto out = op.process({{&xt, {{k}, true}}, {&w, {{k, n}, false}}});
-    std::vector<double> want(n, 0.0);
-    for (int r = 0; r < n; ++r)
-        for (int c = 0; c < k; ++c) want[r] += static_cast<double>(q[static_cast<size_t>(r) * k + c]) * x[c];
-    EXPECT(max_abs_diff(device_operand(out[0], "out").to_host_f32(), want) < 1e-3);
+    auto build = [&](Graph &g, NodeIndex &xi, NodeIndex &wi) {
+        xi = g.add(std::make_unique<Function>());
+        wi = g.add(std::make_unique<Function>());
+        const NodeIndex y = build_matmul(g, xi, {1, k}, wi, n);
+        g.to_retrieve.insert(y);
+        fn(g, xi)->value = host_tensor(x);
+    };
+    Graph f32g, q8g;
+    NodeIndex xi, wi;
+    build(f32g, xi, wi);
+    fn(f32g, wi)->value = host_tensor(dense);
+    f32g.execute();
+    const std::vector<float> want = host_operand(f32g.results.at(*f32g.to_retrieve.begin()), "y");
+    build(q8g, xi, wi);
+    auto q_weights = q8_load_hip(q8g, {{wi, GgufTensor{true, n, k, &w.raw}}});
+    HipQuantizedCompiler(q_weights).compile(q8g);
+    q8g.execute();
+    EXPECT(max_abs_diff(host_operand(q8g.results.at(*q8g.to_retrieve.begin()), "y"), want) < 1e-3);
 }
 
-static void test_quantized_matmul_and_graph_execution() {
-    // tokens -> QuantizedGather(embed 100 x 64) -> QuantizedMatmul(w 96 x 64), real scales and negative quants,
-    // through compile() + execute(); M = 16 rows like the reference's matmul test.
+static void test_graph_end_to_end(DType dtype) {
+    // tokens -> gather(Q8_0 table 100 x 64) -> matmul(Q8_0 96 x 64) -> relu on the HOST -> matmul(Q8_0 40 x 96), 16 rows
+    // like the reference's matmul test, real scales and negative quants; and a second consumer of the first matmul
+    // that stays on the host.  The same graph with dequantised f32 weights runs on the host primitives as the check.
     std::mt19937 rng(2);
-    const int vocab = 100, dim = 64, n = 96, m = 16;
-    std::normal_distribution<float> gauss(0.f, 0.02f);
-    auto make = [&](int rows, int cols, std::vector<int8_t> &q, std::vector<float> &d) {
-        q.resize(static_cast<size_t>(rows) * cols);
-        d.resize(q.size() / 32);
-        for (auto &v : q) v = static_cast<int8_t>(static_cast<int>(rng() % 255) - 127);
-        for (auto &v : d) v = f16_value(f16_code(std::fabs(gauss(rng)) / 127.f + 1e-4f));
-        return q8_0_blocks(q, d);
-    };
-    std::vector<int8_t> eq, wq;
-    std::vector<float> ed, wd;
-    auto e_raw = make(vocab, dim, eq, ed), w_raw = make(n, dim, wq, wd);
+    const int vocab = 100, dim = 64, n1 = 96, n2 = 40, m = 16;
+    const Q8 table = random_q8(rng, vocab, dim, 1e-3f), w1 = random_q8(rng, n1, dim, 1e-3f), w2 = random_q8(rng, n2, n1, 1e-3f);
     std::vector<float> ids(m);
     for (auto &v : ids) v = static_cast<float>(rng() % vocab);
-
-    Graph g;
-    auto tok = g.add(std::make_unique<Function>());
-    auto embed = g.add(std::make_unique<Function>());
-    auto w = g.add(std::make_unique<Function>());
-    auto gather = g.add(std::make_unique<Gather>(dim));
-    auto mm = g.add(std::make_unique<MatMul2D>());
-    g.connect(tok, gather, 0, {{m}, true});
-    g.connect(embed, gather, 1, {{vocab, dim}, true});
-    g.connect(gather, mm, 0, {{m, dim}, true});
-    g.connect(w, mm, 1, {{dim, n}, false});
-    HipQuantizedCompiler({embed, w}).compile(g);
-    dynamic_cast<Function *>(g.nodes[tok].get())->value = Tensor{std::make_shared<std::vector<float>>(ids)};
-    dynamic_cast<Function *>(g.nodes[embed].get())->value = Tensor{HipData::q8_0_from_raw(e_raw, vocab, dim)};
-    dynamic_cast<Function *>(g.nodes[w].get())->value = Tensor{HipData::q8_0_from_raw(w_raw, n, dim)};
-    g.execute();
-
-    auto deq = [](const std::vector<int8_t> &q, const std::vector<float> &d, size_t i) {
-        return static_cast<double>(q[i]) * static_cast<double>(d[i / 32]);
+    NodeIndex tok, ti, w1i, w2i, y2, side;
+    auto build = [&](Graph &g) {
+        tok = g.add(std::make_unique<Function>());
+        ti = g.add(std::make_unique<Function>());
+        w1i = g.add(std::make_unique<Function>());
+        w2i = g.add(std::make_unique<Function>());
+        const NodeIndex rows = build_gather(g, tok, m, ti, vocab, dim);
+        const NodeIndex y1 = build_matmul(g, rows, {m, dim}, w1i, n1);
+        const NodeIndex act = build_relu(g, y1, {m, n1});
+        y2 = build_matmul(g, act, {m, n1}, w2i, n2);
+        side = g.add(std::make_unique<Unary>("Double", [](float v) { return 2 * v; }));
+        g.connect(y1, side, 0, ShapeTracker({m, n1}));
+        g.to_retrieve.insert(y2);
+        g.to_retrieve.insert(side);
+        fn(g, tok)->value = host_tensor(ids);
     };
-    // gather is exact
-    auto rows = device_operand(g.results.at(gather), "gather").to_host_f32();
-    bool exact = true;
-    for (int t = 0; t < m; ++t)
-        for (int c = 0; c < dim; ++c)
-            exact &= rows[static_cast<size_t>(t) * dim + c] ==
-                     static_cast<float>(deq(eq, ed, static_cast<size_t>(ids[t]) * dim + c));
-    EXPECT(exact);
-    std::vector<double> want(static_cast<size_t>(m) * n, 0.0);
-    double rms = 0;
-    for (int t = 0; t < m; ++t)
-        for (int r = 0; r < n; ++r) {
-            double s = 0;
-            for (int c = 0; c < dim; ++c)
-                s += deq(eq, ed, static_cast<size_t>(ids[t]) * dim + c) * deq(wq, wd, static_cast<size_t>(r) * dim + c);
-            want[static_cast<size_t>(t) * n + r] = s;
-            rms += s * s;
-        }
-    rms = std::sqrt(rms / want.size());
-    EXPECT(max_abs_diff(device_operand(g.results.at(mm), "matmul").to_host_f32(), want) < 2e-3 * rms);
+    Graph host;
+    build(host);
+    fn(host, ti)->value = host_tensor(table.dense);
+    fn(host, w1i)->value = host_tensor(w1.dense);
+    fn(host, w2i)->value = host_tensor(w2.dense);
+    host.execute();
+    const std::vector<float> want2 = host_operand(host.results.at(y2), "y2"), want_side = host_operand(host.results.at(side), "side");
 
-    // device-side failure surfaces as a Panic carrying the status name (K not a multiple of 32)
-    Tensor xt{std::make_shared<std::vector<float>>(std::vector<float>(40, 1.f))};
-    QuantizedMatmul op;
-    const std::string msg = panic_message([&] { op.process({{&xt, {{40}, true}}, {&g.results.at(w), {{40, 8}, false}}}); });
-    EXPECT(msg.find("lhip_q8_0_matmul_f32") != std::string::npos && msg.find("INVALID_SHAPE") != std::string::npos);
+    Graph dev;
+    build(dev);
+    const NodeIndex side_dev = side;
+    auto q_weights = q8_load_hip(dev, {{ti, GgufTensor{true, vocab, dim, &table.raw}},
+                                       {w1i, GgufTensor{true, n1, dim, &w1.raw}},
+                                       {w2i, GgufTensor{true, n2, n1, &w2.raw}}});
+    EXPECT(q_weights.size() == 3);
+    HipQuantizedCompiler(q_weights, dtype).compile(dev);
+    dev.execute();
+    std::vector<float> got2;
+    for (NodeIndex r : dev.to_retrieve)
+        if (r != side_dev) got2 = host_operand(dev.results.at(r), "retrieved y2");
+    const std::vector<float> got_side = host_operand(dev.results.at(side_dev), "side");
+    // f32: the operators' 2e-3 bar; f16: one rounding of every intermediate (2^-11 relative each)
+    const double tol = dtype == DType::F32 ? 2e-3 : 1e-2;
+    EXPECT(max_abs_diff(got2, want2) < tol * rms(want2));
+    EXPECT(max_abs_diff(got_side, want_side) < tol * rms(want_side));
+    if (dtype == DType::F32) {
+        // the gather itself is exact: read it back from the quantized node
+        for (NodeIndex n = 0; n < static_cast<NodeIndex>(dev.nodes.size()); ++n)
+            if (dev.nodes[n] && dev.nodes[n]->name() == "QuantizedGather") {
+                auto rows = device_operand(dev.results.at(n), "gather").to_host_f32();
+                bool exact = rows.size() == static_cast<size_t>(m) * dim;
+                for (int t = 0; exact && t < m; ++t)
+                    for (int c = 0; c < dim; ++c)
+                        exact &= rows[static_cast<size_t>(t) * dim + c] == table.dense[static_cast<size_t>(ids[t]) * dim + c];
+                EXPECT(exact);
+            }
+    }
 }
 
-static void test_f16_graph() {
-    // The same two-node graph compiled for T = f16 (the type the reference's llama example runs in):
-    // gather -> f16 rows (exact rows rounded once), matmul -> f32 sums rounded once to f16.
-    std::mt19937 rng(3);
-    const int vocab = 50, dim = 64, n = 40, m = 5;
-    std::normal_distribution<float> gauss(0.f, 0.02f);
-    auto make = [&](int rows, int cols, std::vector<int8_t> &q, std::vector<float> &d) {
-        q.resize(static_cast<size_t>(rows) * cols);
-        d.resize(q.size() / 32);
-        for (auto &v : q) v = static_cast<int8_t>(static_cast<int>(rng() % 255) - 127);
-        for (auto &v : d) v = f16_value(f16_code(std::fabs(gauss(rng)) / 127.f + 1e-3f));
-        return q8_0_blocks(q, d);
-    };
-    std::vector<int8_t> eq, wq;
-    std::vector<float> ed, wd;
-    auto e_raw = make(vocab, dim, eq, ed), w_raw = make(n, dim, wq, wd);
-    std::vector<float> ids(m);
-    for (auto &v : ids) v = static_cast<float>(rng() % vocab);
+static void test_device_errors_surface_as_panics() {
+    // K = 40 is not a multiple of 32: the status of the C ABI becomes a Panic carrying its name
+    std::mt19937 rng(4);
+    const Q8 w = random_q8(rng, 8, 64, 1e-3f);
+    Tensor wt{HipData::q8_0_from_raw(w.raw, 8, 64)};
+    Tensor xt{HipData::from_host(std::vector<float>(40, 1.f))};
+    QuantizedMatmul op;
+    const std::string msg =
+        panic_message([&] { op.process({{&xt, ShapeTracker({1, 40})}, {&wt, ShapeTracker({8, 40}).permute({1, 0})}}); });
+    EXPECT(msg.find("lhip_q8_0_matmul_f32") != std::string::npos && msg.find("INVALID_SHAPE") != std::string::npos);
+    // a host operator fed a device buffer fails the way the reference's downcast_ref::<Vec<f32>>().unwrap() does
+    Unary relu("Relu", [](float v) { return v; });
+    EXPECT(panic_message([&] { relu.process({{&xt, ShapeTracker({40})}}); }).find("not a host f32 vector") != std::string::npos);
+    // F32 tensors of a file go to the host through the same loader
     Graph g;
-    auto tok = g.add(std::make_unique<Function>());
-    auto embed = g.add(std::make_unique<Function>());
-    auto w = g.add(std::make_unique<Function>());
-    auto gather = g.add(std::make_unique<Gather>(dim));
-    auto mm = g.add(std::make_unique<MatMul2D>());
-    g.connect(tok, gather, 0, {{m}, true});
-    g.connect(embed, gather, 1, {{vocab, dim}, true});
-    g.connect(gather, mm, 0, {{m, dim}, true});
-    g.connect(w, mm, 1, {{dim, n}, false});
-    HipQuantizedCompiler({embed, w}, DType::F16).compile(g);
-    EXPECT(dynamic_cast<QuantizedMatmul *>(g.nodes[mm].get())->dtype == DType::F16);
-    dynamic_cast<Function *>(g.nodes[tok].get())->value = Tensor{std::make_shared<std::vector<float>>(ids)};
-    dynamic_cast<Function *>(g.nodes[embed].get())->value = Tensor{HipData::q8_0_from_raw(e_raw, vocab, dim)};
-    dynamic_cast<Function *>(g.nodes[w].get())->value = Tensor{HipData::q8_0_from_raw(w_raw, n, dim)};
-    g.execute();
-    auto rows = device_operand(g.results.at(gather), "gather").to_host_f16_codes();
-    bool exact = rows.size() == static_cast<size_t>(m) * dim;
-    for (int t = 0; exact && t < m; ++t)
-        for (int c = 0; c < dim; ++c) {
-            const size_t i = static_cast<size_t>(ids[t]) * dim + c;
-            exact &= rows[static_cast<size_t>(t) * dim + c] == f16_code(static_cast<float>(eq[i]) * ed[i / 32]);
-        }
-    EXPECT(exact);
-    auto out = device_operand(g.results.at(mm), "matmul").to_host_f16_codes();
-    double worst = 0, rms = 0;
-    for (int t = 0; t < m; ++t)
-        for (int r = 0; r < n; ++r) {
-            double s = 0;
-            for (int c = 0; c < dim; ++c)
-                s += static_cast<double>(f16_value(rows[static_cast<size_t>(t) * dim + c])) *
-                     (static_cast<double>(wq[static_cast<size_t>(r) * dim + c]) * wd[(static_cast<size_t>(r) * dim + c) / 32]);
-            worst = std::max(worst, std::fabs(f16_value(out[static_cast<size_t>(t) * n + r]) - s));
-            rms += s * s;
-        }
-    EXPECT(worst < 2e-3 * std::sqrt(rms / (m * n)));
+    auto a = g.add(std::make_unique<Function>());
+    const std::vector<uint8_t> bytes = f32_bytes({1.f, 2.f, 3.f, 4.f});
+    EXPECT(q8_load_hip(g, {{a, GgufTensor{false, 2, 2, &bytes}}}).empty());
+    EXPECT((host_operand(fn(g, a)->value, "a") == std::vector<float>{1, 2, 3, 4}));
 }
 
 int main(int argc, char **argv) {
     const std::string mode = argc > 1 ? argv[1] : "cpu";
     try {
+        test_primitives_on_the_host();
         test_compiler_pass_cpu();
         if (mode == "gpu") {
             check(lhip_init(0), "lhip_init");
             test_quantized_matvec_like_the_reference();
-            test_quantized_matmul_and_graph_execution();
-            test_f16_graph();
+            test_graph_end_to_end(DType::F32);
+            test_graph_end_to_end(DType::F16);
+            test_device_errors_surface_as_panics();
         }
     } catch (const std::exception &e) {
         std::printf("FAIL unexpected exception: %s\n", e.what());
