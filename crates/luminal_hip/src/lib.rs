@@ -1,13 +1,26 @@
 //! luminal_hip: HIP quantized-matmul backend for Luminal on MI355X.
 //!
-//! Usage, in place of `CudaQuantizedCompiler` (examples/llama/src/main.rs:75-97):
+//! Usage, in place of `CudaQuantizedCompiler` (examples/llama/src/main.rs:75-97) and with no dense backend in
+//! front of it:
 //! ```ignore
-//! let q_weights = loader::q8_load_hip("model.gguf", &model, &mut cx);   // uploads + repacks each Q8_0 tensor
-//! cx.compile((GenericCompiler::default(), HipQuantizedCompiler::<f32>::new(q_weights)), (&mut logits, &mut cache));
+//! let q_weights = luminal_hip::q8_load_hip("model.gguf", &model, &mut cx);   // uploads + repacks each Q8_0 tensor
+//! cx.compile(
+//!     (GenericCompiler::default(), HipQuantizedCompiler::<f32>::new(q_weights)),
+//!     (&mut logits, &mut cache),
+//! );
 //! ```
-//! This crate cannot be compiled where the backend was developed (no Rust toolchain); it is the
-//! maintainer-side half of the boundary declared in include/luminal_hip.h.
+//! Behind `GenericCompiler` the graph still holds luminal's primitive operators, which run on host `Vec<f32>`
+//! (src/op.rs).  The pass therefore recognises the matmul and the gather as those primitives spell them
+//! (Mul -> SumReduce over fake-expanded operands, src/hl_ops/matmul.rs:4-33 and src/hl_ops/other.rs:114-123),
+//! replaces them by `QuantizedMatmul` / `QuantizedGather`, and puts `HipCopyToDevice` / `HipCopyFromDevice` nodes
+//! around them so that every other node keeps seeing host vectors.  It names no type of any other backend crate.
+//!
+//! This crate has not met a compiler: there is no Rust toolchain where the backend was developed.  Its logic is
+//! the one of the C++ restatement `luminal_amd/host/luminal_hip.hpp`, which is compiled and tested on the GPU
+//! (tests/cpp/host_mirror_test.cpp); the C ABI it binds is include/luminal_hip.h.
 pub mod ffi;
+mod loader;
 mod quantized;
 
-pub use quantized::{HipData, HipQuantizedCompiler, QuantizedGather, QuantizedMatmul};
+pub use loader::q8_load_hip;
+pub use quantized::{HipCopyFromDevice, HipCopyToDevice, HipData, HipQuantizedCompiler, QuantizedGather, QuantizedMatmul};

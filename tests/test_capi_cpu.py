@@ -96,3 +96,22 @@ def test_gemv_byte_model():
     assert synth.q8_0_gemv_bytes(14336, 4096) == 62464000
     assert synth.q8_0_gemv_bytes(4096, 14336) == 62464000
     assert synth.q8_0_gemv_bytes(128256, 4096) == 558699520
+
+
+def test_rust_bindings_name_exported_symbols_with_the_header_arity():
+    """crates/luminal_hip/src/ffi.rs is not compiled here (no Rust toolchain): at least every function it declares
+    must exist in the library with as many parameters as the header gives it."""
+    text = open(os.path.join(ROOT, "crates", "luminal_hip", "src", "ffi.rs")).read()
+    block = text[text.index('extern "C" {'):]
+    block = block[: block.index("\n}")]
+    rust = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (lhip_[a-z0-9_]+)\(([^)]*)\)", block)}
+    assert len(rust) >= 12
+    header = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    lib = capi.load_library()
+    for name, params in rust.items():
+        assert hasattr(lib, name), name
+        decl = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)
+        assert decl, name
+        c_params = [p for p in decl.group(1).split(",") if p.strip() not in ("", "void")]
+        rust_params = [p for p in params.split(",") if p.strip()]
+        assert len(c_params) == len(rust_params), name

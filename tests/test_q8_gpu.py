@@ -44,6 +44,17 @@ def test_repack_unpack_round_trip_bit_exact(n, k):
     assert np.array_equal(w.to_raw().cpu().numpy(), raw)
 
 
+@pytest.mark.parametrize("n,k", [(3, 96), (129, 1056), (1024, 4096)])
+def test_planar_form_depends_on_the_block_count_only(n, k):
+    # a loader that knows a tensor's element count but not its (n, k), as the reference's loader does
+    # (examples/llama/src/loader.rs:121-130), may repack it as (n_elements / 32, 32)
+    qs, d = synth.q8_0_random(n, k, seed=n + k)
+    raw = synth.q8_0_raw_blocks(qs, d)
+    by_shape = Q8Weight.from_raw(raw, n, k, DEV).planar.cpu().numpy()
+    by_count = Q8Weight.from_raw(raw, n * k // 32, 32, DEV).planar.cpu().numpy()
+    assert np.array_equal(by_shape, by_count)
+
+
 def test_dequant_bit_exact_every_quant_times_every_scale(oracle):
     # all 256 int8 values x all 65536 f16 codes (NaN codes compared as NaN)
     n, k = 65536, 256
