@@ -21,6 +21,10 @@ extern "C" {
     // weights once per 64 rows instead of once per row
     pub fn lhip_q8_0_matmul_f32(w: *const c_void, x: *const f32, y: *mut f32, m: i64, n: i64, k: i64, s: Stream) -> Status;
     pub fn lhip_q8_0_gather_f32(w: *const c_void, idx: *const f32, out: *mut f32, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;
+    // kernel-level route: names the kernel of luminal_hip_kernels.hsaco and the launch shape the matvec above would use, for a
+    // host that drives hipModuleLoad / hipModuleGetFunction / hipModuleLaunchKernel itself (include/luminal_hip_kernels.h)
+    pub fn lhip_q8_0_gemv_kernel_plan(n: i64, k: i64, f16: i32, kernel_name: *mut c_char, kernel_name_cap: usize,
+                                      grid: *mut u32, block: *mut u32, lds_bytes: *mut u32) -> Status;
     // T = f16: x / y / out are IEEE binary16 buffers, sums stay f32
     pub fn lhip_q8_0_matmul_f16(w: *const c_void, x: *const c_void, y: *mut c_void, m: i64, n: i64, k: i64, s: Stream) -> Status;
     pub fn lhip_q8_0_gather_f16(w: *const c_void, idx: *const f32, out: *mut c_void, n_idx: i64, n: i64, k: i64, s: Stream) -> Status;

@@ -124,6 +124,23 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
                                      int64_t k, int rows_per_wave, int k_unroll, int blocks_per_cu,
                                      int waves_per_block, void *stream);
 
+/* Kernel-level route to the same matvec, for a host that launches kernels itself the way
+ * the reference does (module loaded once, function found by name, launched with explicit
+ * grid / block / arguments: crates/luminal_cuda/src/lib.rs:237-258,
+ * crates/luminal_cuda/src/quantized.rs:42-50,131-148).  luminal_hip_kernels.hsaco holds the
+ * matvec kernels under C names (include/luminal_hip_kernels.h states their arguments).
+ * This call names the kernel and launch shape lhip_q8_0_matmul_f32 / _f16 would use for
+ * an (n, k) weight at few activation rows, so that
+ *   hipModuleLoad(&mod, ".../luminal_hip_kernels.hsaco");
+ *   hipModuleGetFunction(&fn, mod, kernel_name);
+ *   grid[1] = m;   // activation rows, 1..65535
+ *   hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+ *                         lds_bytes, stream, args, NULL);
+ * gives the bits of the library call.  It touches no device.  f16 != 0 selects the f16
+ * activation type.  kernel_name receives a NUL-terminated string (64 bytes are enough). */
+lhip_status lhip_q8_0_gemv_kernel_plan(int64_t n, int64_t k, int f16, char *kernel_name, size_t kernel_name_cap,
+                                       uint32_t grid[3], uint32_t block[3], uint32_t *lds_bytes);
+
 /* Batch-1 decode matvec with fusions.  No counterpart in the reference, whose graph runs
  * each piece as its own operator (RMSNorm: examples/llama/src/model.rs:150-160 through
  * luminal_nn, the sibling projections model.rs:95-100 and :24-32, the residual adds

@@ -16,6 +16,9 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libluminal_hip.so")
+# Code object with the matvec kernels under C names, for hosts that launch through hipModule* themselves.
+MODULE_SRC = os.path.join(CSRC, "module", "q8_gemv_module.hip")
+MODULE = os.path.join(HERE, "luminal_hip_kernels.hsaco")
 
 ARCH = "gfx950"
 # Packed-FP32 instructions are switched off for all device code.
@@ -52,7 +55,17 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(f"[luminal_amd.build] {cc} -> {LIB}", file=sys.stderr)
     _run([cc, *COMMON, *DEVICE_FLAGS, "-shared", "-o", LIB, *srcs])
+    build_module(verbose)
     return LIB
+
+
+def build_module(verbose: bool = True) -> str:
+    """Device-only compile of the kernel module into a plain gfx950 ELF code object."""
+    if verbose:
+        print(f"[luminal_amd.build] {hipcc()} -> {MODULE}", file=sys.stderr)
+    _run([hipcc(), "--cuda-device-only", "--no-gpu-bundle-output", "-O3", "-std=c++17", f"--offload-arch={ARCH}",
+          *DEVICE_FLAGS, "-o", MODULE, MODULE_SRC])
+    return MODULE
 
 
 HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "host_mirror_test.cpp")

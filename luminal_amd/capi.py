@@ -35,6 +35,8 @@ SIGNATURES = {
     "lhip_q8_0_dequant_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "lhip_q8_0_gemv_kernel_plan": (C.c_int32, [_i64, _i64, _int, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32),
+                                               C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "lhip_q8_0_matvec_fused_f32": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _vp]),
     "lhip_q8_0_matvec_fused_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _int, _int,
                                                    _int, _int, _vp]),

@@ -115,3 +115,47 @@ def test_rust_bindings_name_exported_symbols_with_the_header_arity():
         c_params = [p for p in decl.group(1).split(",") if p.strip() not in ("", "void")]
         rust_params = [p for p in params.split(",") if p.strip()]
         assert len(c_params) == len(rust_params), name
+
+
+def kernel_names_in_header():
+    text = open(os.path.join(ROOT, "include", "luminal_hip_kernels.h")).read()
+    macro = text[text.index("#define LHIP_KERNEL_Q8_0_GEMV_NAMES"):]
+    macro = macro[: macro.index("\n\n")]
+    return re.findall(r'"(lhip_kernel_[a-z0-9_]+)"', macro)
+
+
+def test_code_object_holds_every_kernel_the_header_names():
+    names = kernel_names_in_header()
+    assert len(names) == 16 and len(set(names)) == 16
+    blob = open(os.path.join(ROOT, "luminal_amd", "luminal_hip_kernels.hsaco"), "rb").read()
+    assert blob[:4] == b"\x7fELF"
+    for n in names:
+        assert n.encode() + b".kd\0" in blob, n  # kernel descriptor symbol
+
+
+def test_kernel_plan_names_a_kernel_of_the_code_object_and_its_launch_shape():
+    import ctypes as C
+    lib = capi.load_library()
+    names = set(kernel_names_in_header())
+
+    def plan(n, k, f16):
+        name = C.create_string_buffer(64)
+        grid, block, lds = (C.c_uint32 * 3)(), (C.c_uint32 * 3)(), C.c_uint32()
+        st = lib.lhip_q8_0_gemv_kernel_plan(n, k, f16, name, 64, grid, block, C.byref(lds))
+        return st, name.value.decode(), list(grid), list(block), lds.value
+
+    assert plan(4096, 4096, 0) == (0, "lhip_kernel_q8_0_gemv_f32_pipe_r1s2w4", [768, 1, 1], [256, 1, 1], 16384)
+    assert plan(128256, 4096, 1) == (0, "lhip_kernel_q8_0_gemv_f16_pipe_r2s4w4", [256, 1, 1], [256, 1, 1], 16384)
+    assert plan(4096, 14336, 0) == (0, "lhip_kernel_q8_0_gemv_f32_pipe_r1s2w16", [256, 1, 1], [1024, 1, 1], 57344)
+    assert plan(37, 96, 0) == (0, "lhip_kernel_q8_0_gemv_f32_oneshot_r1", [10, 1, 1], [256, 1, 1], 0)
+    for n, k in [(1, 32), (100, 1024), (5000, 3072), (8192, 1056), (300, 15360), (40000, 8192), (7, 20480)]:
+        for f16 in (0, 1):
+            st, name, grid, block, lds = plan(n, k, f16)
+            assert st == 0 and name in names
+            assert block[0] % 64 == 0 and block[0] <= 1024 and grid[0] >= 1 and lds <= 65536
+            assert ("pipe" in name) == (lds == 4 * k)
+    assert plan(4096, 48, 0)[0] == capi.LHIP_ERR_INVALID_SHAPE
+    name = C.create_string_buffer(8)
+    grid, block, lds = (C.c_uint32 * 3)(), (C.c_uint32 * 3)(), C.c_uint32()
+    assert lib.lhip_q8_0_gemv_kernel_plan(64, 64, 0, name, 8, grid, block, C.byref(lds)) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_gemv_kernel_plan(64, 64, 0, None, 64, grid, block, C.byref(lds)) == capi.LHIP_ERR_NULL_PTR
