@@ -353,6 +353,53 @@ lhip_status lhip_attention_f32_bf16out(const float *qkv_dev, const float *k_cach
 lhip_status lhip_attention_bf16(const float *qkv_dev, const float *k_cache_dev, const float *v_cache_dev,
                                 void *out_bf16_dev, const int32_t *pos_dev, int64_t tokens, int64_t q_heads,
                                 int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
+/* ---- persistent decode program --------------------------------------------
+ * A batch-1 decode step as ONE launch: a list of operations that a resident grid (one workgroup
+ * per compute unit) walks in order, a grid-wide barrier between consecutive phases, the weight
+ * stream running across the barriers.  No counterpart in the reference, whose graph executor
+ * runs one operator per kernel launch (src/graph.rs execute loop); the operations are those of
+ * examples/llama/src/model.rs:95-139,150-160 in the fused forms of lhip_q8_0_matvec_fused_f32 and
+ * lhip_attention_decode_f32, with the same arithmetic and reduction orders.
+ *
+ * Operations:
+ *   LHIP_DECODE_MATVEC     y = epilogue(W norm(x)): planar (n, k) weight, x (k floats), y (n floats; n / 2 for
+ *                          SwiGLU, whose weight holds gate and up rows interleaved), norm_weight NULL or the k
+ *                          gains of an RMS norm with eps, epilogue one of LHIP_FUSE_*, residual (n floats, may
+ *                          be y) for LHIP_FUSE_ADD.  k % 1024 == 0 and k <= 14336 (LHIP_ERR_UNSUPPORTED beyond).
+ *   LHIP_DECODE_ATTENTION  rotary + cache append + attention for the new token at *pos_dev: x = fused qkv row,
+ *                          y = attention output rows, k_cache / v_cache of the layer.  Head geometry is that of
+ *                          the create call: head_dim 64 or 128, q_heads / kv_heads in {1, 2, 4, 8}.
+ * Every buffer an operation writes must differ from the buffers it reads, except y == residual; an operation
+ * may read what any earlier one wrote.  Pointers are captured at creation; *pos_dev is read at every run.
+ *
+ * lhip_decode_program_run queues two kernels on the stream (a clear of the barrier counters, then the
+ * program) and allocates nothing, so it can be captured into a graph.  Runs of one program must not overlap
+ * in time.  The program kernel needs every compute unit of the device to itself while it runs: all of its
+ * workgroups must be resident together, which holds when nothing else occupies the device (kernels queued
+ * before it on any stream simply finish first).  Every wait inside is bounded (about a second): if the
+ * workgroups fail to meet, the kernel still ends, the step's results are meaningless, and
+ * lhip_decode_program_status (which waits for the device) reports *timed_out = 1 from then on. */
+enum { LHIP_DECODE_MATVEC = 0, LHIP_DECODE_ATTENTION = 1 };
+enum { LHIP_FUSE_NONE = 0, LHIP_FUSE_ADD = 1, LHIP_FUSE_SWIGLU = 2 };
+typedef struct lhip_decode_op {
+    int32_t type;
+    int32_t epilogue;
+    const void *planar;
+    int64_t n, k;
+    const float *x;
+    float *y;
+    const float *norm_weight;
+    float eps;
+    const float *residual;
+    float *k_cache, *v_cache;
+} lhip_decode_op;
+lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int64_t q_heads, int64_t kv_heads,
+                                       int64_t head_dim, int64_t max_seq, float theta, const int32_t *pos_dev,
+                                       void **program);
+lhip_status lhip_decode_program_run(void *program, void *stream);
+lhip_status lhip_decode_program_status(void *program, int32_t *timed_out);
+lhip_status lhip_decode_program_destroy(void *program);
+
 /* Element-wise casts between f32 and bf16 (round to nearest even), for feeding f32
  * activations to the bf16 prefill GEMM. */
 lhip_status lhip_cast_f32_to_bf16(const float *x_dev, void *y_dev, int64_t n, void *stream);

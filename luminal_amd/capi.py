@@ -37,6 +37,10 @@ SIGNATURES = {
     "lhip_q8_0_matmul_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "lhip_q8_0_gemv_kernel_plan": (C.c_int32, [_i64, _i64, _int, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32),
                                                C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "lhip_decode_program_create": (C.c_int32, [_vp, _int, _i64, _i64, _i64, _i64, C.c_float, _vp, C.POINTER(C.c_void_p)]),
+    "lhip_decode_program_run": (C.c_int32, [_vp, _vp]),
+    "lhip_decode_program_status": (C.c_int32, [_vp, C.POINTER(C.c_int32)]),
+    "lhip_decode_program_destroy": (C.c_int32, [_vp]),
     "lhip_q8_0_matvec_fused_f32": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _vp]),
     "lhip_q8_0_matvec_fused_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _int, _int,
                                                    _int, _int, _vp]),
@@ -87,6 +91,16 @@ class LhipError(RuntimeError):
 
 
 _lib = None
+
+
+class DecodeOp(C.Structure):
+    """lhip_decode_op of include/luminal_hip.h."""
+    _fields_ = [("type", C.c_int32), ("epilogue", C.c_int32), ("planar", C.c_void_p), ("n", C.c_int64),
+                ("k", C.c_int64), ("x", C.c_void_p), ("y", C.c_void_p), ("norm_weight", C.c_void_p),
+                ("eps", C.c_float), ("residual", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p)]
+
+
+LHIP_DECODE_MATVEC, LHIP_DECODE_ATTENTION = 0, 1
 
 
 def load_library(path: str | None = None) -> C.CDLL:

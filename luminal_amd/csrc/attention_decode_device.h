@@ -1,0 +1,363 @@
+// Device code of batch-1 decode attention (rotary + cache append + split-KV attention, and the merge of the
+// partial softmax states), shared by the two-launch form (attention_decode.hip) and by the persistent decode
+// program (decode_program.hip), where both run as phases of one kernel.
+//
+// Template switches:
+//   THREADS  threads of the workgroup that calls the body.  The work is laid out for kDecThreads = 256; further
+//            threads only take part in the barriers.
+//   AGENT    true when the inputs were written, and the outputs will be read, by other workgroups of the SAME
+//            launch.  Such data moves through agent-coherent loads and stores (they bypass the caches that are
+//            private to a part of the chip); within one launch plain accesses could meet stale lines.  The KV
+//            caches are exempt: rows of earlier positions come from earlier launches, and the row of the new
+//            position is served from LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lhip {
+
+constexpr int kDecThreads = 256;
+constexpr int kDecTile = 64;
+
+__device__ __forceinline__ float wave_max64(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum64(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// Pointers that reach a kernel through a table in memory (rather than as kernel arguments) are generic to the
+// compiler, which then emits flat accesses and waits for the LDS counter as well.  All of them are device memory.
+#define LHIP_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ const LHIP_GLOBAL T *as_global(const T *p) {
+    return (const LHIP_GLOBAL T *)p;
+}
+template <typename T>
+__device__ __forceinline__ LHIP_GLOBAL T *as_global(T *p) {
+    return (LHIP_GLOBAL T *)p;
+}
+
+typedef float lhip_f32x4 __attribute__((ext_vector_type(4)));
+typedef float lhip_f32x2 __attribute__((ext_vector_type(2)));
+// plain 16-byte accesses to device memory
+__device__ __forceinline__ float4 ldg4(const float4 *p) {
+    const lhip_f32x4 v = *as_global(reinterpret_cast<const lhip_f32x4 *>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stg4(float4 *p, const float4 &v) {
+    lhip_f32x4 t;
+    t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
+    *as_global(reinterpret_cast<lhip_f32x4 *>(p)) = t;
+}
+
+// ---- agent-coherent accessors (relaxed atomics at agent scope: single instructions with the coherence bit set)
+__device__ __forceinline__ float ld_agent(const float *p) {
+    return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(float *p, float v) {
+    __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 ld_agent2(const float *p) {  // p 8-byte aligned
+    const unsigned long long raw =
+        __hip_atomic_load(as_global(reinterpret_cast<const unsigned long long *>(p)), __ATOMIC_RELAXED,
+                          __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__uint_as_float(static_cast<unsigned>(raw)), __uint_as_float(static_cast<unsigned>(raw >> 32)));
+}
+__device__ __forceinline__ void st_agent2(float *p, float a, float b) {  // p 8-byte aligned
+    const unsigned long long raw =
+        static_cast<unsigned long long>(__float_as_uint(a)) | (static_cast<unsigned long long>(__float_as_uint(b)) << 32);
+    __hip_atomic_store(as_global(reinterpret_cast<unsigned long long *>(p)), raw, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float4 ld_agent4(const float4 *p) {
+    const float2 lo = ld_agent2(reinterpret_cast<const float *>(p)), hi = ld_agent2(reinterpret_cast<const float *>(p) + 2);
+    return make_float4(lo.x, lo.y, hi.x, hi.y);
+}
+__device__ __forceinline__ void st_agent4(float4 *p, const float4 &v) {
+    st_agent2(reinterpret_cast<float *>(p), v.x, v.y);
+    st_agent2(reinterpret_cast<float *>(p) + 2, v.z, v.w);
+}
+
+template <bool AGENT>
+__device__ __forceinline__ float2 ld2(const float *p) {
+    if constexpr (AGENT) return ld_agent2(p);
+    else {
+        const lhip_f32x2 v = *as_global(reinterpret_cast<const lhip_f32x2 *>(p));
+        return make_float2(v.x, v.y);
+    }
+}
+template <bool AGENT>
+__device__ __forceinline__ float ld1(const float *p) {
+    if constexpr (AGENT) return ld_agent(p);
+    else return *as_global(p);
+}
+template <bool AGENT>
+__device__ __forceinline__ float4 ld4(const float4 *p) {
+    if constexpr (AGENT) return ld_agent4(p);
+    else return ldg4(p);
+}
+template <bool AGENT>
+__device__ __forceinline__ void st1(float *p, float v) {
+    if constexpr (AGENT) st_agent(p, v);
+    else *as_global(p) = v;
+}
+template <bool AGENT>
+__device__ __forceinline__ void st4(float4 *p, const float4 &v) {
+    if constexpr (AGENT) st_agent4(p, v);
+    else stg4(p, v);
+}
+
+// Workspace: [float ml[kv_heads][splits][G][2]] padded to a multiple of 256 B, [float acc[kv_heads][splits][G][HD]].
+static inline size_t dec_ml_bytes(int64_t kv_heads, int splits, int64_t g) {
+    return (static_cast<size_t>(kv_heads) * splits * g * 2 * sizeof(float) + 255) & ~size_t{255};
+}
+static inline int dec_splits(int64_t kv_heads) {
+    int64_t s = 256 / kv_heads;
+    return static_cast<int>(s < 1 ? 1 : (s > 64 ? 64 : s));
+}
+
+// LDS of one workgroup in the attention body.
+template <int G, int HD>
+struct AttnShared {
+    static constexpr int C4 = HD / 4;             // float4 columns of a row
+    static constexpr int KG = kDecThreads / C4;   // key groups in P.V
+    float4 q_s[G][C4];
+    float4 knew[C4], vnew[C4];
+    float p_s[G][kDecTile];
+    float m_s[G], l_s[G], corr_s[G];
+    float4 part[KG][G][C4];
+};
+
+// One (KV head, key range) piece: rotary on the G query rows and the new key, append of the new key / value to
+// the caches when the range holds the new position, attention over the range, partial state to the workspace.
+//
+// Inside a workgroup (256 working threads), per tile of 64 keys:
+//   scores: 4 lanes per key, each reading float4 columns sub, sub+4, ... of the row, so a
+//           quad covers 64 contiguous bytes per load; q for the G heads comes from LDS;
+//   online softmax: wave w owns heads w, w+4: lane = key;
+//   P.V:    HD/4 lanes cover a V row as float4, 256/(HD/4) key groups split the tile.
+// The K and V loads of a tile are all issued before the first use.
+template <int G, int HD, int THREADS, bool AGENT>
+__device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int kvh, int split,
+                                                      const float *__restrict__ qkv, float *__restrict__ k_cache,
+                                                      float *__restrict__ v_cache, int pos, int hkv, int max_seq,
+                                                      float theta, int n_splits, float *__restrict__ ws_ml,
+                                                      float4 *__restrict__ ws_acc) {
+    constexpr int C4 = HD / 4;
+    constexpr int KG = kDecThreads / C4;     // key groups in P.V
+    constexpr int KPG = kDecTile / KG;       // keys per group and tile
+    constexpr int J = HD / 16;               // float4 per lane and key in the scores
+    static_assert(KG * KPG == kDecTile && J * 16 == HD, "tile shape");
+    static_assert(THREADS >= kDecThreads && THREADS % 64 == 0, "workgroup size");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool on = THREADS == kDecThreads || tid < kDecThreads;  // wave-uniform
+    const int hq = hkv * G;
+    const int n_keys = min(pos + 1, max_seq);
+    const int chunk = (n_keys + n_splits - 1) / n_splits;
+    const int k0 = split * chunk, k1 = min(n_keys, k0 + chunk);
+    const float inv_sqrt = 1.0f / sqrtf(static_cast<float>(HD));
+    const float4 *kc4 = reinterpret_cast<const float4 *>(k_cache) + static_cast<size_t>(kvh) * max_seq * C4;
+    const float4 *vc4 = reinterpret_cast<const float4 *>(v_cache) + static_cast<size_t>(kvh) * max_seq * C4;
+
+    // ---- rotary on the G query rows and the new key (adjacent pairs, as the rope operator), copy of the new value
+    if (on) {
+        for (int i = tid; i < (G + 1) * (HD / 2); i += kDecThreads) {
+            const int r = i / (HD / 2), j = i - r * (HD / 2);
+            const float *row = qkv + static_cast<size_t>(r < G ? kvh * G + r : hq + kvh) * HD;
+            const float inv_freq = 1.0f / powf(theta, static_cast<float>(2 * j) / static_cast<float>(HD));
+            const float ang = static_cast<float>(pos) * inv_freq;
+            float sn, cs;
+            sincosf(ang, &sn, &cs);
+            const float2 x = ld2<AGENT>(row + 2 * j);
+            float *dst = r < G ? reinterpret_cast<float *>(sh.q_s[r]) : reinterpret_cast<float *>(sh.knew);
+            dst[2 * j] = x.x * cs - x.y * sn;
+            dst[2 * j + 1] = x.x * sn + x.y * cs;
+        }
+        for (int i = tid; i < HD; i += kDecThreads)
+            reinterpret_cast<float *>(sh.vnew)[i] = ld1<AGENT>(qkv + static_cast<size_t>(hq + hkv + kvh) * HD + i);
+        if (tid < G) {
+            sh.m_s[tid] = -INFINITY;
+            sh.l_s[tid] = 0.f;
+        }
+    }
+    __syncthreads();
+    if (on && pos < max_seq && pos >= k0 && pos < k1 && tid < C4) {  // this range holds the new position
+        stg4(reinterpret_cast<float4 *>(k_cache) + (static_cast<size_t>(kvh) * max_seq + pos) * C4 + tid, sh.knew[tid]);
+        stg4(reinterpret_cast<float4 *>(v_cache) + (static_cast<size_t>(kvh) * max_seq + pos) * C4 + tid, sh.vnew[tid]);
+    }
+
+    float4 acc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) acc[g] = make_float4(0, 0, 0, 0);
+    const int sub = tid & 3, kslot = (tid >> 2) & (kDecTile - 1);  // scores: 4 lanes per key
+    const int c4 = tid % C4, kgp = (tid / C4) % KG;                // P.V: column and key group
+
+    for (int t0 = k0; t0 < k1; t0 += kDecTile) {
+        // ---- all loads of the tile; the new position is served from LDS (its cache row may not have landed)
+        const int key = t0 + kslot;
+        const bool live = key < k1;
+        float4 kreg[J];
+        float4 vreg[KPG];
+        if (on) {
+            const float4 *krow = kc4 + static_cast<size_t>(live ? key : k0) * C4;
+#pragma unroll
+            for (int j = 0; j < J; ++j) kreg[j] = (key == pos) ? sh.knew[j * 4 + sub] : ldg4(krow + j * 4 + sub);
+#pragma unroll
+            for (int u = 0; u < KPG; ++u) {
+                const int vkey = t0 + kgp + KG * u;
+                vreg[u] = (vkey == pos) ? sh.vnew[c4] : ldg4(vc4 + static_cast<size_t>(vkey < k1 ? vkey : k0) * C4 + c4);
+            }
+            // ---- scores
+            float s[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float d = 0.f;
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const float4 qv = sh.q_s[g][j * 4 + sub];
+                    d += qv.x * kreg[j].x + qv.y * kreg[j].y + qv.z * kreg[j].z + qv.w * kreg[j].w;
+                }
+                d += __shfl_xor(d, 1);
+                d += __shfl_xor(d, 2);
+                s[g] = d * inv_sqrt;
+            }
+            if (sub == 0) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) sh.p_s[g][kslot] = live ? s[g] : -INFINITY;
+            }
+        }
+        __syncthreads();
+        // ---- online softmax: running max and sum per head, weights back into p_s
+        if (on) {
+            for (int g = wave; g < G; g += kDecThreads / 64) {
+                const float sv = sh.p_s[g][lane];
+                const float m_old = sh.m_s[g];
+                const float m_new = fmaxf(m_old, wave_max64(sv));  // finite: every tile has a live key
+                const float p = expf(sv - m_new);
+                const float psum = wave_sum64(p);
+                const float c = expf(m_old - m_new);
+                sh.p_s[g][lane] = p;
+                if (lane == 0) {
+                    sh.m_s[g] = m_new;
+                    sh.l_s[g] = sh.l_s[g] * c + psum;
+                    sh.corr_s[g] = c;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- P.V
+        if (on) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float c = sh.corr_s[g];
+                float4 a = make_float4(acc[g].x * c, acc[g].y * c, acc[g].z * c, acc[g].w * c);
+#pragma unroll
+                for (int u = 0; u < KPG; ++u) {
+                    const float w = sh.p_s[g][kgp + KG * u];  // 0 for keys past the range
+                    a.x += w * vreg[u].x; a.y += w * vreg[u].y; a.z += w * vreg[u].z; a.w += w * vreg[u].w;
+                }
+                acc[g] = a;
+            }
+        }
+        __syncthreads();  // p_s is rewritten by the next tile
+    }
+
+    // ---- partial state of this range -> workspace
+    if (k0 < k1) {  // uniform over the workgroup
+        if (on) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) sh.part[kgp][g][c4] = acc[g];
+        }
+        __syncthreads();
+        const size_t slot = static_cast<size_t>(kvh) * n_splits + split;
+        if (tid < G * C4) {
+            const int g = tid / C4, c = tid - g * C4;
+            float4 t = sh.part[0][g][c];
+#pragma unroll
+            for (int q = 1; q < KG; ++q) {
+                const float4 u = sh.part[q][g][c];
+                t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+            }
+            st4<AGENT>(ws_acc + (slot * G + g) * C4 + c, t);
+        }
+        if (tid < G) {
+            st1<AGENT>(ws_ml + (slot * G + tid) * 2, sh.m_s[tid]);
+            st1<AGENT>(ws_ml + (slot * G + tid) * 2 + 1, sh.l_s[tid]);
+        }
+    }
+}
+
+// LDS of one workgroup in the merge body.
+template <int G>
+struct MergeShared {
+    float2 ml_s[64 * G];
+    float4 num_s[kDecThreads];
+    float den_s[kDecThreads];
+};
+
+// Merge of the partial states of one KV head.  The (max, sum) pairs go to LDS in one round trip, then the 256
+// working threads split the ranges between them (SG threads per output float4, four loads in flight each) and
+// meet in LDS.
+template <int G, int HD, int THREADS, bool AGENT>
+__device__ __forceinline__ void attention_merge_body(MergeShared<G> &sh, int kvh, float *__restrict__ out, int pos,
+                                                     int max_seq, int n_splits, const float *__restrict__ ws_ml,
+                                                     const float4 *__restrict__ ws_acc) {
+    constexpr int C4 = HD / 4;
+    constexpr int P = G * C4;              // output float4s of this KV head
+    constexpr int SG = kDecThreads / P;    // threads per output
+    static_assert(P * SG == kDecThreads, "merge shape");
+    const int tid = threadIdx.x;
+    const bool on = THREADS == kDecThreads || tid < kDecThreads;
+    const int n_keys = min(pos + 1, max_seq);
+    const int chunk = (n_keys + n_splits - 1) / n_splits;
+    const int n_active = (n_keys + chunk - 1) / chunk;  // ranges that held keys
+    const size_t base = static_cast<size_t>(kvh) * n_splits;
+    if (on)
+        for (int i = tid; i < n_active * G; i += kDecThreads) sh.ml_s[i] = ld2<AGENT>(ws_ml + (base * G + i) * 2);
+    __syncthreads();
+    const int pair = tid % P, sg = (tid / P) % SG;
+    const int g = pair / C4, c = pair - g * C4;
+    float den = 0.f;
+    float4 num = make_float4(0, 0, 0, 0);
+    if (on) {
+        float mx = -INFINITY;
+        for (int sidx = 0; sidx < n_active; ++sidx) mx = fmaxf(mx, sh.ml_s[sidx * G + g].x);
+        for (int s0 = sg; s0 < n_active; s0 += 4 * SG) {
+            float4 a[4];
+            float w[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int sidx = s0 + u * SG;
+                const bool live = sidx < n_active;
+                a[u] = ld4<AGENT>(ws_acc + ((base + (live ? sidx : 0)) * G + g) * C4 + c);
+                const float2 v = sh.ml_s[(live ? sidx : 0) * G + g];
+                w[u] = live ? expf(v.x - mx) : 0.f;
+                den += v.y * w[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                num.x += a[u].x * w[u]; num.y += a[u].y * w[u]; num.z += a[u].z * w[u]; num.w += a[u].w * w[u];
+            }
+        }
+        sh.num_s[sg * P + pair] = num;
+        sh.den_s[sg * P + pair] = den;
+    }
+    __syncthreads();
+    if (on && sg == 0) {
+        for (int q = 1; q < SG; ++q) {
+            const float4 u = sh.num_s[q * P + pair];
+            num.x += u.x; num.y += u.y; num.z += u.z; num.w += u.w;
+            den += sh.den_s[q * P + pair];
+        }
+        const float inv = 1.0f / den;
+        st4<AGENT>(reinterpret_cast<float4 *>(out) + static_cast<size_t>(kvh * G + g) * C4 + c,
+                   make_float4(num.x * inv, num.y * inv, num.z * inv, num.w * inv));
+    }
+}
+
+}  // namespace lhip

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from . import capi
-from .quantized import FusedMatvec, Q8Weight
+from .quantized import DecodeProgram, FusedMatvec, Q8Weight
 
 
 @dataclass(frozen=True)
@@ -68,6 +68,10 @@ class LlamaQ8:
         # The fused matvec stages K activations in LDS in slices of 1024.
         self.fused_decode = all(k % 1024 == 0 and k <= 16384 for k in (cfg.dim, cfg.ffn))
         self._plans = None
+        # One persistent launch per decode step where the library builds it for these shapes; otherwise (and with
+        # persistent_decode = False) one launch per fused operator.
+        self.persistent_decode = True
+        self._program = None
         ws = self.lib.lhip_attention_decode_workspace_nbytes(cfg.q_heads, cfg.kv_heads, cfg.head_dim)
         self._attn_ws = torch.empty(ws, dtype=torch.uint8, device=self.dev) if ws else None
 
@@ -245,6 +249,23 @@ class LlamaQ8:
                 FusedMatvec([w[f"{i}.down"]], [h], residual=h, epilogue=FusedMatvec.EPI_ADD)))
         head = FusedMatvec([w["lm_head"]], [logits], norm_weight=w["out_norm"], eps=cfg.eps)
         self._plans = (plans, head, h, qkv, att, act, logits)
+        self._program = None
+        if self.persistent_decode and self._attn_ws is not None:
+            # the same operations as one persistent launch (lhip_decode_program_*)
+            prog = DecodeProgram(cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.max_seq, cfg.theta, self.pos)
+            for i in range(cfg.layers):
+                prog.matvec(w[f"{i}.qkv"], h, qkv, norm_weight=w[f"{i}.attn_norm"], eps=cfg.eps)
+                prog.attention(qkv, self.k_cache[i], self.v_cache[i], att)
+                prog.matvec(w[f"{i}.o"], att, h, residual=h, epilogue=FusedMatvec.EPI_ADD)
+                prog.matvec(w[f"{i}.gate_up"], h, act, norm_weight=w[f"{i}.ffn_norm"], eps=cfg.eps,
+                            epilogue=FusedMatvec.EPI_SWIGLU)
+                prog.matvec(w[f"{i}.down"], act, h, residual=h, epilogue=FusedMatvec.EPI_ADD)
+            prog.matvec(w["lm_head"], h, logits, norm_weight=w["out_norm"], eps=cfg.eps)
+            try:
+                self._program = prog.build()
+            except capi.LhipError as e:
+                if e.status != capi.LHIP_ERR_UNSUPPORTED:
+                    raise
 
     def forward_decode(self, token_f32: torch.Tensor):
         """One token at position pos through the fused batch-1 path; returns the logits (vocab,)."""
@@ -256,6 +277,9 @@ class LlamaQ8:
             self._build_plans()
         plans, head, h, qkv, att, act, logits = self._plans
         self._embed(token_f32, h, 1)
+        if self._program is not None:
+            self._program.run()
+            return logits
         for i, (p_qkv, p_o, p_gu, p_down) in enumerate(plans):
             p_qkv.run(h)                                   # qkv = Wqkv norm(h)
             self._attend_one(i, qkv, att)

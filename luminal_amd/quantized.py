@@ -205,3 +205,74 @@ class FusedMatvec:
             st = self.lib.lhip_q8_0_matvec_fused_f32(self._w, self._y, self._n, self.count, _ptr(x), self.k,
                                                      self._norm, self.eps, self._res, self.epilogue, _stream())
         capi.check(st, "lhip_q8_0_matvec_fused_f32")
+
+
+class DecodeProgram:
+    """A batch-1 decode step as one persistent launch (lhip_decode_program_*): a list of fused matvecs and attention
+    operations that a resident grid walks in order.  Operand addresses are fixed at construction; `run` queues the
+    launch on the current stream, `timed_out` asks (after a device sync) whether a grid-wide wait ever gave up."""
+
+    def __init__(self, q_heads: int = 0, kv_heads: int = 0, head_dim: int = 0, max_seq: int = 0, theta: float = 0.0,
+                 pos: torch.Tensor | None = None):
+        self._geom = (q_heads, kv_heads, head_dim, max_seq, float(theta))
+        self._pos = pos
+        self._ops, self._keep, self._handle = [], [], None
+        self.lib = capi.load_library()
+
+    def matvec(self, w: Q8Weight, x: torch.Tensor, y: torch.Tensor, norm_weight: torch.Tensor | None = None,
+               eps: float = 0.0, residual: torch.Tensor | None = None, epilogue: int = 0):
+        want = w.n // 2 if epilogue == FusedMatvec.EPI_SWIGLU else w.n
+        for t, size, what in ((x, w.k, "activation"), (y, want, "output")):
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != size or not t.is_contiguous():
+                raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", f"{what} must be f32 ({size},)")
+        if norm_weight is not None and (norm_weight.dtype != torch.float32 or norm_weight.numel() != w.k):
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", "norm weight is f32 (K,)")
+        if residual is not None and (residual.dtype != torch.float32 or residual.numel() != w.n):
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", "residual is f32 (n,)")
+        self._keep += [w, x, y, norm_weight, residual]
+        self._ops.append(capi.DecodeOp(capi.LHIP_DECODE_MATVEC, int(epilogue), w.planar.data_ptr(), w.n, w.k,
+                                       x.data_ptr(), y.data_ptr(),
+                                       norm_weight.data_ptr() if norm_weight is not None else None, float(eps),
+                                       residual.data_ptr() if residual is not None else None, None, None))
+        return self
+
+    def attention(self, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor):
+        q_heads, kv_heads, head_dim, max_seq, _ = self._geom
+        sizes = ((qkv, (q_heads + 2 * kv_heads) * head_dim), (out, q_heads * head_dim),
+                 (k_cache, kv_heads * max_seq * head_dim), (v_cache, kv_heads * max_seq * head_dim))
+        for t, size in sizes:
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != size or not t.is_contiguous():
+                raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", "attention operand shapes")
+        self._keep += [qkv, k_cache, v_cache, out]
+        self._ops.append(capi.DecodeOp(capi.LHIP_DECODE_ATTENTION, 0, None, 0, 0, qkv.data_ptr(), out.data_ptr(), None,
+                                       0.0, None, k_cache.data_ptr(), v_cache.data_ptr()))
+        return self
+
+    def build(self):
+        import ctypes as C
+
+        if self._handle is not None:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", "already built")
+        if self._pos is None or self._pos.dtype != torch.int32 or not self._pos.is_cuda:
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "DecodeProgram", "pos must be an int32 device tensor")
+        arr = (capi.DecodeOp * len(self._ops))(*self._ops)
+        handle = C.c_void_p()
+        capi.check(self.lib.lhip_decode_program_create(arr, len(self._ops), *self._geom, self._pos.data_ptr(),
+                                                       C.byref(handle)), "lhip_decode_program_create")
+        self._handle = handle
+        return self
+
+    def run(self):
+        capi.check(self.lib.lhip_decode_program_run(self._handle, _stream()), "lhip_decode_program_run")
+
+    def timed_out(self) -> bool:
+        import ctypes as C
+
+        flag = C.c_int32()
+        capi.check(self.lib.lhip_decode_program_status(self._handle, C.byref(flag)), "lhip_decode_program_status")
+        return bool(flag.value)
+
+    def __del__(self):
+        if getattr(self, "_handle", None) is not None:
+            self.lib.lhip_decode_program_destroy(self._handle)
+            self._handle = None
