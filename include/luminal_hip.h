@@ -355,30 +355,41 @@ lhip_status lhip_attention_bf16(const float *qkv_dev, const float *k_cache_dev, 
                                 int64_t kv_heads, int64_t head_dim, int64_t max_seq, void *stream);
 /* ---- persistent decode program --------------------------------------------
  * A batch-1 decode step as ONE launch: a list of operations that a resident grid (one workgroup
- * per compute unit) walks in order, a grid-wide barrier between consecutive phases, the weight
- * stream running across the barriers.  No counterpart in the reference, whose graph executor
- * runs one operator per kernel launch (src/graph.rs execute loop); the operations are those of
- * examples/llama/src/model.rs:95-139,150-160 in the fused forms of lhip_q8_0_matvec_fused_f32 and
- * lhip_attention_decode_f32, with the same arithmetic and reduction orders.
+ * per compute unit) walks in order, the weight stream running on from one operation to the next.
+ * No counterpart in the reference, whose graph executor runs one operator per kernel launch
+ * (src/graph.rs execute loop); the operations are those of examples/llama/src/model.rs:95-139,150-160
+ * in the fused forms of lhip_q8_0_matvec_fused_f32 and lhip_attention_decode_f32, with the same
+ * arithmetic and reduction orders: the results equal those calls bit for bit.
+ *
+ * On MI355X this form is SLOWER than the per-operator launches replayed from a graph (Llama-3-8B:
+ * 2.9 against 2.2 ms per token): what a launch boundary costs there (~7 us) is less than what the
+ * exchange of an activation vector between 256 resident workgroups costs here.  It is kept as a
+ * measured alternative, for parts and shapes where that balance differs.
  *
  * Operations:
  *   LHIP_DECODE_MATVEC     y = epilogue(W norm(x)): planar (n, k) weight, x (k floats), y (n floats; n / 2 for
  *                          SwiGLU, whose weight holds gate and up rows interleaved), norm_weight NULL or the k
  *                          gains of an RMS norm with eps, epilogue one of LHIP_FUSE_*, residual (n floats, may
  *                          be y) for LHIP_FUSE_ADD.  k % 1024 == 0 and k <= 14336 (LHIP_ERR_UNSUPPORTED beyond).
- *   LHIP_DECODE_ATTENTION  rotary + cache append + attention for the new token at *pos_dev: x = fused qkv row,
- *                          y = attention output rows, k_cache / v_cache of the layer.  Head geometry is that of
- *                          the create call: head_dim 64 or 128, q_heads / kv_heads in {1, 2, 4, 8}.
- * Every buffer an operation writes must differ from the buffers it reads, except y == residual; an operation
- * may read what any earlier one wrote.  Pointers are captured at creation; *pos_dev is read at every run.
+ *   LHIP_DECODE_ATTENTION  rotary + cache append + attention for the new token at *pos_dev: x = fused qkv row
+ *                          (must be the output of an earlier operation), y = attention output rows, k_cache /
+ *                          v_cache of the layer.  Head geometry is that of the create call: head_dim 64 or 128,
+ *                          q_heads / kv_heads in {1, 2, 4, 8}.
+ * Buffers are told apart by their base address and must not overlap otherwise.  x != y.  Workgroups are not
+ * held back by a barrier: each waits only for the values it reads, which travel with the tag of the operation
+ * that produced them.  An operation may therefore overwrite a buffer only if its own input x was produced at
+ * or after the last operation that read, and the operation that wrote, the buffer's previous contents (y ==
+ * residual of the same operation is fine); a list that breaks this is refused with LHIP_ERR_UNSUPPORTED.  The
+ * decode loop of a transformer (h -> qkv -> attention -> h -> act -> h ...) satisfies it.  After a run every y
+ * holds its operation's result.  Pointers are captured at creation; *pos_dev is read at every run.
  *
- * lhip_decode_program_run queues two kernels on the stream (a clear of the barrier counters, then the
- * program) and allocates nothing, so it can be captured into a graph.  Runs of one program must not overlap
- * in time.  The program kernel needs every compute unit of the device to itself while it runs: all of its
- * workgroups must be resident together, which holds when nothing else occupies the device (kernels queued
- * before it on any stream simply finish first).  Every wait inside is bounded (about a second): if the
- * workgroups fail to meet, the kernel still ends, the step's results are meaningless, and
- * lhip_decode_program_status (which waits for the device) reports *timed_out = 1 from then on. */
+ * lhip_decode_program_run queues two kernels on the stream (a one-thread kernel that starts a new tag range,
+ * then the program) and allocates nothing, so it can be captured into a graph.  Runs of one program must not
+ * overlap in time.  The program kernel needs every compute unit of the device to itself while it runs: all of
+ * its workgroups must be resident together, which holds when nothing else occupies the device (kernels queued
+ * before it simply finish first).  Every wait inside is bounded (about a second): if values fail to arrive,
+ * the kernel still ends, the step's results are meaningless, and lhip_decode_program_status (which waits for
+ * the device) reports *timed_out = 1 from then on. */
 enum { LHIP_DECODE_MATVEC = 0, LHIP_DECODE_ATTENTION = 1 };
 enum { LHIP_FUSE_NONE = 0, LHIP_FUSE_ADD = 1, LHIP_FUSE_SWIGLU = 2 };
 typedef struct lhip_decode_op {
@@ -398,6 +409,13 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
                                        void **program);
 lhip_status lhip_decode_program_run(void *program, void *stream);
 lhip_status lhip_decode_program_status(void *program, int32_t *timed_out);
+/* Per-phase clock of later runs (a profiler sees the program as one kernel): with ticks_dev != NULL, workgroup 0
+ * writes the 100 MHz wall clock when it enters phase p to ticks_dev[2 p] and when it has finished its own share of
+ * the phase (the wait for the phase's input included) to ticks_dev[2 p + 1].  *n_phases (if
+ * given) receives the number of phases: an attention operation is two (attention, merge of the key ranges).
+ * ticks_dev holds 2 * n_phases values, 8-byte aligned; NULL switches the trace off.  Takes effect at the next run
+ * (not in runs already captured into a graph). */
+lhip_status lhip_decode_program_trace(void *program, uint64_t *ticks_dev, int32_t *n_phases);
 lhip_status lhip_decode_program_destroy(void *program);
 
 /* Element-wise casts between f32 and bf16 (round to nearest even), for feeding f32

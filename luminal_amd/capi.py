@@ -41,6 +41,7 @@ SIGNATURES = {
     "lhip_decode_program_run": (C.c_int32, [_vp, _vp]),
     "lhip_decode_program_status": (C.c_int32, [_vp, C.POINTER(C.c_int32)]),
     "lhip_decode_program_destroy": (C.c_int32, [_vp]),
+    "lhip_decode_program_trace": (C.c_int32, [_vp, _vp, C.POINTER(C.c_int32)]),
     "lhip_q8_0_matvec_fused_f32": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _vp]),
     "lhip_q8_0_matvec_fused_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _int, _vp, _i64, _vp, C.c_float, _vp, _int, _int, _int,
                                                    _int, _int, _vp]),

@@ -11,17 +11,9 @@
 // one workgroup each (grid = kv_heads x splits, about one workgroup per CU), and the G
 // query heads that share a KV head are served by the same workgroup, which therefore
 // reads every cache row once.  Each workgroup writes its partial softmax state (max, sum,
-// weighted V) to a workspace and a second, small kernel merges the partials into the output
-// rows.  (Merging in the same launch needs device-scope release/acquire fences in every
-// workgroup; on this part each is a write-back plus invalidate of a whole L2 and the 256 of
-// them cost more than the second launch.)
-//
-// Inside a workgroup (256 threads), per tile of 64 keys:
-//   scores: 4 lanes per key, each reading float4 columns sub, sub+4, ... of the row, so a
-//           quad covers 64 contiguous bytes per load; q for the G heads comes from LDS;
-//   online softmax: wave w owns heads w, w+4: lane = key;
-//   P.V:    HD/4 lanes cover a V row as float4, 256/(HD/4) key groups split the tile.
-// The K and V loads of a tile are all issued before the first use.
+// weighted V) to a workspace and a second, small kernel (one workgroup per query head) merges
+// the partials into the output rows.  The bodies of both kernels live in
+// attention_decode_device.h, which describes the work inside a workgroup.
 #include "attention_decode_device.h"
 #include "common.h"
 
@@ -33,18 +25,18 @@ __global__ __launch_bounds__(kDecThreads) void attention_decode_kernel(
     const int *__restrict__ pos_dev, int hkv, int max_seq, float theta, int n_splits,
     float *__restrict__ ws_ml, float4 *__restrict__ ws_acc) {
     __shared__ AttnShared<G, HD> sh;
-    attention_decode_body<G, HD, kDecThreads, false>(sh, blockIdx.x, blockIdx.y, qkv, k_cache, v_cache, *pos_dev, hkv,
+    attention_decode_body<G, HD, kDecThreads>(PlainIO{}, sh, blockIdx.x, blockIdx.y, qkv, k_cache, v_cache, *pos_dev, hkv,
                                                      max_seq, theta, n_splits, ws_ml, ws_acc);
 }
 
-// One workgroup per KV head.
+// One workgroup per query head.
 template <int G, int HD>
 __global__ __launch_bounds__(kDecThreads) void attention_merge_kernel(float *__restrict__ out,
                                                                       const int *__restrict__ pos_dev, int max_seq,
                                                                       int n_splits, const float *__restrict__ ws_ml,
                                                                       const float4 *__restrict__ ws_acc) {
-    __shared__ MergeShared<G> sh;
-    attention_merge_body<G, HD, kDecThreads, false>(sh, blockIdx.x, out, *pos_dev, max_seq, n_splits, ws_ml, ws_acc);
+    __shared__ MergeShared sh;
+    attention_merge_body<G, HD, kDecThreads>(PlainIO{}, sh, blockIdx.x, out, *pos_dev, max_seq, n_splits, ws_ml, ws_acc);
 }
 
 template <int G, int HD>
@@ -57,7 +49,7 @@ static lhip_status launch_decode(const float *qkv, float *kc, float *vc, float *
     hipLaunchKernelGGL((attention_decode_kernel<G, HD>), dim3(static_cast<unsigned>(hkv), static_cast<unsigned>(splits)),
                        dim3(kDecThreads), 0, s, qkv, kc, vc, pos, hkv, max_seq, theta, splits, ml, acc);
     LHIP_CHECK_LAUNCH();
-    hipLaunchKernelGGL((attention_merge_kernel<G, HD>), dim3(static_cast<unsigned>(hkv)), dim3(kDecThreads), 0, s, out,
+    hipLaunchKernelGGL((attention_merge_kernel<G, HD>), dim3(static_cast<unsigned>(hkv * G)), dim3(kDecThreads), 0, s, out,
                        pos, max_seq, splits, ml, acc);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;

@@ -2,12 +2,18 @@
 // partial softmax states), shared by the two-launch form (attention_decode.hip) and by the persistent decode
 // program (decode_program.hip), where both run as phases of one kernel.
 //
+// Every sum of products below is spelled as explicit fused multiply-adds (or explicitly separate operations), so
+// that the instantiations of a body cannot differ in how the compiler contracts them: the forms agree bit for bit.
+//
 // Template switches:
 //   THREADS  threads of the workgroup that calls the body.  The work is laid out for kDecThreads = 256; further
 //            threads only take part in the barriers.
-//   AGENT    true when the inputs were written, and the outputs will be read, by other workgroups of the SAME
-//            launch.  Such data moves through agent-coherent loads and stores (they bypass the caches that are
-//            private to a part of the chip); within one launch plain accesses could meet stale lines.  The KV
+//   IO       how the operands that other kernels or workgroups produce / consume are accessed.  PlainIO: ordinary
+//            loads and stores (the two-launch form: a kernel boundary orders everything).  TaggedIO: the inputs
+//            were written, and the outputs will be read, by other workgroups of the SAME launch, with nothing
+//            but the data to synchronise on: every 32-bit value travels as one 64-bit word (value, tag) written
+//            and read with agent-coherent accesses (which bypass the caches private to a part of the chip); a
+//            reader polls until all the words it needs carry the tag of the phase that produces them.  The KV
 //            caches are exempt: rows of earlier positions come from earlier launches, and the row of the new
 //            position is served from LDS.
 #pragma once
@@ -82,33 +88,79 @@ __device__ __forceinline__ void st_agent4(float4 *p, const float4 &v) {
     st_agent2(reinterpret_cast<float *>(p) + 2, v.z, v.w);
 }
 
-template <bool AGENT>
-__device__ __forceinline__ float2 ld2(const float *p) {
-    if constexpr (AGENT) return ld_agent2(p);
-    else {
-        const lhip_f32x2 v = *as_global(reinterpret_cast<const lhip_f32x2 *>(p));
+// Operand access policies of the bodies below.  Addresses are given as (base, element index): a tagged array
+// has the element order of the plain one, 8 bytes per element.
+struct PlainIO {
+    __device__ __forceinline__ float ld1(const float *b, size_t i, bool &) const { return as_global(b)[i]; }
+    __device__ __forceinline__ float2 ld2(const float *b, size_t i, bool &) const {  // i even
+        const lhip_f32x2 v = *as_global(reinterpret_cast<const lhip_f32x2 *>(b + i));
         return make_float2(v.x, v.y);
     }
-}
-template <bool AGENT>
-__device__ __forceinline__ float ld1(const float *p) {
-    if constexpr (AGENT) return ld_agent(p);
-    else return *as_global(p);
-}
-template <bool AGENT>
-__device__ __forceinline__ float4 ld4(const float4 *p) {
-    if constexpr (AGENT) return ld_agent4(p);
-    else return ldg4(p);
-}
-template <bool AGENT>
-__device__ __forceinline__ void st1(float *p, float v) {
-    if constexpr (AGENT) st_agent(p, v);
-    else *as_global(p) = v;
-}
-template <bool AGENT>
-__device__ __forceinline__ void st4(float4 *p, const float4 &v) {
-    if constexpr (AGENT) st_agent4(p, v);
-    else stg4(p, v);
+    __device__ __forceinline__ float4 ld4(const float4 *b, size_t i4, bool &) const { return ldg4(b + i4); }
+    __device__ __forceinline__ void st1(float *b, size_t i, float v) const { as_global(b)[i] = v; }
+    __device__ __forceinline__ void st4(float4 *b, size_t i4, const float4 &v) const { stg4(b + i4, v); }
+    __device__ __forceinline__ bool again(bool) { return false; }
+};
+
+constexpr unsigned kTagSpinLimit = 1u << 20;
+
+struct TaggedIO {
+    unsigned in_tag, out_tag;
+    unsigned *abort_flag, *sticky;  // raised when a wait is given up; seen by every other waiter
+    unsigned spins = 0;
+    __device__ __forceinline__ float ld1(const float *b, size_t i, bool &ok) const {
+        const unsigned long long raw = __hip_atomic_load(as_global(reinterpret_cast<const unsigned long long *>(b)) + i,
+                                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && static_cast<unsigned>(raw >> 32) == in_tag;
+        return __uint_as_float(static_cast<unsigned>(raw));
+    }
+    __device__ __forceinline__ float2 ld2(const float *b, size_t i, bool &ok) const {
+        const float x = ld1(b, i, ok), y = ld1(b, i + 1, ok);
+        return make_float2(x, y);
+    }
+    __device__ __forceinline__ float4 ld4(const float4 *b, size_t i4, bool &ok) const {
+        const float *f = reinterpret_cast<const float *>(b);
+        const float x = ld1(f, 4 * i4, ok), y = ld1(f, 4 * i4 + 1, ok), z = ld1(f, 4 * i4 + 2, ok), w = ld1(f, 4 * i4 + 3, ok);
+        return make_float4(x, y, z, w);
+    }
+    __device__ __forceinline__ void st1(float *b, size_t i, float v) const {
+        const unsigned long long raw =
+            static_cast<unsigned long long>(__float_as_uint(v)) | (static_cast<unsigned long long>(out_tag) << 32);
+        __hip_atomic_store(as_global(reinterpret_cast<unsigned long long *>(b)) + i, raw, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ void st4(float4 *b, size_t i4, const float4 &v) const {
+        float *f = reinterpret_cast<float *>(b);
+        st1(f, 4 * i4, v.x);
+        st1(f, 4 * i4 + 1, v.y);
+        st1(f, 4 * i4 + 2, v.z);
+        st1(f, 4 * i4 + 3, v.w);
+    }
+    // After a round of loads: true = some word was not there yet, load again.  Bounded: past the limit, or once
+    // anybody has given up, the caller goes on with whatever it has.
+    __device__ __forceinline__ bool again(bool ok) {
+        if (ok) return false;
+        ++spins;
+        if (spins > kTagSpinLimit) {
+            __hip_atomic_store(as_global(abort_flag), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(as_global(sticky), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return false;
+        }
+        if ((spins & 63u) == 0u &&
+            __hip_atomic_load(as_global(abort_flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
+            return false;
+        return true;
+    }
+};
+
+// sin and cos of the rotary angle pos / theta^(two_j / hd).  Kept out of line: the library routines inside are
+// open to re-association, and a copy inlined into each caller could round differently from caller to caller.
+__device__ __noinline__ float2 rope_sin_cos(float theta, int two_j, int hd, int pos) {
+    const float inv_freq = 1.0f / powf(theta, static_cast<float>(two_j) / static_cast<float>(hd));
+    const float ang = static_cast<float>(pos) * inv_freq;
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    return make_float2(sn, cs);
 }
 
 // Workspace: [float ml[kv_heads][splits][G][2]] padded to a multiple of 256 B, [float acc[kv_heads][splits][G][HD]].
@@ -141,8 +193,8 @@ struct AttnShared {
 //   online softmax: wave w owns heads w, w+4: lane = key;
 //   P.V:    HD/4 lanes cover a V row as float4, 256/(HD/4) key groups split the tile.
 // The K and V loads of a tile are all issued before the first use.
-template <int G, int HD, int THREADS, bool AGENT>
-__device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int kvh, int split,
+template <int G, int HD, int THREADS, typename IO>
+__device__ __forceinline__ void attention_decode_body(IO io, AttnShared<G, HD> &sh, int kvh, int split,
                                                       const float *__restrict__ qkv, float *__restrict__ k_cache,
                                                       float *__restrict__ v_cache, int pos, int hkv, int max_seq,
                                                       float theta, int n_splits, float *__restrict__ ws_ml,
@@ -164,22 +216,57 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
     const float4 *kc4 = reinterpret_cast<const float4 *>(k_cache) + static_cast<size_t>(kvh) * max_seq * C4;
     const float4 *vc4 = reinterpret_cast<const float4 *>(v_cache) + static_cast<size_t>(kvh) * max_seq * C4;
 
+    // ---- cache rows of a tile of keys: all loads issued before the first use.  The first tile is requested at
+    // once, ahead of the wait for q: the caches do not depend on it (the row of the new position, which may not
+    // have been written yet, is replaced from LDS below).
+    const int sub = tid & 3, kslot = (tid >> 2) & (kDecTile - 1);  // scores: 4 lanes per key
+    const int c4 = tid % C4, kgp = (tid / C4) % KG;                // P.V: column and key group
+    float4 kreg[J];
+    float4 vreg[KPG];
+    auto load_tile = [&](int t0) {
+        const int key = t0 + kslot;
+        const float4 *krow = kc4 + static_cast<size_t>(key < k1 ? key : k0) * C4;
+#pragma unroll
+        for (int j = 0; j < J; ++j) kreg[j] = ldg4(krow + j * 4 + sub);
+#pragma unroll
+        for (int u = 0; u < KPG; ++u) {
+            const int vkey = t0 + kgp + KG * u;
+            vreg[u] = ldg4(vc4 + static_cast<size_t>(vkey < k1 ? vkey : k0) * C4 + c4);
+        }
+    };
+    if (on && k0 < k1) load_tile(k0);
+
     // ---- rotary on the G query rows and the new key (adjacent pairs, as the rope operator), copy of the new value
     if (on) {
-        for (int i = tid; i < (G + 1) * (HD / 2); i += kDecThreads) {
-            const int r = i / (HD / 2), j = i - r * (HD / 2);
-            const float *row = qkv + static_cast<size_t>(r < G ? kvh * G + r : hq + kvh) * HD;
-            const float inv_freq = 1.0f / powf(theta, static_cast<float>(2 * j) / static_cast<float>(HD));
-            const float ang = static_cast<float>(pos) * inv_freq;
-            float sn, cs;
-            sincosf(ang, &sn, &cs);
-            const float2 x = ld2<AGENT>(row + 2 * j);
-            float *dst = r < G ? reinterpret_cast<float *>(sh.q_s[r]) : reinterpret_cast<float *>(sh.knew);
-            dst[2 * j] = x.x * cs - x.y * sn;
-            dst[2 * j + 1] = x.x * sn + x.y * cs;
+        constexpr int NPAIR = (G + 1) * (HD / 2);
+        constexpr int ITER = (NPAIR + kDecThreads - 1) / kDecThreads;
+        float2 xr[ITER];
+        float vn = 0.f;
+        bool ok;
+        do {  // the raw values first (in the tagged form: until all of them are there), the arithmetic once
+            ok = true;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int i = min(tid + it * kDecThreads, NPAIR - 1);
+                const int r = i / (HD / 2), j = i - r * (HD / 2);
+                xr[it] = io.ld2(qkv, static_cast<size_t>(r < G ? kvh * G + r : hq + kvh) * HD + 2 * j, ok);
+            }
+            if (tid < HD) vn = io.ld1(qkv, static_cast<size_t>(hq + hkv + kvh) * HD + tid, ok);
+        } while (io.again(ok));
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int i = tid + it * kDecThreads;
+            if (i < NPAIR) {
+                const int r = i / (HD / 2), j = i - r * (HD / 2);
+                const float2 sc = rope_sin_cos(theta, 2 * j, HD, pos);
+                const float sn = sc.x, cs = sc.y;
+                float *dst = r < G ? reinterpret_cast<float *>(sh.q_s[r]) : reinterpret_cast<float *>(sh.knew);
+                // products rounded one by one, as the rope operator of the graph does
+                dst[2 * j] = __fsub_rn(__fmul_rn(xr[it].x, cs), __fmul_rn(xr[it].y, sn));
+                dst[2 * j + 1] = __fadd_rn(__fmul_rn(xr[it].x, sn), __fmul_rn(xr[it].y, cs));
+            }
         }
-        for (int i = tid; i < HD; i += kDecThreads)
-            reinterpret_cast<float *>(sh.vnew)[i] = ld1<AGENT>(qkv + static_cast<size_t>(hq + hkv + kvh) * HD + i);
+        if (tid < HD) reinterpret_cast<float *>(sh.vnew)[tid] = vn;
         if (tid < G) {
             sh.m_s[tid] = -INFINITY;
             sh.l_s[tid] = 0.f;
@@ -194,24 +281,19 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
     float4 acc[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) acc[g] = make_float4(0, 0, 0, 0);
-    const int sub = tid & 3, kslot = (tid >> 2) & (kDecTile - 1);  // scores: 4 lanes per key
-    const int c4 = tid % C4, kgp = (tid / C4) % KG;                // P.V: column and key group
-
     for (int t0 = k0; t0 < k1; t0 += kDecTile) {
-        // ---- all loads of the tile; the new position is served from LDS (its cache row may not have landed)
+        // ---- the tile's cache rows; the new position is served from LDS (its cache row may not have landed)
         const int key = t0 + kslot;
         const bool live = key < k1;
-        float4 kreg[J];
-        float4 vreg[KPG];
         if (on) {
-            const float4 *krow = kc4 + static_cast<size_t>(live ? key : k0) * C4;
+            if (t0 != k0) load_tile(t0);
+            if (key == pos) {
 #pragma unroll
-            for (int j = 0; j < J; ++j) kreg[j] = (key == pos) ? sh.knew[j * 4 + sub] : ldg4(krow + j * 4 + sub);
-#pragma unroll
-            for (int u = 0; u < KPG; ++u) {
-                const int vkey = t0 + kgp + KG * u;
-                vreg[u] = (vkey == pos) ? sh.vnew[c4] : ldg4(vc4 + static_cast<size_t>(vkey < k1 ? vkey : k0) * C4 + c4);
+                for (int j = 0; j < J; ++j) kreg[j] = sh.knew[j * 4 + sub];
             }
+#pragma unroll
+            for (int u = 0; u < KPG; ++u)
+                if (t0 + kgp + KG * u == pos) vreg[u] = sh.vnew[c4];
             // ---- scores
             float s[G];
 #pragma unroll
@@ -220,7 +302,10 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
 #pragma unroll
                 for (int j = 0; j < J; ++j) {
                     const float4 qv = sh.q_s[g][j * 4 + sub];
-                    d += qv.x * kreg[j].x + qv.y * kreg[j].y + qv.z * kreg[j].z + qv.w * kreg[j].w;
+                    d = fmaf(qv.x, kreg[j].x, d);
+                    d = fmaf(qv.y, kreg[j].y, d);
+                    d = fmaf(qv.z, kreg[j].z, d);
+                    d = fmaf(qv.w, kreg[j].w, d);
                 }
                 d += __shfl_xor(d, 1);
                 d += __shfl_xor(d, 2);
@@ -244,7 +329,7 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
                 sh.p_s[g][lane] = p;
                 if (lane == 0) {
                     sh.m_s[g] = m_new;
-                    sh.l_s[g] = sh.l_s[g] * c + psum;
+                    sh.l_s[g] = fmaf(sh.l_s[g], c, psum);
                     sh.corr_s[g] = c;
                 }
             }
@@ -259,7 +344,8 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
 #pragma unroll
                 for (int u = 0; u < KPG; ++u) {
                     const float w = sh.p_s[g][kgp + KG * u];  // 0 for keys past the range
-                    a.x += w * vreg[u].x; a.y += w * vreg[u].y; a.z += w * vreg[u].z; a.w += w * vreg[u].w;
+                    a.x = fmaf(w, vreg[u].x, a.x); a.y = fmaf(w, vreg[u].y, a.y);
+                    a.z = fmaf(w, vreg[u].z, a.z); a.w = fmaf(w, vreg[u].w, a.w);
                 }
                 acc[g] = a;
             }
@@ -283,80 +369,96 @@ __device__ __forceinline__ void attention_decode_body(AttnShared<G, HD> &sh, int
                 const float4 u = sh.part[q][g][c];
                 t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
             }
-            st4<AGENT>(ws_acc + (slot * G + g) * C4 + c, t);
+            io.st4(ws_acc, (slot * G + g) * C4 + c, t);
         }
         if (tid < G) {
-            st1<AGENT>(ws_ml + (slot * G + tid) * 2, sh.m_s[tid]);
-            st1<AGENT>(ws_ml + (slot * G + tid) * 2 + 1, sh.l_s[tid]);
+            io.st1(ws_ml, (slot * G + tid) * 2, sh.m_s[tid]);
+            io.st1(ws_ml, (slot * G + tid) * 2 + 1, sh.l_s[tid]);
         }
     }
 }
 
 // LDS of one workgroup in the merge body.
-template <int G>
 struct MergeShared {
-    float2 ml_s[64 * G];
+    float2 ml_s[64];  // (max, sum) of every key range, for the one head
     float4 num_s[kDecThreads];
     float den_s[kDecThreads];
 };
 
-// Merge of the partial states of one KV head.  The (max, sum) pairs go to LDS in one round trip, then the 256
-// working threads split the ranges between them (SG threads per output float4, four loads in flight each) and
-// meet in LDS.
-template <int G, int HD, int THREADS, bool AGENT>
-__device__ __forceinline__ void attention_merge_body(MergeShared<G> &sh, int kvh, float *__restrict__ out, int pos,
+// Merge of the partial states of one query head (head = kvh * G + g).  The 256 working threads are HD/4 output
+// columns x SG sub-groups; a thread takes the key ranges sg, sg + SG, ..., four per round of loads, the first round
+// together with the (max, sum) pairs, so that the usual 32 ranges cost a single memory round trip; the
+// sub-groups meet in LDS.
+template <int G, int HD, int THREADS, typename IO>
+__device__ __forceinline__ void attention_merge_body(IO io, MergeShared &sh, int head, float *__restrict__ out, int pos,
                                                      int max_seq, int n_splits, const float *__restrict__ ws_ml,
-                                                     const float4 *__restrict__ ws_acc) {
+                                                     const float4 *__restrict__ ws_acc,
+                                                     float *__restrict__ out_copy = nullptr) {
     constexpr int C4 = HD / 4;
-    constexpr int P = G * C4;              // output float4s of this KV head
-    constexpr int SG = kDecThreads / P;    // threads per output
-    static_assert(P * SG == kDecThreads, "merge shape");
+    constexpr int SG = kDecThreads / C4;  // sub-groups: 8 (HD 128) or 16 (HD 64)
     const int tid = threadIdx.x;
     const bool on = THREADS == kDecThreads || tid < kDecThreads;
+    const int kvh = head / G, g = head - kvh * G;
     const int n_keys = min(pos + 1, max_seq);
     const int chunk = (n_keys + n_splits - 1) / n_splits;
-    const int n_active = (n_keys + chunk - 1) / chunk;  // ranges that held keys
+    const int n_active = (n_keys + chunk - 1) / chunk;  // ranges that held keys (<= 64)
     const size_t base = static_cast<size_t>(kvh) * n_splits;
-    if (on)
-        for (int i = tid; i < n_active * G; i += kDecThreads) sh.ml_s[i] = ld2<AGENT>(ws_ml + (base * G + i) * 2);
+    const int c = tid % C4, sg = (tid / C4) % SG;
+    auto acc_index = [&](int sidx) { return ((base + min(sidx, n_active - 1)) * G + g) * C4 + c; };
+
+    float4 a[4];
+    float2 mine = make_float2(0.f, 0.f);
+    if (on) {
+        bool ok;
+        do {
+            ok = true;
+            if (tid < n_active) mine = io.ld2(ws_ml, ((base + tid) * G + g) * 2, ok);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) a[u] = io.ld4(ws_acc, acc_index(sg + u * SG), ok);
+        } while (io.again(ok));
+        if (tid < n_active) sh.ml_s[tid] = mine;
+    }
     __syncthreads();
-    const int pair = tid % P, sg = (tid / P) % SG;
-    const int g = pair / C4, c = pair - g * C4;
     float den = 0.f;
     float4 num = make_float4(0, 0, 0, 0);
     if (on) {
         float mx = -INFINITY;
-        for (int sidx = 0; sidx < n_active; ++sidx) mx = fmaxf(mx, sh.ml_s[sidx * G + g].x);
+        for (int sidx = 0; sidx < n_active; ++sidx) mx = fmaxf(mx, sh.ml_s[sidx].x);
         for (int s0 = sg; s0 < n_active; s0 += 4 * SG) {
-            float4 a[4];
-            float w[4];
+            if (s0 != sg) {  // further rounds (more than 4 * SG ranges)
+                bool ok;
+                do {
+                    ok = true;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) a[u] = io.ld4(ws_acc, acc_index(s0 + u * SG), ok);
+                } while (io.again(ok));
+            }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int sidx = s0 + u * SG;
                 const bool live = sidx < n_active;
-                a[u] = ld4<AGENT>(ws_acc + ((base + (live ? sidx : 0)) * G + g) * C4 + c);
-                const float2 v = sh.ml_s[(live ? sidx : 0) * G + g];
-                w[u] = live ? expf(v.x - mx) : 0.f;
-                den += v.y * w[u];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                num.x += a[u].x * w[u]; num.y += a[u].y * w[u]; num.z += a[u].z * w[u]; num.w += a[u].w * w[u];
+                const float2 v = sh.ml_s[live ? sidx : 0];
+                const float wgt = live ? expf(v.x - mx) : 0.f;
+                den = fmaf(v.y, wgt, den);
+                num.x = fmaf(a[u].x, wgt, num.x); num.y = fmaf(a[u].y, wgt, num.y);
+                num.z = fmaf(a[u].z, wgt, num.z); num.w = fmaf(a[u].w, wgt, num.w);
             }
         }
-        sh.num_s[sg * P + pair] = num;
-        sh.den_s[sg * P + pair] = den;
+        sh.num_s[sg * C4 + c] = num;
+        sh.den_s[sg * C4 + c] = den;
     }
     __syncthreads();
     if (on && sg == 0) {
         for (int q = 1; q < SG; ++q) {
-            const float4 u = sh.num_s[q * P + pair];
+            const float4 u = sh.num_s[q * C4 + c];
             num.x += u.x; num.y += u.y; num.z += u.z; num.w += u.w;
-            den += sh.den_s[q * P + pair];
+            den += sh.den_s[q * C4 + c];
         }
         const float inv = 1.0f / den;
-        st4<AGENT>(reinterpret_cast<float4 *>(out) + static_cast<size_t>(kvh * G + g) * C4 + c,
-                   make_float4(num.x * inv, num.y * inv, num.z * inv, num.w * inv));
+        const float4 o = make_float4(num.x * inv, num.y * inv, num.z * inv, num.w * inv);
+        io.st4(reinterpret_cast<float4 *>(out), static_cast<size_t>(head) * C4 + c, o);
+        // the tagged form writes a shadow array: the caller's own buffer gets the plain values as well
+        if (out_copy != nullptr) stg4(reinterpret_cast<float4 *>(out_copy) + static_cast<size_t>(head) * C4 + c, o);
     }
 }
 

@@ -5,25 +5,29 @@
 // rate once they are going, but every launch pays ~7 us around that: ~3 us between the end of one kernel and
 // the first wave of the next, ~2.5 us until the first weights and the staged activations have arrived, ~1.3 us
 // while the slowest waves finish.  With 6 launches per layer that is 40 us of a 65 us layer.  Here the grid
-// (one workgroup of 8 wavefronts per compute unit) stays resident and walks a list of phases; consecutive
-// phases are separated by a grid-wide barrier (~2.6 us), and the weight stream does not stop there: weights do
-// not depend on the previous phase, so every wave requests the first two pipeline steps of the next matvec
-// before it arrives at the barrier and holds them in registers across it.
+// (one workgroup of 8 wavefronts per compute unit) stays resident and walks a list of phases, and the weight
+// stream does not stop between them: weights do not depend on the previous phase, so every wave requests the
+// first two pipeline steps of the next matvec while it finishes the current one and holds them in registers.
 //
 // Phases.  MATVEC: the fused Q8_0 matvec of q8_gemv.hip (optional RMS-norm prologue; epilogues none / residual
 // add / SwiGLU) with the same per-row arithmetic and the same reduction orders, so results equal the per-kernel
 // path bit for bit where that path runs four-wave workgroups.  ATTENTION and MERGE: the bodies of
 // attention_decode_device.h, one (KV head, key range) piece or one KV head per workgroup.
 //
-// Coherence.  Data produced in one phase and consumed in a later one (activation vectors, attention partials)
-// crosses between workgroups of one launch, so it is written and read with agent-coherent accesses; no cache
-// write-back or invalidate is needed at the barrier, which is what makes it cheap.  A wave waits for its own
-// stores to be acknowledged, the workgroup meets, one thread adds to one of 8 arrival counters and the first
-// wave polls all 8 with one load.  Weights, norm gains and the KV caches of earlier positions are read-only
-// within a launch and use plain (non-temporal) loads.
+// Synchronisation is carried by the data.  A vector produced in one phase and consumed in a later one
+// (activations, attention partials) lives in a shadow array of 64-bit words (value, tag), the tag naming the
+// launch and the producing phase.  Producers write each word with one agent-coherent store; a consumer reads
+// the words it needs with agent-coherent loads and repeats until all of them carry the tag it expects.  There
+// is no barrier, no fence and no cache write-back: a consumer starts one memory round trip after the last
+// producer's store (measured: 1.8 us per hop for 256 workgroups exchanging 4096 values, against 2.6 us for a
+// counter barrier plus 3 us for the loads that can only start behind it), and workgroups that have nothing to
+// wait for run ahead.  An array may be overwritten two phases after it was written: a workgroup that writes in
+// phase p + 2 has read all of phase p + 1's output, so every workgroup has finished phase p + 1 and with it
+// its reads of phase p's output.  The program is checked for this when it is created.  Weights, norm gains and
+// the KV caches of earlier positions are read-only within a launch and use ordinary (non-temporal) loads.
 //
-// Termination.  Every wait is bounded: a workgroup that polls kSpinLimit times without seeing the others raises
-// a flag, everyone who sees the flag stops waiting, and the kernel runs to its end (with meaningless results).
+// Termination.  Every wait is bounded: a thread that repeats its loads kTagSpinLimit times raises a flag, every
+// other waiter that sees the flag stops waiting, and the kernel runs to its end (with meaningless results).
 // The flag is sticky and reported by lhip_decode_program_status.  All workgroups must be resident at once:
 // the grid is one workgroup per compute unit, which the register and LDS budget of the kernel guarantees.
 #include <hip/hip_fp16.h>
@@ -42,13 +46,13 @@ constexpr int kProgWaves = 8;
 constexpr int kProgThreads = kProgWaves * 64;
 constexpr int kProgSlots = 8;            // 16-byte weight loads per lane and pipeline step
 constexpr int kProgMaxK = 14336;         // activations staged in LDS as f32: 56 KiB
-constexpr unsigned kSpinLimit = 1u << 20;
-constexpr int kSyncGroups = 8;           // arrival counters
-constexpr int kSyncStride = 32;          // unsigned words between counters (128 B)
-constexpr int kSyncWords = kSyncGroups * kSyncStride + kSyncStride;  // counters, then the abort flag
+constexpr int kSyncWords = 64;           // [0] launch counter, [32] abort flag of the running launch, [48] sticky flag
+constexpr unsigned kTagsPerLaunch = 8192;  // tag = launch * kTagsPerLaunch + phase + 1; never 0
 
 enum { PHASE_MATVEC = 0, PHASE_ATTENTION = 1, PHASE_MERGE = 2 };
 enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+
+typedef unsigned long long tagged_t;  // (tag << 32) | float bits
 
 struct ProgOp {
     int type;
@@ -57,20 +61,24 @@ struct ProgOp {
     int epi, norm;
     float eps;
     int next_matvec;   // index of the next MATVEC phase, -1 if none
+    int x_phase;       // phase that produces x (its tag is expected), -1: x is there before the launch
     const int8_t *qs;
     const unsigned short *ds;
-    const float *x;    // MATVEC: activations (K);  ATTENTION: fused qkv row
-    float *y;          // MATVEC: output;  MERGE: attention output rows
+    const float *x;    // MATVEC: activations (K);  ATTENTION: fused qkv row.  Read when x_phase < 0 ...
+    const tagged_t *x_t;  // ... otherwise this shadow
+    float *y;          // MATVEC: output;  MERGE: attention output rows (written besides the shadow)
+    tagged_t *y_t;
     const float *norm_w;
-    const float *residual;
+    const float *residual;     // EPI_ADD: read when res_t is null
+    const tagged_t *res_t;     // shadow of the residual when an earlier phase of the launch wrote it
     float *k_cache, *v_cache;
 };
 
 struct AttnParams {
     int hkv, max_seq, splits;
     float theta;
-    float *ws_ml;
-    float4 *ws_acc;
+    tagged_t *ws_ml;   // shadows of the partial softmax states
+    tagged_t *ws_acc;
 };
 
 struct Buf8 {
@@ -79,8 +87,10 @@ struct Buf8 {
     float res;               // EPI_ADD: residual of the step's row (lane < r)
 };
 
-// One pipeline step of weights: slot i = slice (i / r), row (i % r); slots past r * s and dead steps aim at the
-// first bytes of the planes (one cached line), so every step issues the same number of loads.
+// One pipeline step of weights: slot i = slice (i / r), row (i % r).  Every step issues the same number of loads
+// (the wait counts the compiler derives stay exact on every path): slots past r * s, and steps past a wave's
+// last, read the first bytes of the planes with ordinary loads, which the compute unit's own cache serves once
+// one wave has fetched the line; live slots stream past that cache.
 __device__ __forceinline__ void load8(Buf8 &b, const int8_t *__restrict__ qs, const unsigned short *__restrict__ ds,
                                       int row0, int n, int k, int slice0, int r, int s, unsigned lane, bool live) {
     const int nblk = k >> 5;
@@ -88,14 +98,18 @@ __device__ __forceinline__ void load8(Buf8 &b, const int8_t *__restrict__ qs, co
     const int used = live ? r * s : 0;
 #pragma unroll
     for (int i = 0; i < kProgSlots; ++i) {
-        const bool on = i < used;
-        const int sl = r == 2 ? (i >> 1) : i, rr = r == 2 ? (i & 1) : 0;
-        const int row = on ? min(row0 + rr, n - 1) : 0;  // rows past the end re-read the last row
-        const unsigned kb = on ? static_cast<unsigned>(slice0 + sl) * 1024u : 0u;
-        const char *qrow = reinterpret_cast<const char *>(qs) + static_cast<size_t>(row) * k + kb;
-        const char *drow = reinterpret_cast<const char *>(ds) + (static_cast<size_t>(row) * nblk + (kb >> 5)) * 2;
-        b.q[i] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4 *>(qrow + (on ? qoff : 0u))));
-        b.d[i] = __builtin_nontemporal_load(as_global(reinterpret_cast<const unsigned short *>(drow + (on ? doff : 0u))));
+        if (i < used) {  // wave-uniform
+            const int sl = r == 2 ? (i >> 1) : i, rr = r == 2 ? (i & 1) : 0;
+            const int row = min(row0 + rr, n - 1);  // rows past the end re-read the last row
+            const unsigned kb = static_cast<unsigned>(slice0 + sl) * 1024u;
+            const char *qrow = reinterpret_cast<const char *>(qs) + static_cast<size_t>(row) * k + kb;
+            const char *drow = reinterpret_cast<const char *>(ds) + (static_cast<size_t>(row) * nblk + (kb >> 5)) * 2;
+            b.q[i] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4 *>(qrow + qoff)));
+            b.d[i] = __builtin_nontemporal_load(as_global(reinterpret_cast<const unsigned short *>(drow + doff)));
+        } else {
+            b.q[i] = *as_global(reinterpret_cast<const u32x4 *>(qs));
+            b.d[i] = *as_global(ds);
+        }
     }
     asm volatile("" ::"v"(qoff), "v"(doff));
 }
@@ -124,56 +138,26 @@ __device__ __forceinline__ void compute8(Buf8 &b, const float4 *xs4, int slice0,
     }
 }
 
-// Grid-wide barrier number `phase` (1, 2, ...).  `aborted` is workgroup-uniform on return.
-__device__ __forceinline__ void grid_barrier(unsigned *sync, unsigned phase, unsigned *sticky, bool &aborted,
-                                             unsigned *flag_lds) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's stores have been acknowledged
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        unsigned *abort_flag = sync + kSyncGroups * kSyncStride;
-        if (threadIdx.x == 0)
-            __hip_atomic_fetch_add(sync + (blockIdx.x % kSyncGroups) * kSyncStride, 1u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        const unsigned lane = threadIdx.x;
-        // workgroups that add to counter `lane`
-        const unsigned members = lane < kSyncGroups ? (gridDim.x - lane + kSyncGroups - 1) / kSyncGroups : 0u;
-        const unsigned want = phase * members;
-        bool stop = aborted;
-        unsigned spins = 0;
-        while (!stop) {
-            unsigned v = want;
-            if (lane < kSyncGroups)
-                v = __hip_atomic_load(sync + lane * kSyncStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            else if (lane == kSyncGroups)
-                stop = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-            if (__builtin_amdgcn_ballot_w64(v >= want) == ~0ull) break;
-            if (++spins > kSpinLimit) {
-                if (lane == 0) {
-                    __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-                stop = true;
-            }
-            stop = __builtin_amdgcn_ballot_w64(stop) != 0ull;
-        }
-        if (lane == 0) *flag_lds = stop ? 1u : 0u;
-    }
-    __syncthreads();
-    aborted = *flag_lds != 0u;
-}
-
 struct WaveCtx {
     int wave_global, total_waves;
     unsigned lane;
     int tid;
 };
 
-// Steps 0 and 1 of a wave in matvec phase `idx` (dead loads when there is no such phase or step).
-__device__ __forceinline__ void load_phase_step(Buf8 &buf, const ProgOp *__restrict__ ops, int idx, int fallback, int j,
-                                                const WaveCtx &w) {
-    const ProgOp &o = ops[idx >= 0 ? idx : fallback];
+// What a wave needs of a matvec phase to request its steps.
+struct StepGeom {
+    const int8_t *qs;
+    const unsigned short *ds;
+    int n, k, r, s, n_groups, chunks;
+};
+__device__ __forceinline__ StepGeom geom_of(const ProgOp &o) {
+    return StepGeom{o.qs, o.ds, o.n, o.k, o.r, o.s, o.n_groups, o.chunks};
+}
+
+// Steps 0 and 1 of a wave in the matvec phase described by `o` (dead loads when !valid or there is no such step).
+__device__ __forceinline__ void load_phase_step(Buf8 &buf, const StepGeom &o, bool valid, int j, const WaveCtx &w) {
     const int my_groups = w.wave_global < o.n_groups ? (o.n_groups - w.wave_global + w.total_waves - 1) / w.total_waves : 0;
-    const bool live = idx >= 0 && j < my_groups * o.chunks;
+    const bool live = valid && j < my_groups * o.chunks;
     const int g = w.wave_global + ((j == 1 && o.chunks == 1) ? w.total_waves : 0);
     const int c = (j == 1 && o.chunks > 1) ? 1 : 0;
     load8(buf, o.qs, o.ds, g * o.r, o.n, o.k, c * o.s, o.r, o.s, w.lane, live);
@@ -181,9 +165,9 @@ __device__ __forceinline__ void load_phase_step(Buf8 &buf, const ProgOp *__restr
 
 // One MATVEC phase.  On entry a / b hold this wave's steps 0 / 1 of the phase; on return its steps 0 / 1 of the
 // next MATVEC phase.
-__device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int p, Buf8 &a, Buf8 &b, float4 *xs4,
-                                             float *red, const WaveCtx &w) {
-    const ProgOp &op = ops[p];
+__device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int p, unsigned tag_base, unsigned *flags,
+                                             Buf8 &a, Buf8 &b, float4 *xs4, float *red, const WaveCtx &w) {
+    const ProgOp op = ops[p];
     const int R = op.r, S = op.s;
     const int k = op.k, chunks = op.chunks, n_groups = op.n_groups, n = op.n;
     const int epi = op.epi;
@@ -191,11 +175,20 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
     const unsigned lane = w.lane;
     const int my_groups = w.wave_global < n_groups ? (n_groups - w.wave_global + w.total_waves - 1) / w.total_waves : 0;
     const int T = my_groups * chunks;
+    TaggedIO io{tag_base + static_cast<unsigned>(op.x_phase) + 1u, tag_base + static_cast<unsigned>(p) + 1u, flags,
+                flags + 16};
+    // The next matvec phase's geometry is fetched now: by the time this phase's last steps ask for it, it is there.
+    const int nx = op.next_matvec;
+    const StepGeom nxt = geom_of(ops[nx >= 0 ? nx : p]);
 
-    // Residuals of the first two steps' rows: requested now, together with the staging loads.
+    // Residuals of the first two steps' rows: requested now, together with the staging loads.  Whoever wrote
+    // them finished before this phase's input could be complete, so their tags need no look.
     auto residual_of = [&](int g) -> float {
         const int row = min(g * R + static_cast<int>(lane < static_cast<unsigned>(R) ? lane : 0u), n - 1);
-        return ld_agent(op.residual + row);
+        if (op.res_t != nullptr)
+            return __uint_as_float(static_cast<unsigned>(
+                __hip_atomic_load(as_global(op.res_t) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+        return as_global(op.residual)[row];
     };
     if (epi == EPI_ADD) {
         a.res = residual_of(T > 0 ? w.wave_global : 0);
@@ -203,35 +196,90 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
     }
 
     // ---- activations to LDS: float4 index slice*256 + j*64 + lane holds x[slice*1024 + lane*16 + j*4 .. +3].
-    // With the norm, x * gain is staged and the sum of squares rides on the loads; the first 256 threads do it,
-    // which keeps the order of that sum the one of a four-wave workgroup.
+    // A thread fetches up to 7 float4 per round and, when they come from an earlier phase, repeats the round
+    // until every word carries that phase's tag.  With the norm, x * gain is staged and the sum of squares is
+    // taken on the way by the first 256 threads in increasing index, the order of a four-wave workgroup.
     {
+        constexpr int kBatch = 7;  // K = 14336 over 512 threads in one round
         const float4 *x4 = reinterpret_cast<const float4 *>(op.x);
+        const float4 *g4 = reinterpret_cast<const float4 *>(op.norm_w);
+        const bool tagged = op.x_phase >= 0;
         const int k4 = k >> 2;
-        if (norm) {
-            const float4 *g4 = reinterpret_cast<const float4 *>(op.norm_w);
-            float ss = 0.f;
-            if (w.tid < 256) {
-#pragma unroll 4
-                for (int i = w.tid; i < k4; i += 256) {
-                    const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
-                    float4 v = ld_agent4(x4 + src);
-                    const float4 g = ldg4(g4 + src);
-                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-                    xs4[i] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+        const int workers = norm ? 256 : kProgThreads;
+        float ss = 0.f;
+        if (w.tid < workers) {
+            for (int i0 = w.tid; i0 < k4; i0 += kBatch * workers) {
+                float4 v[kBatch];
+                if (!tagged) {
+#pragma unroll
+                    for (int u = 0; u < kBatch; ++u) {
+                        const int i = min(i0 + u * workers, k4 - 1);
+                        v[u] = ldg4(x4 + ((i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3)));
+                    }
+                } else {
+                    // A round requests every word still missing before it looks at any of them, so it costs one
+                    // memory round trip; words that have arrived are not requested again.
+                    tagged_t raw[kBatch][4];
+                    unsigned have = 0u;  // bit u: v[u] is complete
+                    bool ok;
+                    do {
+#pragma unroll
+                        for (int u = 0; u < kBatch; ++u) {
+                            if ((have >> u) & 1u) continue;
+                            const int i = min(i0 + u * workers, k4 - 1);
+                            const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
+#pragma unroll
+                            for (int c = 0; c < 4; ++c)
+                                raw[u][c] = __hip_atomic_load(as_global(op.x_t) + 4 * src + c, __ATOMIC_RELAXED,
+                                                              __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                        ok = true;
+#pragma unroll
+                        for (int u = 0; u < kBatch; ++u) {
+                            if ((have >> u) & 1u) continue;
+                            bool mine = true;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) mine = mine && static_cast<unsigned>(raw[u][c] >> 32) == io.in_tag;
+                            if (mine) {
+                                have |= 1u << u;
+                                v[u] = make_float4(__uint_as_float(static_cast<unsigned>(raw[u][0])),
+                                                   __uint_as_float(static_cast<unsigned>(raw[u][1])),
+                                                   __uint_as_float(static_cast<unsigned>(raw[u][2])),
+                                                   __uint_as_float(static_cast<unsigned>(raw[u][3])));
+                            } else {
+                                ok = false;
+                            }
+                        }
+                    } while (io.again(ok));
                 }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const int i = i0 + u * workers;
+                    if (i < k4) {
+                        if (norm) {
+                            const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
+                            const float4 g = ldg4(g4 + src);
+                            ss = fmaf(v[u].x, v[u].x, ss);
+                            ss = fmaf(v[u].y, v[u].y, ss);
+                            ss = fmaf(v[u].z, v[u].z, ss);
+                            ss = fmaf(v[u].w, v[u].w, ss);
+                            xs4[i] = make_float4(v[u].x * g.x, v[u].y * g.y, v[u].z * g.z, v[u].w * g.w);
+                        } else {
+                            xs4[i] = v[u];
+                        }
+                    }
+                }
+            }
+            if (norm) {
                 ss = wave_sum(ss);
                 if (lane == 0) red[w.tid >> 6] = ss;
-            }
-        } else {
-#pragma unroll 4
-            for (int i = w.tid; i < k4; i += kProgThreads) {
-                const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
-                xs4[i] = ld_agent4(x4 + src);
             }
         }
     }
     __syncthreads();
+    // Stores of earlier phases have been acknowledged before this phase issues its own (see the header): they
+    // were issued at least one exchange ago, and the loads this also waits for are needed now anyway.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     float scale = 1.f;
     if (norm) {
         float total = 0.f;
@@ -265,11 +313,18 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
         if (epi == EPI_SWIGLU) {  // R == 2: rows (gate, up) of one output
             const float v = sum1 * (sum0 * (1.0f / (1.0f + expf(-sum0))));
             const int pair = row0 / 2;
-            if (lane == 0 && 2 * pair + 1 < n) st_agent(op.y + pair, v);
+            if (lane == 0 && 2 * pair + 1 < n) {
+                if (op.y_t != nullptr) io.st1(reinterpret_cast<float *>(op.y_t), pair, v);
+                as_global(op.y)[pair] = v;
+            }
         } else {
             const float out = lane == 1 ? sum1 : sum0;
             const int row = row0 + static_cast<int>(lane);
-            if (lane < static_cast<unsigned>(R) && row < n) st_agent(op.y + row, epi == EPI_ADD ? out + res : out);
+            if (lane < static_cast<unsigned>(R) && row < n) {
+                const float v = epi == EPI_ADD ? out + res : out;
+                if (op.y_t != nullptr) io.st1(reinterpret_cast<float *>(op.y_t), row, v);
+                as_global(op.y)[row] = v;
+            }
         }
     };
     auto compute = [&](Buf8 &cur) {
@@ -284,10 +339,9 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
         next(g2, c2);
         __builtin_amdgcn_sched_barrier(0);
     };
-    const int nx = op.next_matvec;
     auto load_next = [&](Buf8 &cur, int j) {
         __builtin_amdgcn_sched_barrier(0);
-        load_phase_step(cur, ops, nx, p, j, w);
+        load_phase_step(cur, nxt, nx >= 0, j, w);
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -316,7 +370,7 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
 template <int G, int HD>
 union ProgShared {
     AttnShared<G, HD> attn;
-    MergeShared<G> merge;
+    MergeShared merge;
 };
 
 template <int G, int HD>
@@ -324,11 +378,10 @@ __global__ __launch_bounds__(kProgThreads) void decode_program_kernel(const Prog
                                                                       int first_matvec,
                                                                       const int *__restrict__ pos_dev,
                                                                       const AttnParams ap, unsigned *sync,
-                                                                      unsigned *sticky) {
-    // dynamic LDS: [staged activations | attention / merge scratch] (never live together), then red[4], flag
+                                                                      unsigned long long *trace) {
+    // dynamic LDS: staged activations or attention / merge scratch (never live together)
     extern __shared__ float4 lds4[];
     __shared__ float red[4];
-    __shared__ unsigned flag_lds;
     auto &sh = *reinterpret_cast<ProgShared<G, HD> *>(lds4);
 
     WaveCtx w;
@@ -337,40 +390,59 @@ __global__ __launch_bounds__(kProgThreads) void decode_program_kernel(const Prog
     w.wave_global = blockIdx.x * kProgWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     w.total_waves = gridDim.x * kProgWaves;
     const int pos = *pos_dev;
-    bool aborted = false;
+    const unsigned tag_base = sync[0] * kTagsPerLaunch;  // the launch counter was advanced by the kernel before this one
+    unsigned *flags = sync + 32;                         // [0] abort flag of this launch, [16] sticky flag
 
     Buf8 a, b;
     a.res = b.res = 0.f;
     if (first_matvec >= 0) {
-        load_phase_step(a, ops, first_matvec, first_matvec, 0, w);
-        load_phase_step(b, ops, first_matvec, first_matvec, 1, w);
+        const StepGeom first = geom_of(ops[first_matvec]);
+        load_phase_step(a, first, true, 0, w);
+        load_phase_step(b, first, true, 1, w);
     }
 
+    const bool tracing = trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0;
     for (int p = 0; p < n_ops; ++p) {
-        if (p > 0) grid_barrier(sync, static_cast<unsigned>(p), sticky, aborted, &flag_lds);
+        if (tracing) trace[2 * p] = wall_clock64();
         const ProgOp &op = ops[p];
+        // LDS changes hands: the slowest wave of the workgroup has finished the previous phase's reads of it
+        __syncthreads();
         if (op.type == PHASE_MATVEC) {
-            matvec_phase(ops, p, a, b, lds4, red, w);
-        } else if (op.type == PHASE_ATTENTION) {
-            const int items = ap.hkv * ap.splits;
-            for (int item = blockIdx.x; item < items; item += gridDim.x) {
-                attention_decode_body<G, HD, kProgThreads, true>(sh.attn, item / ap.splits, item % ap.splits, op.x,
-                                                                 op.k_cache, op.v_cache, pos, ap.hkv, ap.max_seq,
-                                                                 ap.theta, ap.splits, ap.ws_ml, ap.ws_acc);
-                __syncthreads();
-            }
+            matvec_phase(ops, p, tag_base, flags, a, b, lds4, red, w);
         } else {
-            for (int item = blockIdx.x; item < ap.hkv; item += gridDim.x) {
-                attention_merge_body<G, HD, kProgThreads, true>(sh.merge, item, op.y, pos, ap.max_seq, ap.splits,
-                                                                ap.ws_ml, ap.ws_acc);
-                __syncthreads();
+            TaggedIO io{tag_base + static_cast<unsigned>(op.x_phase) + 1u, tag_base + static_cast<unsigned>(p) + 1u, flags,
+                        flags + 16};
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // earlier phases' stores acknowledged
+            if (op.type == PHASE_ATTENTION) {
+                const int items = ap.hkv * ap.splits;
+                for (int item = blockIdx.x; item < items; item += gridDim.x) {
+                    attention_decode_body<G, HD, kProgThreads>(io, sh.attn, item / ap.splits, item % ap.splits,
+                                                               reinterpret_cast<const float *>(op.x_t), op.k_cache,
+                                                               op.v_cache, pos, ap.hkv, ap.max_seq, ap.theta, ap.splits,
+                                                               reinterpret_cast<float *>(ap.ws_ml),
+                                                               reinterpret_cast<float4 *>(ap.ws_acc));
+                    __syncthreads();
+                }
+            } else {
+                for (int item = blockIdx.x; item < ap.hkv * G; item += gridDim.x) {
+                    attention_merge_body<G, HD, kProgThreads>(io, sh.merge, item, reinterpret_cast<float *>(op.y_t), pos,
+                                                              ap.max_seq, ap.splits,
+                                                              reinterpret_cast<const float *>(ap.ws_ml),
+                                                              reinterpret_cast<const float4 *>(ap.ws_acc), op.y);
+                    __syncthreads();
+                }
             }
         }
+        if (tracing) trace[2 * p + 1] = wall_clock64();
     }
 }
 
-__global__ void decode_program_clear_kernel(unsigned *sync) {
-    for (int i = threadIdx.x; i < kSyncWords; i += blockDim.x) sync[i] = 0u;
+// Runs before the program kernel: next launch number (the tags of the previous launch become stale), abort flag off.
+__global__ void decode_program_begin_kernel(unsigned *sync) {
+    if (threadIdx.x == 0) {
+        sync[0] += 1u;
+        sync[32] = 0u;
+    }
 }
 
 struct Program {
@@ -382,8 +454,9 @@ struct Program {
     AttnParams ap{};
     const int32_t *pos = nullptr;
     ProgOp *ops_dev = nullptr;
-    unsigned *sync_dev = nullptr;  // kSyncWords, then the sticky flag
-    void *ws_dev = nullptr;
+    unsigned *sync_dev = nullptr;  // kSyncWords
+    void *shadow_dev = nullptr;    // every shadow array, one allocation
+    unsigned long long *trace_dev = nullptr;  // caller's buffer, or null
 };
 
 template <int G, int HD>
@@ -392,10 +465,10 @@ static lhip_status launch_program(const Program &pr, hipStream_t s) {
     if (pr.lds_bytes > 48 * 1024)
         LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(pr.lds_bytes)));
-    hipLaunchKernelGGL(decode_program_clear_kernel, dim3(1), dim3(256), 0, s, pr.sync_dev);
+    hipLaunchKernelGGL(decode_program_begin_kernel, dim3(1), dim3(64), 0, s, pr.sync_dev);
     LHIP_CHECK_LAUNCH();
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pr.grid)), dim3(kProgThreads), pr.lds_bytes, s, pr.ops_dev,
-                       pr.n_phases, pr.first_matvec, pr.pos, pr.ap, pr.sync_dev, pr.sync_dev + kSyncWords);
+                       pr.n_phases, pr.first_matvec, pr.pos, pr.ap, pr.sync_dev, pr.trace_dev);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
@@ -409,6 +482,14 @@ static bool prog_attention_supported(int64_t g, int64_t hd) {
     return (g == 1 || g == 2 || g == 4 || g == 8) && (hd == 64 || hd == 128);
 }
 
+// What the host knows about a caller's buffer while it lays the phases out.
+struct BufferState {
+    const void *base;
+    size_t shadow_offset;  // in words, into the shadow allocation
+    int writer;            // phase that wrote the current contents, -1: the caller
+    int last_reader;       // latest phase that reads the current contents (-1: none)
+};
+
 }  // namespace lhip
 
 using namespace lhip;
@@ -420,35 +501,92 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
                                        void **program) {
     if (!ops || !program) return LHIP_ERR_NULL_PTR;
     *program = nullptr;
-    if (n_ops <= 0 || n_ops > 4096) return LHIP_ERR_INVALID_SHAPE;
+    if (n_ops <= 0 || n_ops > 2048) return LHIP_ERR_INVALID_SHAPE;
+    if (!pos_dev) return LHIP_ERR_NULL_PTR;  // the kernel reads it in any case
     int device = 0;
     LHIP_HIP_TRY(hipGetDevice(&device));
     hipDeviceProp_t prop;
     LHIP_HIP_TRY(hipGetDeviceProperties(&prop, device));
     const int grid = prop.multiProcessorCount;
-    if (grid < kSyncGroups) return LHIP_ERR_UNSUPPORTED;
+    if (grid < 1) return LHIP_ERR_UNSUPPORTED;
     const int total_waves = grid * kProgWaves;
 
     bool has_attention = false;
     for (int i = 0; i < n_ops; ++i) has_attention |= ops[i].type == LHIP_DECODE_ATTENTION;
-    int g = 0;
+    int g = 0, splits = 0;
     if (has_attention) {
-        if (!pos_dev) return LHIP_ERR_NULL_PTR;
         if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_seq <= 0 || q_heads % kv_heads != 0 ||
             max_seq > kMaxDim || kv_heads > 65535)
             return LHIP_ERR_INVALID_SHAPE;
         if (!prog_attention_supported(q_heads / kv_heads, head_dim)) return LHIP_ERR_UNSUPPORTED;
         g = static_cast<int>(q_heads / kv_heads);
-    } else if (!pos_dev) {
-        return LHIP_ERR_NULL_PTR;  // the kernel reads it in any case
+        splits = dec_splits(kv_heads);
     }
 
+    // Buffers the operations name, by base address.  A buffer written by a phase gets a shadow array of tagged
+    // words that later phases read instead of it.
+    std::vector<BufferState> buffers;
+    size_t shadow_words = 0;
+    auto find = [&](const void *base) -> BufferState * {
+        for (auto &b : buffers)
+            if (b.base == base) return &b;
+        return nullptr;
+    };
+    // A read of `base` by phase `reader`: the phase whose tag to expect (-1: plain read) and the shadow's offset.
+    // own = the in-place residual, which the writing thread reads itself before it writes: no hazard, not noted.
+    auto note_read = [&](const void *base, int reader, bool own, size_t *offset) -> int {
+        BufferState *b = find(base);
+        if (!b) {
+            buffers.push_back(BufferState{base, SIZE_MAX, -1, own ? -1 : reader});
+            return -1;
+        }
+        if (!own && reader > b->last_reader) b->last_reader = reader;
+        *offset = b->shadow_offset;
+        return b->writer;
+    };
+    // A write of `words` values to `base` by phase `writer` whose own input comes from phase `input_phase`.
+    // A workgroup that writes has seen the whole output of `input_phase`: every workgroup has therefore begun
+    // that phase's arithmetic, i.e. has finished the reads of every phase up to it, and (a wave waits for its
+    // stores to be acknowledged before it stores for a later phase) the stores of every phase up to it have
+    // landed.  So the old contents may go if their writer and all their readers are phases <= input_phase.
+    auto note_write = [&](const void *base, size_t words, int writer, int input_phase, size_t *offset) -> bool {
+        BufferState *b = find(base);
+        if (!b) {
+            buffers.push_back(BufferState{base, SIZE_MAX, -1, -1});
+            b = &buffers.back();
+        }
+        if (b->last_reader > input_phase || b->writer > input_phase) return false;
+        if (b->shadow_offset == SIZE_MAX) {
+            b->shadow_offset = shadow_words;
+            shadow_words += (words + 31) & ~size_t{31};
+        }
+        b->writer = writer;
+        b->last_reader = -1;
+        *offset = b->shadow_offset;
+        return true;
+    };
+
+    struct Pending {  // offsets are turned into pointers once the shadow allocation exists
+        size_t x = SIZE_MAX, y = SIZE_MAX, res = SIZE_MAX;
+    };
     std::vector<ProgOp> phases;
+    std::vector<Pending> pend;
     size_t max_k = 0;
+    size_t ws_ml_off = SIZE_MAX, ws_acc_off = SIZE_MAX;
+    int ws_last_reader = -1;  // latest merge phase that reads the partial states
+    if (has_attention) {
+        ws_ml_off = shadow_words;
+        shadow_words += dec_ml_bytes(kv_heads, splits, g) / sizeof(float);
+        ws_acc_off = shadow_words;
+        shadow_words += static_cast<size_t>(kv_heads) * splits * g * static_cast<size_t>(head_dim);
+    }
     for (int i = 0; i < n_ops; ++i) {
         const lhip_decode_op &o = ops[i];
-        ProgOp p{};
-        p.next_matvec = -1;
+        const int p = static_cast<int>(phases.size());
+        ProgOp ph{};
+        Pending pe;
+        ph.next_matvec = -1;
+        ph.x_phase = -1;
         if (o.type == LHIP_DECODE_MATVEC) {
             if (!o.planar || !o.x || !o.y) return LHIP_ERR_NULL_PTR;
             if (lhip_status st = check_q8_shape(o.n, o.k)) return st;
@@ -459,42 +597,59 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
             if (!aligned(o.planar, 256) || !aligned(o.x, 16) || !aligned(o.y, 4) ||
                 (o.norm_weight && !aligned(o.norm_weight, 16)) || (o.residual && !aligned(o.residual, 4)))
                 return LHIP_ERR_MISALIGNED;
+            if (o.x == o.y) return LHIP_ERR_INVALID_SHAPE;
             const int slices = static_cast<int>(o.k / 1024);
-            p.type = PHASE_MATVEC;
-            p.s = slices % 4 == 0 ? 4 : slices % 7 == 0 ? 7 : slices % 2 == 0 ? 2 : 1;
+            ph.type = PHASE_MATVEC;
+            ph.s = slices % 4 == 0 ? 4 : slices % 7 == 0 ? 7 : slices % 2 == 0 ? 2 : 1;
             // two rows per wave where SwiGLU pairs need it, or where that still leaves every wave two row groups
-            p.r = (p.s <= 4 && (o.epilogue == LHIP_FUSE_SWIGLU || o.n / 2 >= 2 * static_cast<int64_t>(total_waves))) ? 2 : 1;
-            if (o.epilogue == LHIP_FUSE_SWIGLU && p.r != 2) return LHIP_ERR_UNSUPPORTED;
-            p.n = static_cast<int>(o.n);
-            p.k = static_cast<int>(o.k);
-            p.n_groups = (p.n + p.r - 1) / p.r;
-            p.chunks = slices / p.s;
-            p.epi = o.epilogue;
-            p.norm = o.norm_weight != nullptr;
-            p.eps = o.eps;
+            ph.r = (ph.s <= 4 && (o.epilogue == LHIP_FUSE_SWIGLU || o.n / 2 >= 2 * static_cast<int64_t>(total_waves))) ? 2 : 1;
+            if (o.epilogue == LHIP_FUSE_SWIGLU && ph.r != 2) return LHIP_ERR_UNSUPPORTED;
+            ph.n = static_cast<int>(o.n);
+            ph.k = static_cast<int>(o.k);
+            ph.n_groups = (ph.n + ph.r - 1) / ph.r;
+            ph.chunks = slices / ph.s;
+            ph.epi = o.epilogue;
+            ph.norm = o.norm_weight != nullptr;
+            ph.eps = o.eps;
             auto *base = static_cast<const uint8_t *>(o.planar);
-            p.qs = reinterpret_cast<const int8_t *>(base);
-            p.ds = reinterpret_cast<const unsigned short *>(base + q8_scale_offset(o.n, o.k));
-            p.x = o.x;
-            p.y = o.y;
-            p.norm_w = o.norm_weight;
-            p.residual = o.residual;
+            ph.qs = reinterpret_cast<const int8_t *>(base);
+            ph.ds = reinterpret_cast<const unsigned short *>(base + q8_scale_offset(o.n, o.k));
+            ph.x = o.x;
+            ph.y = o.y;
+            ph.norm_w = o.norm_weight;
+            ph.residual = o.epilogue == LHIP_FUSE_ADD ? o.residual : nullptr;
+            ph.x_phase = note_read(o.x, p, false, &pe.x);
+            if (ph.residual && note_read(ph.residual, p, ph.residual == o.y, &pe.res) < 0) pe.res = SIZE_MAX;
+            const size_t out_words = static_cast<size_t>(o.epilogue == LHIP_FUSE_SWIGLU ? o.n / 2 : o.n);
+            if (!note_write(o.y, out_words, p, ph.x_phase, &pe.y)) return LHIP_ERR_UNSUPPORTED;
             max_k = o.k > static_cast<int64_t>(max_k) ? static_cast<size_t>(o.k) : max_k;
-            phases.push_back(p);
+            phases.push_back(ph);
+            pend.push_back(pe);
         } else if (o.type == LHIP_DECODE_ATTENTION) {
             if (!o.x || !o.y || !o.k_cache || !o.v_cache) return LHIP_ERR_NULL_PTR;
             if (!aligned(o.x, 16) || !aligned(o.y, 16) || !aligned(o.k_cache, 16) || !aligned(o.v_cache, 16))
                 return LHIP_ERR_MISALIGNED;
-            p.type = PHASE_ATTENTION;
-            p.x = o.x;
-            p.k_cache = o.k_cache;
-            p.v_cache = o.v_cache;
-            phases.push_back(p);
+            if (o.x == o.y) return LHIP_ERR_INVALID_SHAPE;
+            ph.type = PHASE_ATTENTION;
+            ph.x = o.x;
+            ph.k_cache = o.k_cache;
+            ph.v_cache = o.v_cache;
+            ph.x_phase = note_read(o.x, p, false, &pe.x);
+            // the body reads its input through the tagged accessors: it must come from a phase of this program
+            if (ph.x_phase < 0) return LHIP_ERR_UNSUPPORTED;
+            if (ws_last_reader > ph.x_phase) return LHIP_ERR_UNSUPPORTED;  // the previous merge may still be reading
+            phases.push_back(ph);
+            pend.push_back(pe);
             ProgOp m{};
+            Pending pm;
             m.next_matvec = -1;
             m.type = PHASE_MERGE;
+            m.x_phase = p;  // the partial states of the attention phase
             m.y = o.y;
+            ws_last_reader = p + 1;
+            if (!note_write(o.y, static_cast<size_t>(q_heads * head_dim), p + 1, p, &pm.y)) return LHIP_ERR_UNSUPPORTED;
             phases.push_back(m);
+            pend.push_back(pm);
         } else {
             return LHIP_ERR_INVALID_SHAPE;
         }
@@ -525,29 +680,32 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
     pr->lds_bytes = max_k * 4 > scratch ? max_k * 4 : scratch;
     if (pr->lds_bytes < 16) pr->lds_bytes = 16;
 
-    lhip_status st = LHIP_OK;
     auto fail = [&](lhip_status s) {
         lhip_decode_program_destroy(pr);
         return s;
     };
+    const size_t shadow_bytes = (shadow_words ? shadow_words : 1) * sizeof(tagged_t);
     if (hipMalloc(&pr->ops_dev, phases.size() * sizeof(ProgOp)) != hipSuccess) return fail(LHIP_ERR_HIP);
-    if (hipMalloc(&pr->sync_dev, (kSyncWords + kSyncStride) * sizeof(unsigned)) != hipSuccess) return fail(LHIP_ERR_HIP);
-    if (hipMemset(pr->sync_dev, 0, (kSyncWords + kSyncStride) * sizeof(unsigned)) != hipSuccess) return fail(LHIP_ERR_HIP);
+    if (hipMalloc(&pr->sync_dev, kSyncWords * sizeof(unsigned)) != hipSuccess) return fail(LHIP_ERR_HIP);
+    if (hipMemset(pr->sync_dev, 0, kSyncWords * sizeof(unsigned)) != hipSuccess) return fail(LHIP_ERR_HIP);
+    if (hipMalloc(&pr->shadow_dev, shadow_bytes) != hipSuccess) return fail(LHIP_ERR_HIP);
+    if (hipMemset(pr->shadow_dev, 0, shadow_bytes) != hipSuccess) return fail(LHIP_ERR_HIP);  // tag 0: never valid
+    auto *shadow = static_cast<tagged_t *>(pr->shadow_dev);
+    for (size_t i = 0; i < phases.size(); ++i) {
+        if (pend[i].x != SIZE_MAX && phases[i].x_phase >= 0) phases[i].x_t = shadow + pend[i].x;
+        if (pend[i].y != SIZE_MAX) phases[i].y_t = shadow + pend[i].y;
+        if (pend[i].res != SIZE_MAX) phases[i].res_t = shadow + pend[i].res;
+    }
     if (has_attention) {
-        const int splits = dec_splits(kv_heads);
-        const size_t ml = dec_ml_bytes(kv_heads, splits, g);
-        const size_t total = ml + static_cast<size_t>(kv_heads) * splits * g * static_cast<size_t>(head_dim) * sizeof(float);
-        if (hipMalloc(&pr->ws_dev, total) != hipSuccess) return fail(LHIP_ERR_HIP);
         pr->ap.hkv = static_cast<int>(kv_heads);
         pr->ap.max_seq = static_cast<int>(max_seq);
         pr->ap.splits = splits;
         pr->ap.theta = theta;
-        pr->ap.ws_ml = static_cast<float *>(pr->ws_dev);
-        pr->ap.ws_acc = reinterpret_cast<float4 *>(static_cast<uint8_t *>(pr->ws_dev) + ml);
+        pr->ap.ws_ml = shadow + ws_ml_off;
+        pr->ap.ws_acc = shadow + ws_acc_off;
     }
     if (hipMemcpy(pr->ops_dev, phases.data(), phases.size() * sizeof(ProgOp), hipMemcpyHostToDevice) != hipSuccess)
         return fail(LHIP_ERR_HIP);
-    (void)st;
     *program = pr;
     return LHIP_OK;
 }
@@ -565,11 +723,20 @@ lhip_status lhip_decode_program_run(void *program, void *stream) {
     return LHIP_ERR_UNSUPPORTED;
 }
 
+lhip_status lhip_decode_program_trace(void *program, uint64_t *ticks_dev, int32_t *n_phases) {
+    if (!program) return LHIP_ERR_NULL_PTR;
+    auto *pr = static_cast<Program *>(program);
+    if (ticks_dev && !aligned(ticks_dev, 8)) return LHIP_ERR_MISALIGNED;
+    pr->trace_dev = reinterpret_cast<unsigned long long *>(ticks_dev);
+    if (n_phases) *n_phases = pr->n_phases;
+    return LHIP_OK;
+}
+
 lhip_status lhip_decode_program_status(void *program, int32_t *timed_out) {
     if (!program || !timed_out) return LHIP_ERR_NULL_PTR;
     const Program &pr = *static_cast<const Program *>(program);
     unsigned flag = 0;
-    LHIP_HIP_TRY(hipMemcpy(&flag, pr.sync_dev + kSyncWords, sizeof(flag), hipMemcpyDeviceToHost));
+    LHIP_HIP_TRY(hipMemcpy(&flag, pr.sync_dev + 48, sizeof(flag), hipMemcpyDeviceToHost));
     *timed_out = flag != 0;
     return LHIP_OK;
 }
@@ -579,7 +746,7 @@ lhip_status lhip_decode_program_destroy(void *program) {
     auto *pr = static_cast<Program *>(program);
     if (pr->ops_dev) (void)hipFree(pr->ops_dev);
     if (pr->sync_dev) (void)hipFree(pr->sync_dev);
-    if (pr->ws_dev) (void)hipFree(pr->ws_dev);
+    if (pr->shadow_dev) (void)hipFree(pr->shadow_dev);
     delete pr;
     return LHIP_OK;
 }

@@ -148,7 +148,11 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
             float4 v = x4[src];
             if (NORM) {
                 const float4 g = g4[src];
-                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                // spelled out, so that every kernel that takes this sum rounds it the same way
+                ss = fmaf(v.x, v.x, ss);
+                ss = fmaf(v.y, v.y, ss);
+                ss = fmaf(v.z, v.z, ss);
+                ss = fmaf(v.w, v.w, ss);
                 v = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
             }
             xs4[i] = v;

@@ -68,9 +68,10 @@ class LlamaQ8:
         # The fused matvec stages K activations in LDS in slices of 1024.
         self.fused_decode = all(k % 1024 == 0 and k <= 16384 for k in (cfg.dim, cfg.ffn))
         self._plans = None
-        # One persistent launch per decode step where the library builds it for these shapes; otherwise (and with
-        # persistent_decode = False) one launch per fused operator.
-        self.persistent_decode = True
+        # persistent_decode = True runs a decode step as one persistent launch (lhip_decode_program_*) where the
+        # library builds it for these shapes.  Same bits; measured slower on MI355X than one launch per fused operator
+        # replayed from a graph (2.9 against 2.2 ms per token at Llama-3-8B), so it is off unless asked for.
+        self.persistent_decode = False
         self._program = None
         ws = self.lib.lhip_attention_decode_workspace_nbytes(cfg.q_heads, cfg.kv_heads, cfg.head_dim)
         self._attn_ws = torch.empty(ws, dtype=torch.uint8, device=self.dev) if ws else None

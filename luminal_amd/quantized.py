@@ -265,6 +265,21 @@ class DecodeProgram:
     def run(self):
         capi.check(self.lib.lhip_decode_program_run(self._handle, _stream()), "lhip_decode_program_run")
 
+    def trace(self, on: bool = True):
+        """Switches the per-phase clock on (returns the int64 device tensor later runs fill: enter / done ticks of
+        workgroup 0 per phase, 100 MHz) or off."""
+        import ctypes as C
+
+        n = C.c_int32()
+        if not on:
+            capi.check(self.lib.lhip_decode_program_trace(self._handle, None, C.byref(n)), "lhip_decode_program_trace")
+            self._ticks = None
+            return None
+        capi.check(self.lib.lhip_decode_program_trace(self._handle, None, C.byref(n)), "lhip_decode_program_trace")
+        self._ticks = torch.zeros(2 * n.value, dtype=torch.int64, device=self._pos.device)
+        capi.check(self.lib.lhip_decode_program_trace(self._handle, self._ticks.data_ptr(), None), "lhip_decode_program_trace")
+        return self._ticks
+
     def timed_out(self) -> bool:
         import ctypes as C
 
