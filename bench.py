@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # reader can tell where it came from (they go stale when a kernel changes and the profile is not refreshed).
 TRAFFIC = {
     "gemv": (138310222, "profiles/q8_gemv_decode_projection_set.md"),
-    "gemm": (None, "profiles/q8_gemm_prefill_set.md"),
+    "gemm": (694005145, "profiles/q8_gemm_prefill_set.md"),
     "moe_t64": (2 * (158755 + 82880) * 1024, "profiles/mxfp4_moe_layer.md"),
 }
 
@@ -505,7 +505,37 @@ def llama_decode(torch):
                                     [(cfg.qkv_rows, cfg.dim), (cfg.dim, cfg.dim), (2 * cfg.ffn, cfg.dim),
                                      (cfg.dim, cfg.ffn)]) + synth_bytes(cfg.vocab, cfg.dim)
     ms = t_decode / 256 * 1e3
-    return {"tok_s": round(256 / t_decode, 1), "ms_per_token": round(ms, 3),
+    # The same steps as one persistent launch each (lhip_decode_program_*): a measured alternative, not the default.
+    alt = LlamaQ8(cfg, w, max_seq=1024)
+    alt.persistent_decode = True
+    alt.prefill(prompt, bf16=True)
+    alt_first = alt.decode(8, use_graph=True).tolist()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    alt.decode(64, use_graph=True)
+    torch.cuda.synchronize()
+    t_alt = time.perf_counter() - t0
+    program = {"tok_s": round(64 / t_alt, 1), "ms_per_token": round(t_alt / 64 * 1e3, 3), "decode_steps": 64,
+               "first_8_tokens_equal": alt_first == eager,
+               "timed_out": bool(alt._program.timed_out()) if alt._program is not None else None}
+    if alt._program is not None:
+        # where the time goes inside the one kernel: workgroup 0's clock per phase (wait for the phase's input
+        # included), averaged over 8 eager steps and over the layers
+        ticks = alt._program.trace(True)
+        acc = None
+        for _ in range(8):
+            alt.decode_step()
+            torch.cuda.synchronize()
+            t = ticks.cpu().numpy().astype(np.float64)
+            d = (t[1::2] - t[0::2]) / 100.0
+            acc = d if acc is None else acc + d
+        acc /= 8
+        names = ["qkv", "attention", "merge", "o", "gate_up", "down"]
+        program["phase_us_workgroup0"] = {nm: round(float(acc[i:6 * cfg.layers:6].mean()), 2) for i, nm in enumerate(names)}
+        program["phase_us_workgroup0"]["lm_head"] = round(float(acc[-1]), 2)
+        alt._program.trace(False)
+    del alt
+    return {"tok_s": round(256 / t_decode, 1), "ms_per_token": round(ms, 3), "persistent_program": program,
             "prefill_tokens": 512, "prefill_ms": round(t_prefill * 1e3, 2),
             "prefill_tok_s": round(512 / t_prefill, 1), "decode_steps": 256,
             "q8_0_weight_bytes_per_token": weight_bytes,
