@@ -243,6 +243,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
 }
 
 constexpr int kNumCUs = 256;
+constexpr int64_t kMaxGridRows = 65535;  // grid y
 constexpr int kMaxLdsK = 16384;  // 64 KiB of staged activations
 
 template <int R, int W, int U, typename T>
@@ -423,7 +424,7 @@ static void choose_fused(int64_t n_total, int k, int epi, int *r, int *sl, int *
 static lhip_status check_args(const void *planar, const float *x, float *y, int64_t m, int64_t n, int64_t k) {
     if (!planar || !x || !y) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_q8_shape(n, k)) return s;
-    if (m <= 0 || m > 65535) return LHIP_ERR_INVALID_SHAPE;
+    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     if (!aligned(planar, 256) || !aligned(x, 16) || !aligned(y, 4)) return LHIP_ERR_MISALIGNED;
     // Rows of x start at multiples of K floats; K % 32 == 0 keeps them 16-byte aligned.
     return LHIP_OK;
@@ -445,9 +446,16 @@ lhip_status lhip_q8_0_matmul_f32_cfg(const void *planar_dev, const float *x_dev,
                                      int waves_per_block, void *stream) {
     if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
     auto *base = static_cast<const uint8_t *>(planar_dev);
-    return dispatch(rows_per_wave, k_unroll, blocks_per_cu, waves_per_block, reinterpret_cast<const int8_t *>(base),
-                    reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_dev, y_dev, static_cast<int>(m),
-                    static_cast<int>(n), static_cast<int>(k), as_stream(stream));
+    // the activation rows are the grid's y dimension: passes of at most kMaxGridRows
+    for (int64_t m0 = 0; m0 < m; m0 += kMaxGridRows) {
+        const int mc = static_cast<int>(m - m0 < kMaxGridRows ? m - m0 : kMaxGridRows);
+        if (lhip_status st = dispatch(rows_per_wave, k_unroll, blocks_per_cu, waves_per_block,
+                                      reinterpret_cast<const int8_t *>(base),
+                                      reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_dev + m0 * k,
+                                      y_dev + m0 * n, mc, static_cast<int>(n), static_cast<int>(k), as_stream(stream)))
+            return st;
+    }
+    return LHIP_OK;
 }
 
 lhip_status lhip_q8_0_matmul_f32(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
@@ -487,7 +495,7 @@ lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, 
                                  int64_t k, void *stream) {
     if (!planar_dev || !x_f16_dev || !y_f16_dev) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_q8_shape(n, k)) return s;
-    if (m <= 0 || m > 65535) return LHIP_ERR_INVALID_SHAPE;
+    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     // Rows of x start at multiples of K halves; K % 32 == 0 keeps them 8-byte aligned.
     if (!aligned(planar_dev, 256) || !aligned(x_f16_dev, 8) || !aligned(y_f16_dev, 2)) return LHIP_ERR_MISALIGNED;
     if (m >= split_min_rows(n, k) && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_f16_dev, y_f16_dev, true))
@@ -495,10 +503,16 @@ lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, 
     auto *base = static_cast<const uint8_t *>(planar_dev);
     int r, u, b, w;
     choose(static_cast<int>(n), static_cast<int>(k), &r, &u, &b, &w);
-    return dispatch_f16(r, u, b, w, reinterpret_cast<const int8_t *>(base),
-                        reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)),
-                        static_cast<const __half *>(x_f16_dev), static_cast<__half *>(y_f16_dev), static_cast<int>(m),
-                        static_cast<int>(n), static_cast<int>(k), as_stream(stream));
+    for (int64_t m0 = 0; m0 < m; m0 += kMaxGridRows) {
+        const int mc = static_cast<int>(m - m0 < kMaxGridRows ? m - m0 : kMaxGridRows);
+        if (lhip_status st = dispatch_f16(r, u, b, w, reinterpret_cast<const int8_t *>(base),
+                                          reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)),
+                                          static_cast<const __half *>(x_f16_dev) + m0 * k,
+                                          static_cast<__half *>(y_f16_dev) + m0 * n, mc, static_cast<int>(n),
+                                          static_cast<int>(k), as_stream(stream)))
+            return st;
+    }
+    return LHIP_OK;
 }
 
 lhip_status lhip_q8_0_matmul_f32_gemm(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,

@@ -160,6 +160,28 @@ def test_matmul_rows_of_x(oracle, m):
     assert y3.shape == (1, m, 512) and np.array_equal(y3[0], y)
 
 
+def test_more_activation_rows_than_one_grid_dimension_holds():
+    """The matvec form puts the rows of x on the grid's y axis (at most 65 535): a taller x goes in several passes.
+    K = 32 keeps the call on the matvec form (the matrix-core form wants K % 512 == 0)."""
+    n, k, m = 8, 32, 70001
+    qs, d = synth.q8_0_random(n, k, seed=5)
+    w = upload(qs, d)
+    x = torch.randn(m, k, device=DEV)
+    for dt, fn in ((torch.float32, "lhip_q8_0_matmul_f32"), (torch.float16, "lhip_q8_0_matmul_f16")):
+        xs = x.to(dt)
+        y = torch.full((m, n), float("nan"), device=DEV, dtype=dt)
+        lib = capi.load_library()
+        capi.check(getattr(lib, fn)(w.planar.data_ptr(), xs.data_ptr(), y.data_ptr(), m, n, k, None), fn)
+        # every row equals the same row computed in a call of its own size class (bit for bit: one arithmetic)
+        for rows in (slice(0, 3), slice(65533, 65538), slice(m - 2, m)):
+            part = torch.empty((rows.stop - rows.start, n), device=DEV, dtype=dt)
+            capi.check(getattr(lib, fn)(w.planar.data_ptr(), xs[rows].contiguous().data_ptr(), part.data_ptr(),
+                                        rows.stop - rows.start, n, k, None), fn)
+            as_int = torch.int32 if dt == torch.float32 else torch.int16
+            assert torch.equal(y[rows].view(as_int), part.view(as_int))
+        assert not torch.isnan(y.float()).any()
+
+
 def test_reference_metal_matvec_case(oracle):
     """crates/luminal_metal/src/quantized.rs:888-935: W 512x1024 ints in 0..5,
     d = 1.0, x in U(-0.5,0.5), absolute 1e-3 against the f32 graph."""
