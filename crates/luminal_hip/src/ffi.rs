@@ -17,6 +17,12 @@ extern "C" {
     pub fn lhip_q8_0_raw_nbytes(n: i64, k: i64) -> usize;
     pub fn lhip_q8_0_planar_nbytes(n: i64, k: i64) -> usize;
     pub fn lhip_q8_0_repack(raw: *const c_void, planar: *mut c_void, n: i64, k: i64, s: Stream) -> Status;
+    // two planar (n, k) weights -> one planar (2n, k) weight, rows alternating: the (gate, up) order of the SwiGLU epilogue
+    pub fn lhip_q8_0_interleave_rows(a: *const c_void, b: *const c_void, out: *mut c_void, n: i64, k: i64, s: Stream) -> Status;
+    // batch-1 decode matvec with fusions: up to four weights on one activation row, optional RMS-norm prologue, epilogue
+    // 0 none / 1 residual add / 2 SwiGLU over (gate, up) row pairs
+    pub fn lhip_q8_0_matvec_fused_f32(w: *const *const c_void, y: *const *mut f32, n: *const i64, count: i32, x: *const f32, k: i64,
+                                      norm_weight: *const f32, eps: f32, residual: *const f32, epilogue: i32, s: Stream) -> Status;
     // with more than a few rows (a prompt) both matmuls run on the matrix cores by themselves, at f32 accuracy, streaming the
     // weights once per 64 rows instead of once per row
     pub fn lhip_q8_0_matmul_f32(w: *const c_void, x: *const f32, y: *mut f32, m: i64, n: i64, k: i64, s: Stream) -> Status;

@@ -78,6 +78,13 @@ size_t lhip_q8_0_planar_scale_offset(int64_t n, int64_t k);
 lhip_status lhip_q8_0_repack(const void *raw_dev, void *planar_dev, int64_t n, int64_t k, void *stream);
 /* planar (device) -> raw (device): inverse of lhip_q8_0_repack. */
 lhip_status lhip_q8_0_unpack(const void *planar_dev, void *raw_dev, int64_t n, int64_t k, void *stream);
+/* Two planar (n, k) weights -> one planar (2n, k) weight with their rows taken alternately (row 2j = a's row j,
+ * row 2j + 1 = b's row j): the (gate, up) row order that epilogue 2 of lhip_q8_0_matvec_fused_f32 and
+ * lhip_q8_0_matmul_bf16_swiglu read.  No counterpart in the reference, which keeps gate and up as separate tensors
+ * (examples/llama/src/model.rs:17-32); a compiler pass that fuses the two projections makes this weight once.
+ * All three buffers 256-byte aligned, out_planar_dev of lhip_q8_0_planar_nbytes(2n, k) bytes, no overlap. */
+lhip_status lhip_q8_0_interleave_rows(const void *a_planar_dev, const void *b_planar_dev, void *out_planar_dev, int64_t n,
+                                      int64_t k, void *stream);
 
 /* ---- Q8_0 operators --------------------------------------------------------
  */

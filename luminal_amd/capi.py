@@ -32,6 +32,7 @@ SIGNATURES = {
     "lhip_q8_0_planar_scale_offset": (_sz, [_i64, _i64]),
     "lhip_q8_0_repack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
     "lhip_q8_0_unpack": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
+    "lhip_q8_0_interleave_rows": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "lhip_q8_0_dequant_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f32_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),

@@ -41,6 +41,27 @@ __global__ __launch_bounds__(kThreads) void q8_unpack_kernel(const uint16_t *__r
     }
 }
 
+// Rows of two planar (n, k) weights taken alternately into one planar (2n, k) weight: row 2j = a's row j, row
+// 2j + 1 = b's row j.  Quants move as 16-byte pieces (a row is k bytes, k a multiple of 32), scales as 16-bit units.
+__global__ __launch_bounds__(kThreads) void q8_interleave_rows_kernel(const uint4 *__restrict__ qa, const uint4 *__restrict__ qb,
+                                                                       uint4 *__restrict__ qo,
+                                                                       const uint16_t *__restrict__ da,
+                                                                       const uint16_t *__restrict__ db,
+                                                                       uint16_t *__restrict__ dout, size_t n_pieces,
+                                                                       size_t n_scales, unsigned pieces_per_row,
+                                                                       unsigned scales_per_row) {
+    const size_t first = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    for (size_t c = first; c < n_pieces; c += stride) {
+        const size_t row = c / pieces_per_row, at = (row >> 1) * pieces_per_row + (c - row * pieces_per_row);
+        qo[c] = (row & 1) ? qb[at] : qa[at];
+    }
+    for (size_t c = first; c < n_scales; c += stride) {
+        const size_t row = c / scales_per_row, at = (row >> 1) * scales_per_row + (c - row * scales_per_row);
+        dout[c] = (row & 1) ? db[at] : da[at];
+    }
+}
+
 // One thread dequantises 4 consecutive quants: w = (float)q * (float)d.  The
 // product of an int8 and a binary16 value is exact in binary32.
 __device__ __forceinline__ float4 dequant4(uint32_t q4, float d) {
@@ -143,6 +164,26 @@ lhip_status lhip_q8_0_unpack(const void *planar_dev, void *raw_dev, int64_t n, i
                        reinterpret_cast<const uint16_t *>(base),
                        reinterpret_cast<const uint16_t *>(base + q8_scale_offset(n, k)),
                        static_cast<uint16_t *>(raw_dev), n_units);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
+}
+
+lhip_status lhip_q8_0_interleave_rows(const void *a_planar_dev, const void *b_planar_dev, void *out_planar_dev, int64_t n,
+                                      int64_t k, void *stream) {
+    if (!a_planar_dev || !b_planar_dev || !out_planar_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (lhip_status s = check_q8_shape(2 * n, k)) return s;
+    if (!aligned(a_planar_dev, 256) || !aligned(b_planar_dev, 256) || !aligned(out_planar_dev, 256)) return LHIP_ERR_MISALIGNED;
+    auto *a = static_cast<const uint8_t *>(a_planar_dev), *b = static_cast<const uint8_t *>(b_planar_dev);
+    auto *o = static_cast<uint8_t *>(out_planar_dev);
+    const size_t rows = static_cast<size_t>(2 * n);
+    const unsigned pieces_per_row = static_cast<unsigned>(k / 16), scales_per_row = static_cast<unsigned>(k / 32);
+    hipLaunchKernelGGL(q8_interleave_rows_kernel, dim3(grid_for(rows * pieces_per_row)), dim3(kThreads), 0, as_stream(stream),
+                       reinterpret_cast<const uint4 *>(a), reinterpret_cast<const uint4 *>(b), reinterpret_cast<uint4 *>(o),
+                       reinterpret_cast<const uint16_t *>(a + q8_scale_offset(n, k)),
+                       reinterpret_cast<const uint16_t *>(b + q8_scale_offset(n, k)),
+                       reinterpret_cast<uint16_t *>(o + q8_scale_offset(2 * n, k)), rows * pieces_per_row,
+                       rows * scales_per_row, pieces_per_row, scales_per_row);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }

@@ -32,6 +32,7 @@
 #include <cstdint>
 #include <cstring>
 #include <functional>
+#include <iterator>
 #include <map>
 #include <memory>
 #include <set>
@@ -163,6 +164,7 @@ using Input = std::pair<const Tensor *, ShapeTracker>;
 
 struct Operator {
     virtual ~Operator() = default;
+    // One tensor per output (src/op.rs:82-90 returns Vec<Tensor>); most operators have one.
     virtual std::vector<Tensor> process(const std::vector<Input> &inp) = 0;
     virtual std::string name() const = 0;
 };
@@ -373,24 +375,30 @@ struct Unary : Operator {  // any single-input host op, e.g. the contiguous copy
 
 using NodeIndex = int;
 
-struct Edge {
+struct Edge {  // Dependency::Data { input_order, output_order, shape } of src/graph.rs
     NodeIndex src, dst;
     int input_order;
     ShapeTracker shape;
+    int output_order = 0;
 };
 
 struct Graph {
     std::vector<std::unique_ptr<Operator>> nodes;  // a removed node leaves a null slot
     std::vector<Edge> edges;
     std::set<NodeIndex> to_retrieve;               // nodes whose results the caller reads as host vectors
-    std::map<NodeIndex, Tensor> results;
+    std::set<NodeIndex> no_delete;                 // nodes whose results outlive an execution (weights and what is made of them once)
+    std::map<NodeIndex, Tensor> results;           // output 0 of every executed node
+    std::map<std::pair<NodeIndex, int>, Tensor> more_results;  // outputs 1.. of the operators that have them
 
     NodeIndex add(std::unique_ptr<Operator> op) {
         nodes.push_back(std::move(op));
         return static_cast<NodeIndex>(nodes.size()) - 1;
     }
-    void connect(NodeIndex src, NodeIndex dst, int input_order, ShapeTracker shape) {
-        edges.push_back({src, dst, input_order, std::move(shape)});
+    void connect(NodeIndex src, NodeIndex dst, int input_order, ShapeTracker shape, int output_order = 0) {
+        edges.push_back({src, dst, input_order, std::move(shape), output_order});
+    }
+    const Tensor &result(NodeIndex n, int output_order = 0) const {
+        return output_order == 0 ? results.at(n) : more_results.at({n, output_order});
     }
     void remove_node(NodeIndex n) {
         nodes.at(n).reset();
@@ -410,9 +418,12 @@ struct Graph {
         std::sort(v.begin(), v.end(), [](auto a, auto b) { return a->input_order < b->input_order; });
         return v;
     }
-    // Forward execution in topological order.
+    // Forward execution in topological order.  As in src/graph.rs:199-202 a node whose result is already there is
+    // not run again; only the results of no_delete nodes are there when an execution starts.
     void execute() {
-        results.clear();
+        for (auto it = results.begin(); it != results.end();) it = no_delete.count(it->first) ? std::next(it) : results.erase(it);
+        for (auto it = more_results.begin(); it != more_results.end();)
+            it = no_delete.count(it->first.first) ? std::next(it) : more_results.erase(it);
         std::vector<int> pending(nodes.size(), 0);
         for (auto &e : edges) ++pending[e.dst];
         std::vector<NodeIndex> ready;
@@ -423,9 +434,13 @@ struct Graph {
         while (!ready.empty()) {
             const NodeIndex n = ready.back();
             ready.pop_back();
-            std::vector<Input> inp;
-            for (auto e : incoming(n)) inp.emplace_back(&results.at(e->src), e->shape);
-            results[n] = nodes[n]->process(inp).at(0);
+            if (!results.count(n)) {
+                std::vector<Input> inp;
+                for (auto e : incoming(n)) inp.emplace_back(&result(e->src, e->output_order), e->shape);
+                std::vector<Tensor> out = nodes[n]->process(inp);
+                results[n] = out.at(0);
+                for (size_t i = 1; i < out.size(); ++i) more_results[{n, static_cast<int>(i)}] = out[i];
+            }
             ++done;
             for (auto e : outgoing(n))
                 if (--pending[e->dst] == 0) ready.push_back(e->dst);

@@ -54,6 +54,20 @@ class Q8Weight:
             torch.cuda.current_stream().synchronize()  # raw_dev is released on return
         return cls(planar, n, k)
 
+    @classmethod
+    def interleave_rows(cls, a: "Q8Weight", b: "Q8Weight") -> "Q8Weight":
+        """(2n, k) weight whose rows alternate between a's and b's: the (gate, up) order the SwiGLU epilogues read
+        (gate and up are separate tensors in examples/llama/src/model.rs:17-32)."""
+        if (a.n, a.k) != (b.n, b.k):
+            raise capi.LhipError(capi.LHIP_ERR_INVALID_SHAPE, "Q8Weight.interleave_rows",
+                                 f"shapes differ: ({a.n}, {a.k}) and ({b.n}, {b.k})")
+        lib = capi.load_library()
+        out = torch.empty(cls.planar_nbytes(2 * a.n, a.k), dtype=torch.uint8, device=a.planar.device)
+        with torch.cuda.device(out.device):
+            capi.check(lib.lhip_q8_0_interleave_rows(_ptr(a.planar), _ptr(b.planar), _ptr(out), a.n, a.k, _stream()),
+                       "lhip_q8_0_interleave_rows")
+        return cls(out, 2 * a.n, a.k)
+
     def to_raw(self) -> torch.Tensor:
         lib = capi.load_library()
         raw = torch.empty(lib.lhip_q8_0_raw_nbytes(self.n, self.k), dtype=torch.uint8, device=self.planar.device)

@@ -14,6 +14,7 @@
 #include <random>
 
 #include "../../luminal_amd/host/luminal_hip.hpp"
+#include "../../luminal_amd/host/luminal_hip_fusion.hpp"
 
 using namespace luminal_hip;
 
@@ -111,6 +112,88 @@ static NodeIndex build_gather(Graph &g, NodeIndex idx, int64_t batch, NodeIndex 
 static NodeIndex build_relu(Graph &g, NodeIndex src, std::vector<int64_t> dims) {
     const NodeIndex n = g.add(std::make_unique<Unary>("Relu", [](float v) { return v > 0 ? v : 0.f; }));
     g.connect(src, n, 0, ShapeTracker(std::move(dims)));
+    return n;
+}
+
+static NodeIndex binary(Graph &g, Binary::Kind kind, NodeIndex a, ShapeTracker as, NodeIndex b, ShapeTracker bs) {
+    const NodeIndex n = g.add(std::make_unique<Binary>(kind));
+    g.connect(a, n, 0, std::move(as));
+    g.connect(b, n, 1, std::move(bs));
+    return n;
+}
+static NodeIndex unary(Graph &g, const char *label, std::function<float(float)> f, NodeIndex src, ShapeTracker s) {
+    const NodeIndex n = g.add(std::make_unique<Unary>(label, std::move(f)));
+    g.connect(src, n, 0, std::move(s));
+    return n;
+}
+static ShapeTracker expanded_scalar(const std::vector<int64_t> &dims) {
+    ShapeTracker s;
+    for (size_t i = 0; i < dims.size(); ++i) s = s.expand_dim(i, dims[i]);
+    return s;
+}
+// LayerNorm(weight, no bias, no mean_norm).forward(x) as crates/luminal_nn/src/norm.rs:56-70 puts it on the graph:
+// std_norm (src/hl_ops/unary.rs:93-104) with mean = sum / D (src/hl_ops/reduction.rs:38-45, a division by an
+// Expression: times Recip(expand(Constant(D)))), then times expand(weight).  x has dims [.., D].
+static NodeIndex build_rms_norm(Graph &g, NodeIndex x, std::vector<int64_t> dims, NodeIndex w, float eps) {
+    const size_t r = dims.size();
+    const int64_t d = dims.back();
+    const ShapeTracker full(dims);
+    std::vector<int64_t> lead(dims.begin(), dims.end() - 1);
+    const ShapeTracker red(lead), c = expanded_scalar(lead);
+    const NodeIndex sq = binary(g, Binary::Mul, x, full, x, full);
+    const NodeIndex sum = g.add(std::make_unique<SumReduce>(r - 1));
+    g.connect(sq, sum, 0, full);
+    const NodeIndex inv_d = unary(g, "Recip", [](float v) { return 1.f / v; }, g.add(std::make_unique<Constant>(static_cast<float>(d))), c);
+    const NodeIndex mean = binary(g, Binary::Mul, sum, red, inv_d, red);
+    const NodeIndex plus = binary(g, Binary::Add, mean, red, g.add(std::make_unique<Constant>(eps)), c);
+    const NodeIndex root = unary(g, "Sqrt", [](float v) { return std::sqrt(v); }, plus, red);
+    const NodeIndex factor = unary(g, "Recip", [](float v) { return 1.f / v; }, root, red);
+    const NodeIndex scaled = binary(g, Binary::Mul, factor, red.expand_dim(r - 1, d), x, full);
+    ShapeTracker ws({d});
+    for (size_t i = 0; i + 1 < r; ++i) ws = ws.expand_dim(0, dims[r - 2 - i]);
+    return binary(g, Binary::Mul, scaled, full, w, ws);
+}
+// up * gate.swish() (examples/llama/src/model.rs:27-29) in primitives: swish = gate * sigmoid(gate),
+// sigmoid(t) = 1. / (1. + (-t).exp()), exp(t) = (t * (1/ln 2)).exp2() (src/hl_ops/unary.rs:4-10,33-36,168-177), with
+// `f32 op tensor` spelled as `tensor op constant` (src/hl_ops/binary.rs:35-41,90-96,113-120).
+static NodeIndex build_swiglu(Graph &g, NodeIndex gate, NodeIndex up, std::vector<int64_t> dims) {
+    const ShapeTracker full(dims), c = expanded_scalar(dims);
+    const NodeIndex neg = binary(g, Binary::Mul, gate, full, g.add(std::make_unique<Constant>(-1.f)), c);
+    const NodeIndex scaled = binary(g, Binary::Mul, neg, full, g.add(std::make_unique<Constant>(1.f / std::log(2.f))), c);
+    const NodeIndex e = unary(g, "Exp2", [](float v) { return std::exp2(v); }, scaled, full);
+    const NodeIndex plus = binary(g, Binary::Add, e, full, g.add(std::make_unique<Constant>(1.f)), c);
+    const NodeIndex rec = unary(g, "Recip", [](float v) { return 1.f / v; }, plus, full);
+    const NodeIndex sig = binary(g, Binary::Mul, rec, full, g.add(std::make_unique<Constant>(1.f)), c);
+    const NodeIndex swish = binary(g, Binary::Mul, gate, full, sig, full);
+    return binary(g, Binary::Mul, up, full, swish, full);
+}
+
+// One decoder layer at one position the way examples/llama/src/model.rs:150-175 strings it together, with the
+// attention itself (model.rs:112-139, no weights in it) stood in for by a host operator on q; k and v are
+// retrieved like the cache rows they become.
+struct LayerNodes {
+    NodeIndex x, attn_norm, ffn_norm, wq, wk, wv, wo, wg, wu, wd, k, v, out;
+};
+static LayerNodes build_decoder_layer(Graph &g, int64_t dim, int64_t kv_dim, int64_t ffn, float eps) {
+    LayerNodes n{};
+    for (NodeIndex *f : {&n.x, &n.attn_norm, &n.ffn_norm, &n.wq, &n.wk, &n.wv, &n.wo, &n.wg, &n.wu, &n.wd}) *f = g.add(std::make_unique<Function>());
+    const std::vector<int64_t> row{1, 1, dim};
+    const NodeIndex normed = build_rms_norm(g, n.x, row, n.attn_norm, eps);
+    const NodeIndex q = build_matmul(g, normed, row, n.wq, dim);
+    n.k = build_matmul(g, normed, row, n.wk, kv_dim);
+    n.v = build_matmul(g, normed, row, n.wv, kv_dim);
+    const NodeIndex attn = unary(g, "AttentionStandIn", [](float v) { return std::tanh(v); }, q, ShapeTracker(row));
+    const NodeIndex o = build_matmul(g, attn, row, n.wo, dim);
+    const NodeIndex mid = binary(g, Binary::Add, n.x, ShapeTracker(row), o, ShapeTracker(row));  // x += y
+    const NodeIndex normed2 = build_rms_norm(g, mid, row, n.ffn_norm, eps);
+    const NodeIndex gate = build_matmul(g, normed2, row, n.wg, ffn);
+    const NodeIndex up = build_matmul(g, normed2, row, n.wu, ffn);
+    const NodeIndex act = build_swiglu(g, gate, up, {1, 1, ffn});
+    const NodeIndex down = build_matmul(g, act, {1, 1, ffn}, n.wd, dim);
+    n.out = binary(g, Binary::Add, mid, ShapeTracker(row), down, ShapeTracker(row));
+    g.to_retrieve.insert(n.k);
+    g.to_retrieve.insert(n.v);
+    g.to_retrieve.insert(n.out);
     return n;
 }
 
@@ -233,6 +316,112 @@ static void test_compiler_pass_cpu() {
     EXPECT(panic_message([&] { HipData::q8_0_from_raw(std::vector<uint8_t>(33), 1, 32); }).find("n + n/16") != std::string::npos);
 }
 
+static std::vector<FusedMatvec *> fused_nodes(Graph &g) {
+    std::vector<FusedMatvec *> v;
+    for (auto &n : g.nodes)
+        if (auto *f = dynamic_cast<FusedMatvec *>(n.get())) v.push_back(f);
+    return v;
+}
+
+static void test_fusion_pass_cpu() {
+    // a decoder layer at one position: seven projections become four fused launches
+    Graph g;
+    const LayerNodes n = build_decoder_layer(g, 1024, 256, 2048, 1e-5f);
+    HipQuantizedCompiler({n.wq, n.wk, n.wv, n.wo, n.wg, n.wu, n.wd}).compile(g, false);
+    EXPECT(count_nodes(g, "QuantizedMatmul") == 7);
+    HipFusedMatvecCompiler().compile(g);
+    EXPECT(count_nodes(g, "QuantizedMatmul") == 0 && count_nodes(g, "FusedMatvec") == 4 && count_nodes(g, "Q8InterleaveRows") == 1);
+    // both norms and the SwiGLU are gone from the host side; the two residual adds went into epilogues
+    EXPECT(count_nodes(g, "Mul") == 0 && count_nodes(g, "Add") == 0 && count_nodes(g, "Sqrt") == 0 && count_nodes(g, "Recip") == 0 &&
+           count_nodes(g, "Exp2") == 0 && count_nodes(g, "SumReduce(2)") == 0);
+    EXPECT(count_nodes(g, "AttentionStandIn") == 1);
+    int qkv = 0, o = 0, gate_up = 0, down = 0;
+    for (FusedMatvec *f : fused_nodes(g)) {
+        if (f->n == std::vector<int64_t>{1024, 256, 256} && f->k == 1024 && f->norm && f->epilogue == FusedMatvec::None && f->eps == 1e-5f) ++qkv;
+        if (f->n == std::vector<int64_t>{1024} && f->k == 1024 && !f->norm && f->epilogue == FusedMatvec::Residual) ++o;
+        if (f->n == std::vector<int64_t>{4096} && f->k == 1024 && f->norm && f->epilogue == FusedMatvec::SwiGLU) ++gate_up;
+        if (f->n == std::vector<int64_t>{1024} && f->k == 2048 && !f->norm && f->epilogue == FusedMatvec::Residual) ++down;
+    }
+    EXPECT(qkv == 1 && o == 1 && gate_up == 1 && down == 1);
+    // host <-> device crossings left: x up (once, shared), the two norm weights up (kept), the stand-in's input
+    // down and its result up, k, v and the layer output down
+    EXPECT(count_nodes(g, "HipCopyToDevice") == 4 && count_nodes(g, "HipCopyFromDevice") == 4);
+    EXPECT(g.no_delete.size() == 3);  // two norm weights on the device, the interleaved gate|up weight
+    EXPECT(g.to_retrieve.size() == 3);
+    for (NodeIndex r : g.to_retrieve) EXPECT(g.nodes[r] && g.nodes[r]->name() == "HipCopyFromDevice");
+    // o -> (residual) -> gate|up -> down never leave the device: the gate|up launch reads the o launch's output, the
+    // down launch reads gate|up's output and o's output (its residual)
+    for (NodeIndex i = 0; i < static_cast<NodeIndex>(g.nodes.size()); ++i) {
+        auto *f = dynamic_cast<FusedMatvec *>(g.nodes[i].get());
+        if (!f || f->epilogue == FusedMatvec::None) continue;
+        auto in = g.incoming(i);
+        if (f->epilogue == FusedMatvec::SwiGLU) EXPECT(g.nodes[in.at(0)->src]->name() == "FusedMatvec" && g.nodes[in.at(1)->src]->name() == "Q8InterleaveRows");
+        if (f->k == 2048) EXPECT(g.nodes[in.at(0)->src]->name() == "FusedMatvec" && g.nodes[in.at(2)->src]->name() == "FusedMatvec");
+    }
+
+    // patterns that must NOT fuse: a norm whose result something else reads too; a projection of several rows; K not
+    // a multiple of 1024; a gate whose swish is read elsewhere too
+    {
+        Graph h;
+        auto x = h.add(std::make_unique<Function>()), nw = h.add(std::make_unique<Function>()), w = h.add(std::make_unique<Function>());
+        const NodeIndex normed = build_rms_norm(h, x, {1, 1, 1024}, nw, 1e-5f);
+        const NodeIndex y = build_matmul(h, normed, {1, 1, 1024}, w, 64);
+        const NodeIndex side = build_relu(h, normed, {1, 1, 1024});
+        h.to_retrieve.insert(y);
+        h.to_retrieve.insert(side);
+        HipQuantizedCompiler({w}).compile(h, false);
+        HipFusedMatvecCompiler().compile(h);
+        EXPECT(count_nodes(h, "FusedMatvec") == 0 && count_nodes(h, "QuantizedMatmul") == 1 && count_nodes(h, "Sqrt") == 1);
+    }
+    {
+        Graph h;
+        auto x = h.add(std::make_unique<Function>()), wa = h.add(std::make_unique<Function>()), wb = h.add(std::make_unique<Function>());
+        h.to_retrieve.insert(build_matmul(h, x, {1, 4, 1024}, wa, 64));  // four rows
+        h.to_retrieve.insert(build_matmul(h, x, {1, 4, 1024}, wb, 64));
+        auto x2 = h.add(std::make_unique<Function>()), wc = h.add(std::make_unique<Function>()), wd = h.add(std::make_unique<Function>());
+        h.to_retrieve.insert(build_matmul(h, x2, {1, 1, 512}, wc, 64));  // K = 512
+        h.to_retrieve.insert(build_matmul(h, x2, {1, 1, 512}, wd, 64));
+        HipQuantizedCompiler({wa, wb, wc, wd}).compile(h, false);
+        HipFusedMatvecCompiler().compile(h);
+        EXPECT(count_nodes(h, "FusedMatvec") == 0 && count_nodes(h, "QuantizedMatmul") == 4);
+    }
+    {
+        // siblings without norm or epilogue still share one launch and one upload of x; five siblings make 4 + 1
+        Graph h;
+        auto x = h.add(std::make_unique<Function>());
+        std::vector<NodeIndex> ws;
+        for (int i = 0; i < 5; ++i) {
+            ws.push_back(h.add(std::make_unique<Function>()));
+            h.to_retrieve.insert(build_matmul(h, x, {1, 1, 2048}, ws.back(), 32 * (i + 1)));
+        }
+        HipQuantizedCompiler(ws).compile(h, false);
+        HipFusedMatvecCompiler().compile(h);
+        EXPECT(count_nodes(h, "FusedMatvec") == 1 && count_nodes(h, "QuantizedMatmul") == 1);
+        for (FusedMatvec *f : fused_nodes(h)) EXPECT((f->n == std::vector<int64_t>{32, 64, 96, 128}) && !f->norm && f->epilogue == FusedMatvec::None);
+        EXPECT(h.to_retrieve.size() == 5);
+    }
+    {
+        // the swish of the gate is read by a second consumer: gate and up still share a launch, the SwiGLU stays on the host
+        Graph h;
+        auto x = h.add(std::make_unique<Function>()), wg = h.add(std::make_unique<Function>()), wu = h.add(std::make_unique<Function>());
+        const NodeIndex gate = build_matmul(h, x, {1, 1, 1024}, wg, 64), up = build_matmul(h, x, {1, 1, 1024}, wu, 64);
+        const NodeIndex act = build_swiglu(h, gate, up, {1, 1, 64});
+        h.to_retrieve.insert(act);
+        const NodeIndex swish = h.incoming(act).at(1)->src;
+        h.to_retrieve.insert(build_relu(h, swish, {1, 1, 64}));
+        HipQuantizedCompiler({wg, wu}).compile(h, false);
+        HipFusedMatvecCompiler().compile(h);
+        EXPECT(count_nodes(h, "FusedMatvec") == 1 && count_nodes(h, "Exp2") == 1 && count_nodes(h, "Q8InterleaveRows") == 0);
+        for (FusedMatvec *f : fused_nodes(h)) EXPECT(f->epilogue == FusedMatvec::None && f->n.size() == 2);
+    }
+    // operator-level checks without a device
+    FusedMatvec op({64}, 1024, false, 0.f, FusedMatvec::None);
+    Tensor dummy;
+    EXPECT(panic_message([&] { op.process({{&dummy, ShapeTracker({1024})}}); }).find("wrong number of inputs") != std::string::npos);
+    EXPECT(panic_message([&] { op.process({{&dummy, ShapeTracker({2, 1024})}, {&dummy, ShapeTracker({64, 1024}).permute({1, 0})}}); })
+               .find("one contiguous row") != std::string::npos);
+}
+
 // ---------------------------------------------------------------- device
 struct Q8 {
     std::vector<int8_t> q;
@@ -350,6 +539,110 @@ static void test_graph_end_to_end(DType dtype) {
     }
 }
 
+// The retrieved node that holds the projection by `weight` (a host copy behind a QuantizedMatmul or behind one output
+// of a FusedMatvec); -1 if there is none.
+static NodeIndex retrieved_projection(const Graph &g, NodeIndex weight) {
+    for (NodeIndex r : g.to_retrieve) {
+        if (!g.nodes[r] || g.nodes[r]->name() != "HipCopyFromDevice") continue;
+        const Edge *e = g.incoming(r).at(0);
+        const std::string producer = g.nodes[e->src]->name();
+        if (producer == "QuantizedMatmul" && g.incoming(e->src).at(1)->src == weight) return r;
+        if (producer == "FusedMatvec" && g.incoming(e->src).at(1 + e->output_order)->src == weight) return r;
+    }
+    return -1;
+}
+
+static void test_fused_decoder_layer() {
+    // The decoder layer of test_fusion_pass_cpu with real Q8_0 weights: host primitives on the dequantised weights,
+    // the device graph operator by operator, and the fused graph, twice with different activations (what is kept
+    // between executions - the interleaved gate|up weight, the norm weights on the device - is made once).
+    std::mt19937 rng(7);
+    const int dim = 1024, kv = 256, ffn = 2048;
+    const float eps = 1e-5f;
+    const Q8 wq = random_q8(rng, dim, dim, 1e-3f), wk = random_q8(rng, kv, dim, 1e-3f), wv = random_q8(rng, kv, dim, 1e-3f),
+             wo = random_q8(rng, dim, dim, 1e-3f), wg = random_q8(rng, ffn, dim, 1e-3f), wu = random_q8(rng, ffn, dim, 1e-3f),
+             wd = random_q8(rng, dim, ffn, 1e-3f);
+    std::normal_distribution<float> gauss(0.f, 1.f);
+    std::vector<float> norm1(dim), norm2(dim);
+    for (auto &v : norm1) v = 1.f + 0.1f * gauss(rng);
+    for (auto &v : norm2) v = 1.f + 0.1f * gauss(rng);
+    auto activations = [&] {
+        std::vector<float> x(dim);
+        for (auto &v : x) v = gauss(rng);
+        return x;
+    };
+    Graph host, plain, fused;
+    const LayerNodes hn = build_decoder_layer(host, dim, kv, ffn, eps);
+    struct Weight { NodeIndex node; const Q8 *w; int64_t n, k; };
+    const std::vector<Weight> weights{{hn.wq, &wq, dim, dim}, {hn.wk, &wk, kv, dim}, {hn.wv, &wv, kv, dim}, {hn.wo, &wo, dim, dim},
+                                      {hn.wg, &wg, ffn, dim}, {hn.wu, &wu, ffn, dim}, {hn.wd, &wd, dim, ffn}};
+    for (const Weight &w : weights) fn(host, w.node)->value = host_tensor(w.w->dense);
+    auto prepare_device = [&](Graph &g, bool fuse) {
+        const LayerNodes n = build_decoder_layer(g, dim, kv, ffn, eps);
+        EXPECT(n.wd == hn.wd && n.out == hn.out);  // same construction order, same node numbers
+        std::map<NodeIndex, GgufTensor> tensors;
+        for (const Weight &w : weights) tensors[w.node] = GgufTensor{true, w.n, w.k, &w.w->raw};
+        HipQuantizedCompiler(q8_load_hip(g, tensors)).compile(g);
+        if (fuse) HipFusedMatvecCompiler().compile(g);
+    };
+    prepare_device(plain, false);
+    prepare_device(fused, true);
+    EXPECT(count_nodes(plain, "QuantizedMatmul") == 7 && count_nodes(fused, "FusedMatvec") == 4 && count_nodes(fused, "QuantizedMatmul") == 0);
+    for (Graph *g : {&host, &plain, &fused}) {
+        fn(*g, hn.attn_norm)->value = host_tensor(norm1);
+        fn(*g, hn.ffn_norm)->value = host_tensor(norm2);
+    }
+    const Tensor *kept_weight = nullptr;
+    const void *first_buffer = nullptr;
+    for (int round = 0; round < 2; ++round) {
+        const std::vector<float> x = activations();
+        for (Graph *g : {&host, &plain, &fused}) {
+            fn(*g, hn.x)->value = host_tensor(x);
+            g->execute();
+        }
+        struct Out { const char *what; NodeIndex host_node, weight; };
+        for (const Out &o : {Out{"k", hn.k, hn.wk}, Out{"v", hn.v, hn.wv}, Out{"out", hn.out, -1}}) {
+            const std::vector<float> want = host_operand(host.results.at(o.host_node), o.what);
+            auto device_result = [&](Graph &g) {
+                NodeIndex r = o.weight >= 0 ? retrieved_projection(g, o.weight) : -1;
+                if (o.weight < 0)  // the layer output: the retrieved node that is neither k nor v
+                    for (NodeIndex c : g.to_retrieve)
+                        if (c != retrieved_projection(g, hn.wk) && c != retrieved_projection(g, hn.wv)) r = c;
+                return host_operand(g.results.at(r), o.what);
+            };
+            const std::vector<float> got_plain = device_result(plain), got_fused = device_result(fused);
+            EXPECT(got_plain.size() == want.size() && got_fused.size() == want.size());
+            // operators' bar against the dequantised-weight host graph; fused against unfused differs only by f32
+            // summation order (norm, dot products) and the exponential's last bits
+            EXPECT(max_abs_diff(got_plain, want) < 2e-3 * rms(want));
+            EXPECT(max_abs_diff(got_fused, want) < 2e-3 * rms(want));
+            EXPECT(max_abs_diff(got_fused, got_plain) < 1e-4 * rms(want));
+        }
+        for (NodeIndex n = 0; n < static_cast<NodeIndex>(fused.nodes.size()); ++n)
+            if (fused.nodes[n] && fused.nodes[n]->name() == "Q8InterleaveRows") {
+                const Tensor *now = &fused.results.at(n);
+                const void *buffer = device_operand(*now, "gate|up").ptr();
+                if (round == 0) first_buffer = buffer;
+                else EXPECT(buffer == first_buffer);  // not made again
+                kept_weight = now;
+            }
+    }
+    EXPECT(kept_weight != nullptr);
+    // the interleaved weight row by row: unpack it and compare with the two sources' raw blocks
+    {
+        const HipData &both = device_operand(*kept_weight, "gate|up");
+        HipData raw(lhip_q8_0_raw_nbytes(2 * ffn, dim));
+        check(lhip_q8_0_unpack(both.ptr(), raw.ptr(), 2 * ffn, dim, nullptr), "lhip_q8_0_unpack");
+        std::vector<uint8_t> bytes(raw.bytes());
+        check(lhip_memcpy_d2h(bytes.data(), raw.ptr(), bytes.size(), nullptr), "lhip_memcpy_d2h");
+        const size_t row = static_cast<size_t>(dim) / 32 * 34;
+        bool same = true;
+        for (int j = 0; j < ffn && same; ++j)
+            same = std::memcmp(&bytes[(2 * j) * row], &wg.raw[j * row], row) == 0 && std::memcmp(&bytes[(2 * j + 1) * row], &wu.raw[j * row], row) == 0;
+        EXPECT(same);
+    }
+}
+
 static void test_device_errors_surface_as_panics() {
     // K = 40 is not a multiple of 32: the status of the C ABI becomes a Panic carrying its name
     std::mt19937 rng(4);
@@ -376,11 +669,13 @@ int main(int argc, char **argv) {
     try {
         test_primitives_on_the_host();
         test_compiler_pass_cpu();
+        test_fusion_pass_cpu();
         if (mode == "gpu") {
             check(lhip_init(0), "lhip_init");
             test_quantized_matvec_like_the_reference();
             test_graph_end_to_end(DType::F32);
             test_graph_end_to_end(DType::F16);
+            test_fused_decoder_layer();
             test_device_errors_surface_as_panics();
         }
     } catch (const std::exception &e) {

@@ -55,6 +55,35 @@ def test_planar_form_depends_on_the_block_count_only(n, k):
     assert np.array_equal(by_shape, by_count)
 
 
+@pytest.mark.parametrize("n,k", [(1, 32), (5, 96), (129, 1056), (2048, 1024)])
+def test_interleaved_rows_are_the_sources_rows_bit_for_bit(n, k):
+    qa, da = synth.q8_0_random(n, k, seed=3 * n + k)
+    qb, db = synth.q8_0_random(n, k, seed=5 * n + k)
+    both = Q8Weight.interleave_rows(upload(qa, da), upload(qb, db))
+    assert (both.n, both.k) == (2 * n, k)
+    qs = np.empty((2 * n, k), dtype=np.int8)
+    d = np.empty((2 * n, k // 32), dtype=np.float16)
+    qs[0::2], qs[1::2], d[0::2], d[1::2] = qa, qb, da, db
+    planar = both.planar.cpu().numpy()
+    off = capi.load_library().lhip_q8_0_planar_scale_offset(2 * n, k)
+    assert np.array_equal(planar[:2 * n * k].view(np.int8).reshape(2 * n, k), qs)  # the padding behind it is not written
+    assert np.array_equal(planar[off:].view(np.float16).reshape(2 * n, k // 32), d)
+    assert np.array_equal(both.to_raw().cpu().numpy(), synth.q8_0_raw_blocks(qs, d))
+
+
+def test_interleave_rows_rejects_bad_arguments():
+    lib = capi.load_library()
+    a = upload(*synth.q8_0_random(4, 64, seed=1))
+    out = torch.empty(Q8Weight.planar_nbytes(8, 64) + 256, dtype=torch.uint8, device=DEV)
+    p = a.planar.data_ptr()
+    assert lib.lhip_q8_0_interleave_rows(None, p, out.data_ptr(), 4, 64, None) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_interleave_rows(p, p, out.data_ptr() + 16, 4, 64, None) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_interleave_rows(p, p, out.data_ptr(), 4, 48, None) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_interleave_rows(p, p, out.data_ptr(), 0, 64, None) == capi.LHIP_ERR_INVALID_SHAPE
+    with pytest.raises(capi.LhipError):
+        Q8Weight.interleave_rows(a, upload(*synth.q8_0_random(4, 96, seed=2)))
+
+
 def test_dequant_bit_exact_every_quant_times_every_scale(oracle):
     # all 256 int8 values x all 65536 f16 codes (NaN codes compared as NaN)
     n, k = 65536, 256
