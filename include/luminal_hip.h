@@ -235,6 +235,21 @@ lhip_status lhip_q8_0_matmul_f16(const void *planar_dev, const void *x_f16_dev, 
 lhip_status lhip_q8_0_gather_f16(const void *planar_dev, const float *idx_dev, void *out_f16_dev, int64_t n_idx,
                                  int64_t n, int64_t k, void *stream);
 
+/* Re-entrant forms of lhip_q8_0_matmul_f32 / _f16.  With several activation rows those operators may cut K into
+ * slices whose partial sums meet in a scratch array the library keeps per device, so two of their calls that overlap
+ * in time on one device (different streams) race; the reference's operators (quantized.rs:116-149) have no such
+ * constraint.  These forms keep the partial sums in the caller's workspace instead and touch no shared state:
+ *   workspace_dev of lhip_q8_0_matmul_workspace_nbytes(m, n, k) bytes (256-byte aligned; 0 bytes: none is needed,
+ *   NULL is fine) gives the plan, and the bits, of the plain call;
+ *   a smaller one, or NULL, means fewer or no K slices: same accuracy, last bits may differ, and a short-and-small
+ *   product (few rows, few weight rows) leaves compute units idle.
+ * Calls sharing a workspace must be ordered on one stream.  Other arguments and errors as the plain forms. */
+size_t lhip_q8_0_matmul_workspace_nbytes(int64_t m, int64_t n, int64_t k);
+lhip_status lhip_q8_0_matmul_f32_ws(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
+                                    int64_t k, void *workspace_dev, size_t workspace_nbytes, void *stream);
+lhip_status lhip_q8_0_matmul_f16_ws(const void *planar_dev, const void *x_f16_dev, void *y_f16_dev, int64_t m, int64_t n,
+                                    int64_t k, void *workspace_dev, size_t workspace_nbytes, void *stream);
+
 /* ---- MXFP4 weights and the mixture-of-experts layer -------------------------
  * No counterpart in the reference (it has no MXFP4 and no MoE op); built to its
  * conventions: exact dequantisation, then f32-accumulated matmul

@@ -52,6 +52,9 @@ SIGNATURES = {
     "lhip_q8_0_matmul_bf16_cfg": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "lhip_q8_0_gather_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "lhip_q8_0_matmul_workspace_nbytes": (_sz, [_i64, _i64, _i64]),
+    "lhip_q8_0_matmul_f32_ws": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "lhip_q8_0_matmul_f16_ws": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "lhip_q8_0_matmul_f32_gemm": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_matmul_f16_gemm": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_q8_0_gather_f16": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

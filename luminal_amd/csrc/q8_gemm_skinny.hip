@@ -27,6 +27,8 @@
 #include <type_traits>
 #include <utility>
 
+#include <algorithm>
+
 #include "common.h"
 
 namespace lhip {
@@ -520,23 +522,44 @@ bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16
 // weights once, as blockIdx.z of one launch; K is sliced only while strips x passes leave the chip unfilled.  At most
 // kSkMaxPasses passes per launch (the grid's z extent).  `splits` = 0: chosen here.  The caller has checked
 // q8_gemm_split_supports.
+constexpr int64_t kSkMaxPasses = 1024;
+
+// K slices of one chunk of mc rows: as many as fill the chip, within `room` floats of partial planes.
+static int split_slices(int mc, int n, int k, int splits_arg, size_t room) {
+    const int units = k / kSkUnit, strips = (n + kSkRows - 1) / kSkRows, passes = (mc + 63) / 64;
+    int splits = splits_arg > 0 ? splits_arg : 256 / (strips * passes);
+    if (splits < 1) splits = 1;
+    if (splits > units) splits = units;
+    while (splits > 1 && static_cast<size_t>(splits) * mc * n > room) --splits;
+    const int per = (units + splits - 1) / splits;
+    return (units + per - 1) / per;  // no empty slice
+}
+
+// Floats of partial planes the plan of q8_gemm_split_launch uses for (m, n, k) when it has the library's own
+// scratch array to itself: what a caller's workspace must hold for the same plan (and the same bits).
+size_t q8_gemm_split_workspace_floats(int64_t m, int n, int k) {
+    size_t most = 0;
+    for (int64_t m0 = 0; m0 < m; m0 += 64 * kSkMaxPasses) {
+        const int mc = static_cast<int>(m - m0 < 64 * kSkMaxPasses ? m - m0 : 64 * kSkMaxPasses);
+        const int splits = split_slices(mc, n, k, 0, kSkScratchFloats);
+        if (splits > 1) most = std::max(most, static_cast<size_t>(splits) * mc * n);
+    }
+    return most;
+}
+
+// `own_workspace`: partial planes go to `ws` (ws_floats floats; none: no K slices) and the library's scratch array
+// is not touched, so calls may overlap in time.
 lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void *x, void *y, int64_t m, int n, int k,
-                                 bool f16, int splits_arg, hipStream_t s) {
-    constexpr int64_t kSkMaxPasses = 1024;
-    const int units = k / kSkUnit, strips = (n + kSkRows - 1) / kSkRows;
+                                 bool f16, int splits_arg, hipStream_t s, bool own_workspace, float *ws, size_t ws_floats) {
     const size_t esz = f16 ? 2 : 4;
     for (int64_t m0 = 0; m0 < m; m0 += 64 * kSkMaxPasses) {
         const int mc = static_cast<int>(m - m0 < 64 * kSkMaxPasses ? m - m0 : 64 * kSkMaxPasses);
         const int passes = (mc + 63) / 64;
-        int splits = splits_arg > 0 ? splits_arg : 256 / (strips * passes);
-        if (splits < 1) splits = 1;
-        if (splits > units) splits = units;
-        while (splits > 1 && static_cast<size_t>(splits) * mc * n > kSkScratchFloats) --splits;
-        const int per = (units + splits - 1) / splits;
-        splits = (units + per - 1) / per;  // no empty slice
+        const size_t room = own_workspace ? (ws ? std::min(ws_floats, kSkScratchFloats) : 0) : kSkScratchFloats;
+        const int splits = split_slices(mc, n, k, splits_arg, room);
         float *part = nullptr;
         if (splits > 1) {
-            part = sk_scratch_ptr();
+            part = own_workspace ? ws : sk_scratch_ptr();
             if (!part) return LHIP_ERR_HIP;
         }
         const auto *xc = static_cast<const unsigned char *>(x) + static_cast<size_t>(m0) * k * esz;

@@ -28,7 +28,9 @@ namespace lhip {
 // q8_gemm_skinny.hip: the matrix-core form with f32-accurate (head + tail bf16) operands for several activation rows.
 bool q8_gemm_split_supports(int n, int k, const void *x, const void *y, bool f16);
 lhip_status q8_gemm_split_launch(const int8_t *qs, const __half *ds, const void *x, void *y, int64_t m, int n, int k,
-                                 bool f16, int splits, hipStream_t s);
+                                 bool f16, int splits, hipStream_t s, bool own_workspace = false, float *ws = nullptr,
+                                 size_t ws_floats = 0);
+size_t q8_gemm_split_workspace_floats(int64_t m, int n, int k);
 // From this many activation rows on the plain operators take that form where the shape allows it: the weights are
 // then streamed once per 64 rows instead of once per row.  The matrix-core form has a fixed cost (its launch, a
 // reduce launch where K is sliced, staging) that a matvec pass over a small matrix stays under.  Measured, matvec
@@ -537,6 +539,43 @@ lhip_status lhip_q8_0_matmul_f16_gemm(const void *planar_dev, const void *x_f16_
     return q8_gemm_split_launch(reinterpret_cast<const int8_t *>(base),
                                 reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_f16_dev, y_f16_dev, m,
                                 static_cast<int>(n), static_cast<int>(k), true, 0, as_stream(stream));
+}
+
+size_t lhip_q8_0_matmul_workspace_nbytes(int64_t m, int64_t n, int64_t k) {
+    if (check_q8_shape(n, k) != LHIP_OK || m <= 0 || m > kMaxDim) return 0;
+    if (m < split_min_rows(n, k) || k % 512 != 0 || n % 4 != 0) return 0;  // the matvec kernels keep nothing outside their outputs
+    return q8_gemm_split_workspace_floats(m, static_cast<int>(n), static_cast<int>(k)) * sizeof(float);
+}
+
+lhip_status lhip_q8_0_matmul_f32_ws(const void *planar_dev, const float *x_dev, float *y_dev, int64_t m, int64_t n,
+                                    int64_t k, void *workspace_dev, size_t workspace_nbytes, void *stream) {
+    if (lhip_status s = check_args(planar_dev, x_dev, y_dev, m, n, k)) return s;
+    if (workspace_dev && !aligned(workspace_dev, 256)) return LHIP_ERR_MISALIGNED;
+    if (m >= split_min_rows(n, k) && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_dev, y_dev, false)) {
+        auto *base = static_cast<const uint8_t *>(planar_dev);
+        return q8_gemm_split_launch(reinterpret_cast<const int8_t *>(base),
+                                    reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_dev, y_dev, m,
+                                    static_cast<int>(n), static_cast<int>(k), false, 0, as_stream(stream), true,
+                                    static_cast<float *>(workspace_dev), workspace_dev ? workspace_nbytes / sizeof(float) : 0);
+    }
+    return lhip_q8_0_matmul_f32(planar_dev, x_dev, y_dev, m, n, k, stream);  // matvec kernels: no shared state
+}
+
+lhip_status lhip_q8_0_matmul_f16_ws(const void *planar_dev, const void *x_f16_dev, void *y_f16_dev, int64_t m, int64_t n,
+                                    int64_t k, void *workspace_dev, size_t workspace_nbytes, void *stream) {
+    if (!planar_dev || !x_f16_dev || !y_f16_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status s = check_q8_shape(n, k)) return s;
+    if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
+    if (!aligned(planar_dev, 256) || !aligned(x_f16_dev, 8) || !aligned(y_f16_dev, 2)) return LHIP_ERR_MISALIGNED;
+    if (workspace_dev && !aligned(workspace_dev, 256)) return LHIP_ERR_MISALIGNED;
+    if (m >= split_min_rows(n, k) && q8_gemm_split_supports(static_cast<int>(n), static_cast<int>(k), x_f16_dev, y_f16_dev, true)) {
+        auto *base = static_cast<const uint8_t *>(planar_dev);
+        return q8_gemm_split_launch(reinterpret_cast<const int8_t *>(base),
+                                    reinterpret_cast<const __half *>(base + q8_scale_offset(n, k)), x_f16_dev, y_f16_dev, m,
+                                    static_cast<int>(n), static_cast<int>(k), true, 0, as_stream(stream), true,
+                                    static_cast<float *>(workspace_dev), workspace_dev ? workspace_nbytes / sizeof(float) : 0);
+    }
+    return lhip_q8_0_matmul_f16(planar_dev, x_f16_dev, y_f16_dev, m, n, k, stream);
 }
 
 lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float *const *y_dev, const int64_t *n,

@@ -178,3 +178,72 @@ def test_rows_gemm_argument_errors():
     assert f16(w.planar.data_ptr(), xh.data_ptr() + 8, yh.data_ptr(), 7, 64, 512, s) == capi.LHIP_ERR_UNSUPPORTED
     assert f16(w.planar.data_ptr(), xh.data_ptr() + 2, yh.data_ptr(), 7, 64, 512, s) == capi.LHIP_ERR_MISALIGNED
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("m,n,k", [(4, 4096, 4096), (6, 1024, 1024), (16, 1024, 4096), (64, 2048, 2048), (200, 512, 1536)])
+def test_workspace_forms_give_the_plain_calls_bits_and_overlap_safely(oracle, m, n, k):
+    """lhip_q8_0_matmul_f32_ws / _f16_ws keep K-slice partial sums in the caller's workspace: with the recommended
+    size the plan and the bits are those of the plain call; without a workspace K is not sliced (operator's bar
+    still holds); two streams with workspaces of their own run interleaved and each gets its own result."""
+    lib = capi.load_library()
+    qs, d = synth.q8_0_random(n, k, seed=7 * m + n + k)
+    w = upload(qs, d)
+    wf = oracle.q8_0_dequant(synth.q8_0_raw_blocks(qs, d), qs.size).reshape(qs.shape)
+    xs = [torch.from_numpy(synth.activations(m, k, seed=s)).to(DEV) for s in (1, 2)]
+    nbytes = lib.lhip_q8_0_matmul_workspace_nbytes(m, n, k)
+    assert nbytes % 4 == 0 and nbytes <= 32 << 20
+    plain = []
+    for x in xs:
+        y = torch.empty((m, n), device=DEV)
+        capi.check(lib.lhip_q8_0_matmul_f32(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, stream()), "plain")
+        plain.append(y)
+    torch.cuda.synchronize()
+    spaces = [torch.empty(max(nbytes, 256), dtype=torch.uint8, device=DEV) for _ in xs]
+    y_ws = torch.empty((m, n), device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_f32_ws(w.planar.data_ptr(), xs[0].data_ptr(), y_ws.data_ptr(), m, n, k,
+                                           spaces[0].data_ptr() if nbytes else None, nbytes, stream()), "ws")
+    y_none = torch.empty((m, n), device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_f32_ws(w.planar.data_ptr(), xs[0].data_ptr(), y_none.data_ptr(), m, n, k, None, 0,
+                                           stream()), "ws none")
+    torch.cuda.synchronize()
+    assert torch.equal(y_ws.view(torch.int32), plain[0].view(torch.int32))
+    truth = oracle.matmul_f64(xs[0].cpu().numpy(), wf)
+    assert rel_err(y_none.cpu().numpy(), truth) < 2e-3 and rms_err(y_none.cpu().numpy().astype(np.float64), truth) < BAR
+    # f16 form: same plan, bits of the plain f16 call
+    x16 = xs[0].to(torch.float16)
+    y16_plain = torch.empty((m, n), device=DEV, dtype=torch.float16)
+    y16_ws = torch.empty_like(y16_plain)
+    capi.check(lib.lhip_q8_0_matmul_f16(w.planar.data_ptr(), x16.data_ptr(), y16_plain.data_ptr(), m, n, k, stream()), "f16")
+    capi.check(lib.lhip_q8_0_matmul_f16_ws(w.planar.data_ptr(), x16.data_ptr(), y16_ws.data_ptr(), m, n, k,
+                                           spaces[0].data_ptr() if nbytes else None, nbytes, stream()), "f16 ws")
+    torch.cuda.synchronize()
+    assert torch.equal(y16_ws.view(torch.int16), y16_plain.view(torch.int16))
+    # two streams, a workspace each, launches interleaved
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.empty((m, n), device=DEV) for _ in xs]
+    for _ in range(20):
+        for i, s in enumerate(streams):
+            capi.check(lib.lhip_q8_0_matmul_f32_ws(w.planar.data_ptr(), xs[i].data_ptr(), outs[i].data_ptr(), m, n, k,
+                                                   spaces[i].data_ptr() if nbytes else None, nbytes, s.cuda_stream), "ws 2")
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(outs[i].view(torch.int32), plain[i].view(torch.int32))
+
+
+def test_workspace_form_argument_checks():
+    lib = capi.load_library()
+    w = upload(*synth.q8_0_random(1024, 1024, seed=3))
+    x = torch.zeros((8, 1024), device=DEV)
+    y = torch.empty((8, 1024), device=DEV)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    assert lib.lhip_q8_0_matmul_workspace_nbytes(1, 1024, 1024) == 0       # a matvec needs none
+    assert lib.lhip_q8_0_matmul_workspace_nbytes(8, 1024, 1000) == 0       # invalid shape
+    assert lib.lhip_q8_0_matmul_workspace_nbytes(8, 1024, 1024) > 0
+    assert lib.lhip_q8_0_matmul_f32_ws(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 8, 1024, 1024, ws.data_ptr() + 64,
+                                       1 << 19, stream()) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_matmul_f32_ws(None, x.data_ptr(), y.data_ptr(), 8, 1024, 1024, ws.data_ptr(), 1 << 20,
+                                       stream()) == capi.LHIP_ERR_NULL_PTR
+    # one row goes to the matvec kernels, workspace or not
+    capi.check(lib.lhip_q8_0_matmul_f32_ws(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), 1, 1024, 1024, None, 0,
+                                           stream()), "one row")
+    torch.cuda.synchronize()
