@@ -552,12 +552,12 @@ static NodeIndex retrieved_projection(const Graph &g, NodeIndex weight) {
     return -1;
 }
 
-static void test_fused_decoder_layer() {
-    // The decoder layer of test_fusion_pass_cpu with real Q8_0 weights: host primitives on the dequantised weights,
-    // the device graph operator by operator, and the fused graph, twice with different activations (what is kept
-    // between executions - the interleaved gate|up weight, the norm weights on the device - is made once).
+static void test_fused_decoder_layer(const int dim, const int kv, const int ffn, const bool with_host) {
+    // The decoder layer of test_fusion_pass_cpu with real Q8_0 weights: host primitives on the dequantised weights
+    // (left out at the dimensions of Llama-3-8B, where they would take minutes), the device graph operator by
+    // operator, and the fused graph, twice with different activations (what is kept between executions - the
+    // interleaved gate|up weight, the norm weights on the device - is made once).
     std::mt19937 rng(7);
-    const int dim = 1024, kv = 256, ffn = 2048;
     const float eps = 1e-5f;
     const Q8 wq = random_q8(rng, dim, dim, 1e-3f), wk = random_q8(rng, kv, dim, 1e-3f), wv = random_q8(rng, kv, dim, 1e-3f),
              wo = random_q8(rng, dim, dim, 1e-3f), wg = random_q8(rng, ffn, dim, 1e-3f), wu = random_q8(rng, ffn, dim, 1e-3f),
@@ -576,7 +576,8 @@ static void test_fused_decoder_layer() {
     struct Weight { NodeIndex node; const Q8 *w; int64_t n, k; };
     const std::vector<Weight> weights{{hn.wq, &wq, dim, dim}, {hn.wk, &wk, kv, dim}, {hn.wv, &wv, kv, dim}, {hn.wo, &wo, dim, dim},
                                       {hn.wg, &wg, ffn, dim}, {hn.wu, &wu, ffn, dim}, {hn.wd, &wd, dim, ffn}};
-    for (const Weight &w : weights) fn(host, w.node)->value = host_tensor(w.w->dense);
+    if (with_host)
+        for (const Weight &w : weights) fn(host, w.node)->value = host_tensor(w.w->dense);
     auto prepare_device = [&](Graph &g, bool fuse) {
         const LayerNodes n = build_decoder_layer(g, dim, kv, ffn, eps);
         EXPECT(n.wd == hn.wd && n.out == hn.out);  // same construction order, same node numbers
@@ -597,12 +598,14 @@ static void test_fused_decoder_layer() {
     for (int round = 0; round < 2; ++round) {
         const std::vector<float> x = activations();
         for (Graph *g : {&host, &plain, &fused}) {
+            if (g == &host && !with_host) continue;
             fn(*g, hn.x)->value = host_tensor(x);
             g->execute();
         }
         struct Out { const char *what; NodeIndex host_node, weight; };
         for (const Out &o : {Out{"k", hn.k, hn.wk}, Out{"v", hn.v, hn.wv}, Out{"out", hn.out, -1}}) {
-            const std::vector<float> want = host_operand(host.results.at(o.host_node), o.what);
+            const bool have_want = with_host;
+            const std::vector<float> want = have_want ? host_operand(host.results.at(o.host_node), o.what) : std::vector<float>();
             auto device_result = [&](Graph &g) {
                 NodeIndex r = o.weight >= 0 ? retrieved_projection(g, o.weight) : -1;
                 if (o.weight < 0)  // the layer output: the retrieved node that is neither k nor v
@@ -611,12 +614,15 @@ static void test_fused_decoder_layer() {
                 return host_operand(g.results.at(r), o.what);
             };
             const std::vector<float> got_plain = device_result(plain), got_fused = device_result(fused);
-            EXPECT(got_plain.size() == want.size() && got_fused.size() == want.size());
+            EXPECT(got_plain.size() == got_fused.size() && !got_fused.empty());
             // operators' bar against the dequantised-weight host graph; fused against unfused differs only by f32
             // summation order (norm, dot products) and the exponential's last bits
-            EXPECT(max_abs_diff(got_plain, want) < 2e-3 * rms(want));
-            EXPECT(max_abs_diff(got_fused, want) < 2e-3 * rms(want));
-            EXPECT(max_abs_diff(got_fused, got_plain) < 1e-4 * rms(want));
+            if (have_want) {
+                EXPECT(got_plain.size() == want.size());
+                EXPECT(max_abs_diff(got_plain, want) < 2e-3 * rms(want));
+                EXPECT(max_abs_diff(got_fused, want) < 2e-3 * rms(want));
+            }
+            EXPECT(rms(got_plain) > 0 && max_abs_diff(got_fused, got_plain) < 1e-4 * rms(got_plain));
         }
         for (NodeIndex n = 0; n < static_cast<NodeIndex>(fused.nodes.size()); ++n)
             if (fused.nodes[n] && fused.nodes[n]->name() == "Q8InterleaveRows") {
@@ -675,7 +681,8 @@ int main(int argc, char **argv) {
             test_quantized_matvec_like_the_reference();
             test_graph_end_to_end(DType::F32);
             test_graph_end_to_end(DType::F16);
-            test_fused_decoder_layer();
+            test_fused_decoder_layer(1024, 256, 2048, true);
+            test_fused_decoder_layer(4096, 1024, 14336, false);  // the projections of a Llama-3-8B layer
             test_device_errors_surface_as_panics();
         }
     } catch (const std::exception &e) {
