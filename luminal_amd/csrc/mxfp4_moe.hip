@@ -271,6 +271,12 @@ struct MoeGemmArgs {
     // (planes of row stride q_kp, scales of row stride q_kp / 32) instead of writing `out`.
     uint8_t *q_hi, *q_lo, *q_sc;
     int q_kp;
+    // Direct form (a handful of routed rows, no plan launch in front): row tile t is routed entry t, its expert
+    // sel[t]; the activations are the bf16 rows of x, quantised by the workgroup itself; slot_of gets the identity.
+    const int *sel;
+    const __bf16 *x;
+    int *slot_of;
+    int n_experts, direct_rows;
 };
 
 // Maximum over the 16 lanes of a DPP row, in every lane of the row (quad swaps, then the two mirrors): register
@@ -608,17 +614,27 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
 // barriers — with D = 8 chunks of weights in flight per wave.  Needs
 // 2 * 16 * pitch + 16 * Kp/32 bytes of LDS (K up to ~4.6k).
 // ---------------------------------------------------------------------------
-template <int NT, bool GATED>
+template <int NT, bool GATED, bool DIRECT = false, int D = 8>
 __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
     static_assert(!GATED || NT % 2 == 0, "gated tiles pair each gate fragment with its up fragment");
-    constexpr int D = 8;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tile = blockIdx.y;
-    if (tile >= *g.n_tiles) return;
-    const int expert = g.tile_expert[tile];
-    const int row0 = g.tile_row0[tile];
-    const int rows = g.tile_rows[tile];  // 1..16
+    int expert, row0, rows;
+    if (DIRECT) {
+        if (tile >= g.direct_rows) return;
+        expert = g.sel[tile];
+        const bool known = expert >= 0 && expert < g.n_experts;
+        if (blockIdx.x == 0 && threadIdx.x == 0) g.slot_of[tile] = known ? tile : -1;
+        if (!known) return;
+        row0 = tile;
+        rows = 1;
+    } else {
+        if (tile >= *g.n_tiles) return;
+        expert = g.tile_expert[tile];
+        row0 = g.tile_row0[tile];
+        rows = g.tile_rows[tile];  // 1..16
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -668,7 +684,12 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
 #pragma unroll
     for (int j = 0; j < D; ++j) load_b(j, j);
 
-    {
+    if (DIRECT) {
+        // the routed entry's row of x, quantised here as the plan launch would have (groups of four threads share
+        // a 32-block: Kp / 8 is a multiple of four, so a group is whole or absent)
+        const __bf16 *x_row = g.x + static_cast<size_t>(tile / g.a_div) * g.K;
+        for (int q = tid; q < Kp / 8; q += 256) mx_quantize_act_item(q, x_row, lds, lds + a_plane, lds_sc, 1, g.K, Kp);
+    } else {
         const int per_row = Kp / 16;  // 16-byte pieces per row and plane
         const int pieces = rows * per_row * 2;
         for (int q = tid; q < pieces; q += 256) {
@@ -801,6 +822,151 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
             for (int f = 0; f < NT; ++f)
                 if (col[f] < g.N) static_cast<float *>(g.out)[orow + col[f]] = acc[f][v];
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Down projection of a handful of routed rows (at most 4: one token's top-4) with the weighted sum over a token's
+// experts folded in, for the direct form: no plan, no combine launch.  A workgroup owns 16 output columns for
+// ALL routed rows: routed row t multiplies the 16 weight rows of expert sel[t]; the four waves split K (chunk c
+// belongs to wave c % 4) and meet in LDS, then y[token][col] = bf16(sum_s wts * down) in the combine kernel's
+// order.  The rows' quantised activations (all of K) are staged in LDS once; the weight stream runs on across
+// the routed rows, D chunks in flight per wave.
+// ---------------------------------------------------------------------------
+constexpr int kDirectRows = 4;
+
+struct MoeDownDirectArgs {
+    const uint8_t *a_hi, *a_lo, *a_sc;  // quantised activations: R rows of Kp / Kp/32 bytes, row = routed entry
+    const uint8_t *w_nib, *w_sc;        // planar down weights of all experts, rows_per_expert rows each
+    int rows_per_expert, Kp, N;
+    const int *sel;
+    const float *wts;
+    int R, topk, n_experts;
+    float *out;                         // [R][N] f32 rows (read back by lhip_mxfp4_moe_read_intermediates)
+    __bf16 *y;                          // [R / topk][N]
+};
+
+__global__ __launch_bounds__(256) void mx_moe_down_direct_kernel(MoeDownDirectArgs g) {
+    constexpr int D = 8;  // chunks of a routed row per wave: K up to 4 * D * kChunk
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, grp = lane >> 4;
+    const int Kp = g.Kp, chunks = Kp / kChunk, R = g.R;
+    const int a_row = moe_small_pitch(Kp), a_plane = 16 * a_row, sc_row = Kp / 32;
+    unsigned char *lds_sc = lds + 2 * a_plane;
+    const int n0 = blockIdx.x * 16;  // N is a multiple of 16
+    const int col = n0 + r;
+
+    // Per routed row: where its expert's weights start (lane t of a register pair holds routed row t's, read with
+    // v_readlane at a scalar index) and whether it names a real expert (a bit mask).  No selects between 64-bit
+    // scalars and no branches in the loop below: a branch makes the compiler's wait counts for the weight sets in
+    // flight fall back to "wait for everything".
+    unsigned off_lo, off_hi, known;
+    {
+        const int t = lane & (kDirectRows - 1);
+        const int e = t < R ? g.sel[t] : -1;
+        const bool ok = e >= 0 && e < g.n_experts;
+        const size_t off = ((static_cast<size_t>(ok ? e : 0) * g.rows_per_expert + n0) >> 4) * chunks * 64;
+        off_lo = static_cast<unsigned>(off);
+        off_hi = static_cast<unsigned>(off >> 32);
+        known = static_cast<unsigned>(__ballot(ok)) & ((1u << kDirectRows) - 1u);  // lanes 0..3 are rows 0..3
+    }
+    const uint8_t *w_lane = g.w_nib + lane * 16;
+    const uint8_t *s_lane = g.w_sc + (lane & ~3);
+    const int s_shift = 8 * (lane & 3);
+    // Chunk wave + 4 * j of routed row t is weight set (t, j), j < D: all of a wave's share - at most
+    // kDirectRows * D kilobytes - is requested up front and held in registers (a workgroup has the SIMDs to
+    // itself: 512 registers per lane), so the whole launch costs one trip to memory instead of one per D chunks.
+    static_assert(D * 4 * kChunk >= 4096, "K up to 4096");
+    BSet<1, 1> bs[kDirectRows][D];
+#pragma unroll
+    for (int t = 0; t < kDirectRows; ++t) {
+        const int tc = min(t, R - 1);  // rows past R re-read the last row's lines: never used
+        const size_t off = static_cast<size_t>(__builtin_amdgcn_readlane(off_hi, tc)) << 32 | __builtin_amdgcn_readlane(off_lo, tc);
+        const uint8_t *wb = w_lane + off * 16;
+        const uint8_t *sb = s_lane + off;
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int cc = min(wave + 4 * j, chunks - 1);  // chunks past the end re-read the last one: never used
+            bs[t][j].q[0] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(wb + static_cast<size_t>(cc) * 1024));
+            bs[t][j].s[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sb + cc * 64));
+        }
+    }
+    {
+        const int per_row = Kp / 16;
+        const int pieces = R * per_row * 2;
+        for (int q = tid; q < pieces; q += 256) {
+            const int plane = q / (R * per_row), rem = q - plane * (R * per_row);
+            const int row = rem / per_row, c16 = rem - row * per_row;
+            const mu32x4 v = *reinterpret_cast<const mu32x4 *>((plane ? g.a_lo : g.a_hi) + static_cast<size_t>(row) * Kp + c16 * 16);
+            *reinterpret_cast<mu32x4 *>(lds + plane * a_plane + row * a_row + c16 * 16) = v;
+        }
+        const int sc_words = R * (sc_row / 4);
+        for (int q = tid; q < sc_words; q += 256) {
+            const int row = q / (sc_row / 4), w4 = q - row * (sc_row / 4);
+            reinterpret_cast<uint32_t *>(lds_sc + row * sc_row)[w4] =
+                reinterpret_cast<const uint32_t *>(g.a_sc + static_cast<size_t>(row) * sc_row)[w4];
+        }
+    }
+    __syncthreads();
+
+    // Rows past R hold stale LDS bytes; their results are never used.
+    const unsigned char *ap = lds + r * a_row + grp * 16;
+    const unsigned char *sp = lds_sc + r * sc_row + grp;
+    float vals[kDirectRows];  // this wave's share of routed row t's 16 outputs (lanes 0..15)
+#pragma unroll
+    for (int t = 0; t < kDirectRows; ++t) {
+        v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+        const bool live = (t < R) & ((known >> t) & 1u);
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int c = wave + 4 * j;
+            asm volatile("" : "+v"(bs[t][j].q[0]), "+v"(bs[t][j].s[0]));
+            if (live & (c < chunks)) {  // wave-uniform
+                const unsigned char *p = ap + c * kChunk;
+                const mu32x4 h0 = *reinterpret_cast<const mu32x4 *>(p);
+                const mu32x4 h1 = *reinterpret_cast<const mu32x4 *>(p + 64);
+                const mu32x4 l0 = *reinterpret_cast<const mu32x4 *>(p + a_plane);
+                const mu32x4 l1 = *reinterpret_cast<const mu32x4 *>(p + a_plane + 64);
+                const int sa = sp[c * 4];
+                const v8i ah = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
+                const v8i al = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
+                const mu32x4 q = bs[t][j].q[0];
+                const int sb = static_cast<int>(bs[t][j].s[0] >> s_shift);
+                const v8i b = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ah, b, acc, 0, 4, 0, sa, 0, sb);
+                acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(al, b, acc, 0, 4, 0, sa - kLoShift, 0, sb);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        vals[t] = acc[t];  // routed row t is row t of the fragment
+    }
+
+    __syncthreads();  // every wave is done reading the staged activations
+    float *part = reinterpret_cast<float *>(lds);  // [4 waves][kDirectRows][16 columns]
+    if (grp == 0) {
+#pragma unroll
+        for (int t = 0; t < kDirectRows; ++t) part[(wave * kDirectRows + t) * 16 + r] = vals[t];
+    }
+    __syncthreads();
+    if (wave != 0 || grp != 0 || col >= g.N) return;
+    float down[kDirectRows];
+#pragma unroll
+    for (int t = 0; t < kDirectRows; ++t) {
+        down[t] = ((part[t * 16 + r] + part[(kDirectRows + t) * 16 + r]) + part[(2 * kDirectRows + t) * 16 + r]) +
+                  part[(3 * kDirectRows + t) * 16 + r];
+        if (t < R) g.out[static_cast<size_t>(t) * g.N + col] = ((known >> t) & 1u) ? down[t] : 0.f;
+    }
+    for (int token = 0; token * g.topk < R; ++token) {
+        float a = 0.f;
+        for (int sidx = 0; sidx < g.topk; ++sidx) {
+            const int t = token * g.topk + sidx;
+            const float d = t == 0 ? down[0] : t == 1 ? down[1] : t == 2 ? down[2] : down[3];
+            if ((known >> t) & 1u) a = fmaf(g.wts[t], d, a);
+        }
+        g.y[static_cast<size_t>(token) * g.N + col] = static_cast<__bf16>(a);
     }
 }
 
@@ -1020,15 +1186,51 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     // whole-row kernel / chunked: T = 1 31.6 / 39.5, T = 2 45.9 / 42.8, T = 8 80 / 64, T = 32 126 / 92).
     const bool decode_sized = R <= 4;
 
+    auto *gu = static_cast<const uint8_t *>(w_gate_up_planar);
+    auto *dn = static_cast<const uint8_t *>(w_down_planar);
+    if (decode_sized && R <= kDirectRows && moe_small_lds_bytes(Hp) <= 150 * 1024 && Ip <= 4096) {
+        // Direct form: two launches.  The gate/up GEMM takes routed entry t as its row tile t and quantises the
+        // token's row of x itself; the down GEMM sums over the token's experts as it finishes.
+        MoeGemmArgs a1{};
+        a1.a_div = topk_i;
+        a1.w_nib = gu; a1.w_sc = gu + mx_scale_offset(e * 2 * i, h);
+        a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
+        a1.out = w.act;
+        a1.q_hi = w.a_hi; a1.q_lo = w.a_lo; a1.q_sc = w.a_sc; a1.q_kp = Ip;
+        a1.sel = sel_dev; a1.x = static_cast<const __bf16 *>(x_dev); a1.slot_of = w.plan.slot_of;
+        a1.n_experts = E; a1.direct_rows = R;
+        {
+            const size_t lds_bytes = moe_small_lds_bytes(Hp);
+            auto kern = mx_moe_gemm_small_kernel<2, true, true>;
+            if (lds_bytes > 64 * 1024)
+                LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((I + 63) / 64), static_cast<unsigned>(R)), dim3(256), lds_bytes, s, a1);
+            LHIP_CHECK_LAUNCH();
+        }
+        MoeDownDirectArgs a2{};
+        a2.a_hi = w.a_hi; a2.a_lo = w.a_lo; a2.a_sc = w.a_sc;
+        a2.w_nib = dn; a2.w_sc = dn + mx_scale_offset(e * h, i);
+        a2.rows_per_expert = H; a2.Kp = Ip; a2.N = H;
+        a2.sel = sel_dev; a2.wts = wts_dev; a2.R = R; a2.topk = topk_i; a2.n_experts = E;
+        a2.out = w.out; a2.y = static_cast<__bf16 *>(y_dev);
+        {
+            const size_t lds_bytes = moe_small_lds_bytes(Ip);
+            if (lds_bytes > 64 * 1024)
+                LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(mx_moe_down_direct_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            hipLaunchKernelGGL(mx_moe_down_direct_kernel, dim3(static_cast<unsigned>(H / 16)), dim3(256), lds_bytes, s, a2);
+            LHIP_CHECK_LAUNCH();
+        }
+        return LHIP_OK;
+    }
+
     {
         const size_t items = static_cast<size_t>(T) * (Hp / 8);
         hipLaunchKernelGGL(moe_prepare_kernel, dim3(static_cast<unsigned>(1 + (items + 1023) / 1024)), dim3(1024), 0, s,
                            sel_dev, R, E, BM, w.plan, static_cast<const __bf16 *>(x_dev), w.x_hi, w.x_lo, w.x_sc, T, H, Hp);
         LHIP_CHECK_LAUNCH();
     }
-    auto *gu = static_cast<const uint8_t *>(w_gate_up_planar);
-    auto *dn = static_cast<const uint8_t *>(w_down_planar);
-
     MoeGemmArgs a1{};
     a1.a_hi = w.x_hi; a1.a_lo = w.x_lo; a1.a_sc = w.x_sc;
     a1.a_index = w.plan.slot_src; a1.a_div = topk_i;

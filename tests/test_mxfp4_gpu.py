@@ -185,6 +185,29 @@ def test_moe_small_layers_vs_oracle(oracle, t, e, h, i, topk):
     check_stages(oracle, layer, xf, w_gu, w_dn, sel, wts, y)
 
 
+@pytest.mark.parametrize("t,e,h,i,topk", [(1, 8, 256, 128, 4), (1, 8, 160, 96, 3), (1, 4, 64, 64, 1), (2, 8, 128, 288, 2),
+                                          (4, 8, 416, 64, 1), (1, 32, 2880, 2880, 4)])
+def test_moe_direct_form_for_a_handful_of_routed_rows(oracle, t, e, h, i, topk):
+    """At most four routed rows take two launches (no plan launch in front, the weighted sum inside the down GEMM):
+    one to four rows, one or several tokens, ragged K, against the oracle and stage by stage; a routed entry that
+    names no expert contributes nothing."""
+    layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=3 * t + e + h)
+    xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t * 11 + topk, scale=0.05 if h < 1000 else 1.0)
+    truth = oracle.moe_forward(xf, w_gu, w_dn, sel, wts, act_bf16=True)
+    assert norm_err(y, truth) < 4e-3
+    check_stages(oracle, layer, xf, w_gu, w_dn, sel, wts, y)
+    if t * topk >= 2:
+        # the same call with the first routed entry pointing at no expert: as if its weight were zero
+        bad = sel.copy()
+        bad[0, 0] = e + 5
+        xd = torch.from_numpy(oracle.f32_to_bf16_bits(xf).view(np.int16)).to(DEV).view(torch.bfloat16)
+        y_bad = layer.process(xd, torch.from_numpy(bad).to(DEV), torch.from_numpy(wts).to(DEV)).float().cpu().numpy()
+        w0 = wts.copy()
+        w0[0, 0] = 0.0
+        y_zero = layer.process(xd, torch.from_numpy(sel).to(DEV), torch.from_numpy(w0).to(DEV)).float().cpu().numpy()
+        assert np.array_equal(y_bad, y_zero)
+
+
 def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
     # activations spanning many binades inside one 32-block: the hi/lo fp8 split must not lose the small ones
     e, h, i, t, topk = 2, 64, 64, 16, 1
