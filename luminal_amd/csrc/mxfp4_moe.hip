@@ -830,8 +830,8 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
 // experts folded in, for the direct form: no plan, no combine launch.  A workgroup owns 16 output columns for
 // ALL routed rows: routed row t multiplies the 16 weight rows of expert sel[t]; the four waves split K (chunk c
 // belongs to wave c % 4) and meet in LDS, then y[token][col] = bf16(sum_s wts * down) in the combine kernel's
-// order.  The rows' quantised activations (all of K) are staged in LDS once; the weight stream runs on across
-// the routed rows, D chunks in flight per wave.
+// order.  The rows' quantised activations (all of K) are staged in LDS once; a wave requests its whole share of
+// the weights (all routed rows, K up to 4096) before anything else and holds it in registers.
 // ---------------------------------------------------------------------------
 constexpr int kDirectRows = 4;
 
@@ -860,9 +860,9 @@ __global__ __launch_bounds__(256) void mx_moe_down_direct_kernel(MoeDownDirectAr
     const int col = n0 + r;
 
     // Per routed row: where its expert's weights start (lane t of a register pair holds routed row t's, read with
-    // v_readlane at a scalar index) and whether it names a real expert (a bit mask).  No selects between 64-bit
-    // scalars and no branches in the loop below: a branch makes the compiler's wait counts for the weight sets in
-    // flight fall back to "wait for everything".
+    // v_readlane) and whether it names a real expert (a bit mask).  The loads below stay free of branches and of
+    // selects between 64-bit scalars (which compile to branches): a branch between loads makes the compiler's
+    // wait counts for the sets in flight fall back to "wait for everything".
     unsigned off_lo, off_hi, known;
     {
         const int t = lane & (kDirectRows - 1);
