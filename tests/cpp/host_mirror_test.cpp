@@ -13,8 +13,12 @@
 #include <cstdio>
 #include <random>
 
+#include <fstream>
+#include <sstream>
+
 #include "../../luminal_amd/host/luminal_hip.hpp"
 #include "../../luminal_amd/host/luminal_hip_fusion.hpp"
+#include "../../luminal_amd/host/luminal_hip_gguf.hpp"
 
 using namespace luminal_hip;
 
@@ -422,6 +426,92 @@ static void test_fusion_pass_cpu() {
                .find("one contiguous row") != std::string::npos);
 }
 
+// tests/golden/gguf_v3_literal.hex: 644 bytes assembled by hand from examples/llama/src/gguf.rs:190-263 (hex pairs,
+// '#' starts a comment): a v3 header, one key of every value type, alignment 64, one F32 and one Q8_0 tensor.
+static std::string literal_gguf_bytes() {
+    std::string path = __FILE__;
+    path = path.substr(0, path.rfind('/')) + "/../golden/gguf_v3_literal.hex";
+    std::ifstream f(path);
+    std::string line, out;
+    while (std::getline(f, line)) {
+        line = line.substr(0, line.find('#'));
+        int hi = -1;
+        for (char ch : line) {
+            const int v = ch >= '0' && ch <= '9' ? ch - '0' : ch >= 'a' && ch <= 'f' ? ch - 'a' + 10 : ch >= 'A' && ch <= 'F' ? ch - 'A' + 10 : -1;
+            if (v < 0) continue;
+            if (hi < 0) hi = v;
+            else {
+                out.push_back(static_cast<char>(hi * 16 + v));
+                hi = -1;
+            }
+        }
+    }
+    return out;
+}
+
+static void test_gguf_reader_cpu() {
+    const std::string bytes = literal_gguf_bytes();
+    EXPECT(bytes.size() == 644);
+    std::istringstream in(bytes);
+    const GgufHeader h = GgufReader(in).read_header();
+    EXPECT(h.version == 3 && h.alignment == 64 && h.data_offset == 512 && h.tensors.size() == 2);  // 477 header bytes rounded up to 64
+    const GgufTensorInfo &a = h.tensors.at("a.weight"), &q = h.tensors.at("blk.0.attn_q.weight");
+    EXPECT(a.n_elements == 3 && a.offset == 0 && a.dtype == kGgmlF32);
+    EXPECT(q.n_elements == 64 && q.offset == 64 && q.dtype == kGgmlQ8_0);
+    // only integer types of at most 32 bits set the alignment (gguf.rs:246-255): the same key as a u64 is ignored
+    const size_t at = bytes.find("general.alignment") + 17;
+    {
+        std::string head = bytes.substr(0, at);
+        const uint32_t type_u64 = 10;
+        const uint64_t v = 64;
+        head.append(reinterpret_cast<const char *>(&type_u64), 4).append(reinterpret_cast<const char *>(&v), 8);
+        head += bytes.substr(at + 8, 477 - (at + 8));
+        std::istringstream in2(head);
+        const GgufHeader h2 = GgufReader(in2).read_header();
+        EXPECT(h2.alignment == 32 && h2.data_offset == (head.size() + 31) / 32 * 32 && h2.tensors.size() == 2);
+    }
+    // the reference's panics
+    {
+        std::string bad = bytes;
+        bad[0] = 'X';
+        std::istringstream s1(bad);
+        EXPECT(panic_message([&] { GgufReader(s1).read_header(); }).find("unknown magic") != std::string::npos);
+        bad = bytes;
+        bad[4] = 4;  // version
+        std::istringstream s2(bad);
+        EXPECT(panic_message([&] { GgufReader(s2).read_header(); }).find("unsupported version 4") != std::string::npos);
+        bad = bytes.substr(0, 100);
+        std::istringstream s3(bad);
+        EXPECT(panic_message([&] { GgufReader(s3).read_header(); }).find("unexpected end of file") != std::string::npos);
+    }
+}
+
+static void test_gguf_file_to_graph() {
+    // the literal file through the loader and the pass: the F32 tensor lands on the host, the Q8_0 tensor (2 x 32:
+    // row 0 = 0.5 * [0..31], row 1 = -2 * [-16..15]) on the device in planar form and multiplies a row of ones
+    const std::string bytes = literal_gguf_bytes();
+    const std::string path = "/tmp/luminal_hip_literal.gguf";
+    {
+        std::ofstream out(path, std::ios::binary);
+        out.write(bytes.data(), static_cast<std::streamsize>(bytes.size()));
+    }
+    Graph g;
+    const NodeIndex a = g.add(std::make_unique<Function>()), w = g.add(std::make_unique<Function>()), x = g.add(std::make_unique<Function>());
+    const NodeIndex y = build_matmul(g, x, {1, 32}, w, 2);
+    g.to_retrieve.insert(y);
+    fn(g, x)->value = host_tensor(std::vector<float>(32, 1.f));
+    const auto q_weights = q8_load_hip_file(path, g, {{"a/weight", a}, {"blk/0/attn_q/weight", w}});
+    EXPECT((q_weights == std::vector<NodeIndex>{w}));
+    EXPECT((host_operand(fn(g, a)->value, "a") == std::vector<float>{1.f, -2.f, 0.5f}));
+    HipQuantizedCompiler(q_weights).compile(g);
+    g.execute();
+    const std::vector<float> got = host_operand(g.results.at(*g.to_retrieve.begin()), "y");
+    EXPECT((got == std::vector<float>{248.f, 32.f}));
+    EXPECT(panic_message([&] { q8_load_hip_file(path, g, {{"missing", a}}); }).find("is not in the file") != std::string::npos);
+    EXPECT(panic_message([&] { q8_load_hip_file("/tmp/no_such_file.gguf", g, {{"a/weight", a}}); }).find("cannot open") != std::string::npos);
+    std::remove(path.c_str());
+}
+
 // ---------------------------------------------------------------- device
 struct Q8 {
     std::vector<int8_t> q;
@@ -676,11 +766,13 @@ int main(int argc, char **argv) {
         test_primitives_on_the_host();
         test_compiler_pass_cpu();
         test_fusion_pass_cpu();
+        test_gguf_reader_cpu();
         if (mode == "gpu") {
             check(lhip_init(0), "lhip_init");
             test_quantized_matvec_like_the_reference();
             test_graph_end_to_end(DType::F32);
             test_graph_end_to_end(DType::F16);
+            test_gguf_file_to_graph();
             test_fused_decoder_layer(1024, 256, 2048, true);
             test_fused_decoder_layer(4096, 1024, 14336, false);  // the projections of a Llama-3-8B layer
             test_device_errors_surface_as_panics();

@@ -1,6 +1,6 @@
-"""The C++ host mirror (luminal_amd/host/luminal_hip.hpp) through its own test program, tests/cpp/host_mirror_test.cpp:
-the compiler pass and the operators' panics without a device, then the reference-style matvec / gather / matmul
-checks on the GPU."""
+"""The C++ host mirror (luminal_amd/host/*.hpp) through its own test program, tests/cpp/host_mirror_test.cpp:
+the compiler passes, the GGUF header reader and the operators' panics without a device, then the reference-style
+matvec / gather / matmul checks, a GGUF file through loader and pass, and the fused decoder layer on the GPU."""
 import os
 import subprocess
 
@@ -13,8 +13,9 @@ from luminal_amd import capi
 def _binary():
     if not os.path.exists(capi.LIB_PATH):
         pytest.skip("libluminal_hip.so has not been built")
-    src_time = max(os.path.getmtime(lib_build.HOST_TEST_SRC),
-                   os.path.getmtime(os.path.join(os.path.dirname(capi.LIB_PATH), "host", "luminal_hip.hpp")))
+    host_dir = os.path.join(os.path.dirname(capi.LIB_PATH), "host")
+    src_time = max([os.path.getmtime(lib_build.HOST_TEST_SRC)] +
+                   [os.path.getmtime(os.path.join(host_dir, f)) for f in os.listdir(host_dir) if f.endswith(".hpp")])
     if not os.path.exists(lib_build.HOST_TEST_BIN) or os.path.getmtime(lib_build.HOST_TEST_BIN) < src_time:
         lib_build.build_host_test(verbose=False)
     return lib_build.HOST_TEST_BIN
