@@ -762,6 +762,22 @@ static void test_device_errors_surface_as_panics() {
 
 int main(int argc, char **argv) {
     const std::string mode = argc > 1 ? argv[1] : "cpu";
+    if (mode == "gguf-header" && argc > 2) {
+        // the header of a file as this reader sees it, one line per fact, for a caller that compares it with its own
+        try {
+            std::ifstream f(argv[2], std::ios::binary);
+            const GgufHeader h = GgufReader(f).read_header();
+            std::printf("version %u\nalignment %llu\ndata_offset %llu\n", h.version, (unsigned long long)h.alignment,
+                        (unsigned long long)h.data_offset);
+            for (auto &[name, t] : h.tensors)
+                std::printf("tensor %s %llu %llu %u\n", name.c_str(), (unsigned long long)t.n_elements,
+                            (unsigned long long)t.offset, t.dtype);
+            return 0;
+        } catch (const std::exception &e) {
+            std::printf("panic %s\n", e.what());
+            return 3;
+        }
+    }
     try {
         test_primitives_on_the_host();
         test_compiler_pass_cpu();
