@@ -418,7 +418,7 @@ impl HipFusedMatvecCompiler {
         }
         if retrieved(graph, old) || graph.no_delete.contains(&old) {
             let copy = host_copy(graph);
-            remap(old, copy, ids, graph);
+            remap(old, copy, &mut *ids, graph);
         }
     }
 
@@ -522,7 +522,7 @@ impl HipFusedMatvecCompiler {
                     }
                     if retrieved(graph, q) || graph.no_delete.contains(&q) {
                         let down = graph.add_op(HipCopyFromDevice::<f32>::default()).input(fused, i as u8, ShapeTracker::new(())).finish();
-                        remap(q, down, ids, graph);
+                        remap(q, down, &mut *ids, graph);
                     }
                     graph.graph.remove_node(q);
                 }

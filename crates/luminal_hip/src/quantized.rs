@@ -375,7 +375,7 @@ impl<T: HipFloat> HipQuantizedCompiler<T> {
         };
         // the consumers of the SumReduce now read the new node; Mul and SumReduce go, and what only fed them with it
         move_outgoing_edge(red, made, &mut graph.graph);
-        remap(red, made, ids, graph);
+        remap(red, made, &mut *ids, graph);
         graph.graph.remove_node(red);
         graph.graph.remove_node(mul);
         prune_dead(graph, a_src);
@@ -416,7 +416,7 @@ impl<T: HipFloat> HipQuantizedCompiler<T> {
         }
         if retrieved.is_some() {
             // to_retrieve, no_delete and the caller's handles move from the device node to the host copy
-            remap(q, down, ids, graph);
+            remap(q, down, &mut *ids, graph);
         }
     }
 }
