@@ -1174,11 +1174,18 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     MoeWorkspace w = carve(workspace_dev, t, h, i, e, topk);
     const int Hp = static_cast<int>(pad128(h)), Ip = static_cast<int>(pad128(i));
 
-    // Row tile: tall enough for an expert with two standard deviations more rows than the average (rows per
-    // expert are roughly Poisson), so that nearly every expert is one tile and its weights are read once.
+    // Row tile.  Up to 128 rows: the smallest height that holds an expert with two standard deviations more rows
+    // than the average (rows per expert are roughly Poisson), so that nearly every expert is one tile and its
+    // weights are read once.  Heights of 64 and 80 rows run as four-wave workgroups, two to a CU: each wave then
+    // has four or five row fragments of matrix work per weight fragment it loads, enough to cover the two chunks
+    // of weights it keeps in flight, and one workgroup's prologue, barrier and epilogue run under the other's
+    // matrix work.  Experts with more rows than 128 are cut into 80-row tiles as well: their second and third
+    // reads of the weights come out of L2 / the last-level cache, and a short last tile wastes less than it does
+    // at 160 rows (measured, us per layer, 80-row / 160-row tiles: T = 1024 269-275 / 272-281, T = 1536 375 / 419,
+    // T = 2048 485 / 486, T = 4096 885 / 930; and at T = 512 80-row / 128-row tiles: 161 / 183-201).
     const int avg = (R + E - 1) / E;
     const int need = avg + 2 * static_cast<int>(sqrtf(static_cast<float>(avg)) + 0.5f);
-    const int mt = need > 128 ? 10 : need > 64 ? 8 : (need > 32 ? 4 : (need > 16 ? 2 : 1));
+    const int mt = need <= 16 ? 1 : need <= 32 ? 2 : need <= 64 ? 4 : need <= 80 ? 5 : need <= 128 ? 8 : 5;
     const int BM = 16 * mt;
     const int max_tiles = R / BM + E;
     // One token's worth of routed rows (batch-1 decode): stage each tile's activation rows whole and run the
@@ -1251,9 +1258,9 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
                                                        : launch_moe_gemm<1, 4, true>(a1, cb1w, max_tiles, s);
             break;
         case 2: st = launch_moe_gemm<2, 4, true>(a1, cb1w, max_tiles, s); break;
-        case 4: st = launch_moe_gemm<4, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
-        case 8: st = launch_moe_gemm<8, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
-        default: st = launch_moe_gemm<10, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
+        case 4: st = launch_moe_gemm<4, 4, true, 1, 2>(a1, cb1w, max_tiles, s); break;
+        case 5: st = launch_moe_gemm<5, 4, true, 1, 2>(a1, cb1w, max_tiles, s); break;
+        default: st = launch_moe_gemm<8, 4, true, 2, 2>(a1, cb1w, max_tiles, s); break;
     }
     if (st) return st;
     MoeGemmArgs a2{};
@@ -1271,9 +1278,9 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         const int cb2 = (H + 127) / 128, cb2w = (H + 255) / 256;  // 4 waves x NT fragments of 16
         switch (mt) {
             case 2: st = launch_moe_gemm<2, 2, false>(a2, cb2, max_tiles, s); break;
-            case 4: st = launch_moe_gemm<4, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
-            case 8: st = launch_moe_gemm<8, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
-            default: st = launch_moe_gemm<10, 3, false, 2, 2>(a2, (H + 191) / 192, max_tiles, s); break;
+            case 4: st = launch_moe_gemm<4, 4, false, 1, 2>(a2, cb2w, max_tiles, s); break;
+            case 5: st = launch_moe_gemm<5, 3, false, 1, 2>(a2, (H + 191) / 192, max_tiles, s); break;
+            default: st = launch_moe_gemm<8, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
         }
     }
     if (st) return st;

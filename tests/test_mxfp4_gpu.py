@@ -175,9 +175,10 @@ def run_layer(oracle, layer, t, h, e, topk, seed, scale=1.0):
 
 @pytest.mark.parametrize("t,e,h,i,topk", [(1, 4, 64, 64, 2), (5, 4, 160, 96, 2), (40, 8, 128, 288, 4),
                                           (300, 8, 256, 160, 4), (1500, 4, 128, 128, 2), (64, 32, 96, 64, 4),
-                                          (170, 8, 128, 96, 4), (100, 8, 416, 64, 4)])
+                                          (170, 8, 128, 96, 4), (100, 8, 416, 64, 4), (120, 8, 128, 96, 4)])
 def test_moe_small_layers_vs_oracle(oracle, t, e, h, i, topk):
-    # ragged K (not multiples of 128), every row-tile size (16..160 rows), experts with no tokens
+    # ragged K (not multiples of 128), every row-tile height (16, 32, 64, 80, 128 rows; experts of ~150 and ~750 rows
+    # cut into 80-row tiles), experts with no tokens
     layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=t + e + h)
     xf, sel, wts, y = run_layer(oracle, layer, t, h, e, topk, seed=t * 7 + 1, scale=0.05)
     truth = oracle.moe_forward(xf, w_gu, w_dn, sel, wts, act_bf16=True)
