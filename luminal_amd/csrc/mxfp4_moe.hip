@@ -128,8 +128,15 @@ struct MoePlan {
     int *slot_of;      // [R]   routed entry -> slot (-1 if its expert id is invalid)
     int *tile_expert;  // [max_tiles]
     int *tile_row0;    // [max_tiles] first slot of the tile
-    int *tile_rows;    // [max_tiles] valid rows in the tile
+    int *tile_rows;    // [max_tiles] valid rows in the tile (0 = unused entry)
     int *n_tiles;      // [1]
+    int max_tiles;     // entries of the three tile arrays
+    // 0: tiles are listed in expert order from entry 0.  Otherwise the list is cut into eight ranges of this many
+    // entries, one per XCD (range x is read by the workgroups whose dispatch number is x modulo 8), and the
+    // tiles, still in expert order, are dealt to the ranges in eight contiguous, equal shares: the tiles of an
+    // expert, and all column blocks of a tile, then run on one XCD and find each other's weights and
+    // activation rows in its L2.
+    int tiles_per_xcd;
 };
 
 __device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int R, int E, int BM, const MoePlan &p) {
@@ -137,6 +144,11 @@ __device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int 
     for (int e = threadIdx.x; e < E; e += 1024) {
         cnt[e] = 0;
         cur[e] = 0;
+    }
+    for (int t = threadIdx.x; t < p.max_tiles; t += 1024) {  // entries no tile is written to stay marked unused
+        p.tile_expert[t] = 0;
+        p.tile_row0[t] = 0;
+        p.tile_rows[t] = 0;
     }
     __syncthreads();
     for (int r = threadIdx.x; r < R; r += 1024) {
@@ -149,19 +161,28 @@ __device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int 
     // ceil(cnt / BM) tiles of equal height (a multiple of 16 rows): 140 rows with BM = 128 become 80 + 60 rather
     // than 128 + 12, and the GEMM skips the row fragments a tile does not have.
     for (int e = threadIdx.x; e < E; e += 1024) {
-        int o = 0, nt = 0;
-        for (int q = 0; q < e; ++q) {
-            o += cnt[q];
-            nt += (cnt[q] + BM - 1) / BM;  // equals the number of tiles written for q below
+        int o = 0, nt = 0, total = 0;
+        for (int q = 0; q < E; ++q) {
+            const int tq = (cnt[q] + BM - 1) / BM;  // equals the number of tiles written for q below
+            if (q < e) {
+                o += cnt[q];
+                nt += tq;
+            }
+            total += tq;
         }
         off[e] = o;
         p.offsets[e] = o;
         const int tiles_e = (cnt[e] + BM - 1) / BM;
         const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
         for (int m0 = 0; m0 < cnt[e]; m0 += per) {
-            p.tile_expert[nt] = e;
-            p.tile_row0[nt] = o + m0;
-            p.tile_rows[nt] = min(per, cnt[e] - m0);
+            int at = nt;
+            if (p.tiles_per_xcd) {  // tile nt of `total` goes to range x = floor(8 nt / total), behind that range's earlier tiles
+                const int x = nt * 8 / total;
+                at = x * p.tiles_per_xcd + nt - (x * total + 7) / 8;
+            }
+            p.tile_expert[at] = e;
+            p.tile_row0[at] = o + m0;
+            p.tile_rows[at] = min(per, cnt[e] - m0);
             ++nt;
         }
         if (e == E - 1) {
@@ -266,6 +287,7 @@ struct MoeGemmArgs {
     int K, Kp;
     int N;                              // output columns per expert (I or H)
     const int *tile_expert, *tile_row0, *tile_rows, *n_tiles;
+    int tiles_per_xcd;                  // layout of the tile list (MoePlan::tiles_per_xcd)
     void *out;                          // bf16 [R][N] (gated) or f32 [R][N]
     // Gated GEMM with NT == 4 only: when q_hi is set, the epilogue quantises its bf16 result for the next GEMM
     // (planes of row stride q_kp, scales of row stride q_kp / 32) instead of writing `out`.
@@ -324,14 +346,24 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 3 x A_BUF
 
-    // The tile's description is read together with the tile count (the plan arrays have an entry for
-    // every workgroup of the grid), so an unused workgroup costs one memory round trip, not two.
-    const int tile = blockIdx.y;
-    const int n_tiles = *g.n_tiles;
+    // Which tile and which column block.  Workgroups are dispatched in the order of their linear number
+    // (x fastest) and dealt to the eight XCDs in turn, so the workgroups with the same number modulo 8 share an L2.
+    // With a tile list laid out per XCD, those take the entries of their XCD's range in order, all column blocks
+    // of one tile after another: the tile's activation rows, which every column block reads, and the weights
+    // of an expert cut into several tiles then come out of that L2 after their first use.  Entries without a
+    // tile have no rows.
+    int tile = blockIdx.y, cb = blockIdx.x;
+    if (g.tiles_per_xcd) {
+        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+        const int turn = linear >> 3;
+        const int entry = turn / static_cast<int>(gridDim.x);  // < gridDim.y / 8 = tiles_per_xcd
+        cb = turn - entry * static_cast<int>(gridDim.x);
+        tile = (linear & 7) * g.tiles_per_xcd + entry;
+    }
     const int expert = g.tile_expert[tile];
     const int row0 = g.tile_row0[tile];
     const int rows = g.tile_rows[tile];
-    if (tile >= n_tiles) return;
+    if (rows == 0) return;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -354,10 +386,10 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
     for (int f = 0; f < NT; ++f) {
         int n0, wrow0;  // first column of the fragment, first weight row inside the expert
         if (GATED) {  // fragments 2p / 2p+1 = gate / up rows of the same 16 intermediate columns
-            n0 = ((blockIdx.x * 4 + wave) * (NT / 2) + (f >> 1)) * 16;
+            n0 = ((cb * 4 + wave) * (NT / 2) + (f >> 1)) * 16;
             wrow0 = ((f & 1) ? g.N : 0) + min(n0, g.N - 16);
         } else {
-            n0 = ((blockIdx.x * 4 + wave) * NT + f) * 16;
+            n0 = ((cb * 4 + wave) * NT + f) * 16;
             wrow0 = min(n0, g.N - 16);
         }
         col[f] = n0 + r;
@@ -541,11 +573,11 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
     // ---- epilogue: acc[i][f][v] is row i*16 + 4*grp + v, column fragment f, column r
     if constexpr (GATED && NT == 4) {
         if (g.q_hi) {
-            // The wave's two (gate, up) pairs are the 32 intermediate columns [32 b, 32 b + 32), b = 4 blockIdx.x +
+            // The wave's two (gate, up) pairs are the 32 intermediate columns [32 b, 32 b + 32), b = 4 cb +
             // wave: one quantisation block of the next GEMM's activations.  Same arithmetic as
             // mx_quantize_act_item on the bf16-rounded result (block maximum over the 16 lanes of a row group),
             // so the intermediate activations never go through memory as bf16.
-            const int b = blockIdx.x * 4 + wave;
+            const int b = cb * 4 + wave;
 #pragma unroll
             for (int i = 0; i < MTW; ++i)
 #pragma unroll
@@ -1040,7 +1072,7 @@ struct MoeWorkspace {
 static MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
     MoeWorkspace w{};
     const int64_t R = T * topk;
-    const int64_t max_tiles = R / 16 + E + 1;  // tiles of at least 16 rows, one partial tile per expert
+    const int64_t max_tiles = R / 16 + E + 8;  // tiles of at least 16 rows, one partial tile per expert, rounded up to eight
     size_t off = 0;
     auto take = [&](size_t bytes) {
         uint8_t *p = base ? static_cast<uint8_t *>(base) + off : nullptr;
@@ -1187,7 +1219,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     const int need = avg + 2 * static_cast<int>(sqrtf(static_cast<float>(avg)) + 0.5f);
     const int mt = need <= 16 ? 1 : need <= 32 ? 2 : need <= 64 ? 4 : need <= 80 ? 5 : need <= 128 ? 8 : 5;
     const int BM = 16 * mt;
-    const int max_tiles = R / BM + E;
+    const int max_tiles = (R / BM + E + 7) / 8 * 8;  // upper bound of the tile count, whole eighths for the per-XCD list
     // One token's worth of routed rows (batch-1 decode): stage each tile's activation rows whole and run the
     // barrier-free weight stream.  From two tokens on the chunked kernel below is faster (measured, us per layer,
     // whole-row kernel / chunked: T = 1 31.6 / 39.5, T = 2 45.9 / 42.8, T = 8 80 / 64, T = 32 126 / 92).
@@ -1232,6 +1264,9 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         return LHIP_OK;
     }
 
+    // The decode-sized kernels walk the plain tile list; the chunked kernels take the one laid out per XCD.
+    w.plan.max_tiles = max_tiles;
+    w.plan.tiles_per_xcd = decode_sized ? 0 : max_tiles / 8;
     {
         const size_t items = static_cast<size_t>(T) * (Hp / 8);
         hipLaunchKernelGGL(moe_prepare_kernel, dim3(static_cast<unsigned>(1 + (items + 1023) / 1024)), dim3(1024), 0, s,
@@ -1244,7 +1279,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a1.w_nib = gu; a1.w_sc = gu + mx_scale_offset(e * 2 * i, h);
     a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
-    a1.n_tiles = w.plan.n_tiles; a1.out = w.act;
+    a1.n_tiles = w.plan.n_tiles; a1.tiles_per_xcd = w.plan.tiles_per_xcd; a1.out = w.act;
     const bool whole_rows = mt == 1 && decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024;
     // Every gated kernel launched below quantises its result for the down GEMM in its epilogue.
     a1.q_hi = w.a_hi; a1.q_lo = w.a_lo; a1.q_sc = w.a_sc; a1.q_kp = Ip;
@@ -1269,7 +1304,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     a2.w_nib = dn; a2.w_sc = dn + mx_scale_offset(e * h, i);
     a2.rows_per_expert = H; a2.K = I; a2.Kp = Ip; a2.N = H;
     a2.tile_expert = w.plan.tile_expert; a2.tile_row0 = w.plan.tile_row0; a2.tile_rows = w.plan.tile_rows;
-    a2.n_tiles = w.plan.n_tiles; a2.out = w.out;
+    a2.n_tiles = w.plan.n_tiles; a2.tiles_per_xcd = w.plan.tiles_per_xcd; a2.out = w.out;
     if (mt == 1) {
         st = decode_sized && moe_small_lds_bytes(Ip) <= 150 * 1024
                  ? launch_moe_gemm_small<1, false>(a2, (H + 63) / 64, max_tiles, s)
