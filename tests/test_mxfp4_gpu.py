@@ -209,6 +209,32 @@ def test_moe_direct_form_for_a_handful_of_routed_rows(oracle, t, e, h, i, topk):
         assert np.array_equal(y_bad, y_zero)
 
 
+@pytest.mark.parametrize("t,e,h,i,topk,hot", [(700, 8, 128, 96, 2, (2, 5)), (600, 8, 128, 96, 1, (3,)),
+                                              (90, 16, 128, 96, 2, (0, 15)), (400, 12, 160, 64, 1, (11,))])
+def test_moe_lopsided_routing(oracle, t, e, h, i, topk, hot):
+    """Every token goes to the same one or two experts: those experts are many row tiles (up to 18 tiles of one expert in
+    a row of the tile list), all the others none, and the number of tiles is not a multiple of eight - so the eight
+    per-XCD shares of the tile list are ragged and some hold a single expert's tiles only.  Some routed entries name
+    no expert.  Against the oracle."""
+    layer, w_gu, w_dn = make_layer(oracle, e, h, i, seed=t + e)
+    rng = np.random.default_rng(t)
+    x = (rng.standard_normal((t, h)) * 0.05).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x)
+    xf = oracle.bf16_bits_to_f32(bits)
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    logits[:, list(hot)] += 50.0
+    sel, wts = route_topk(torch.from_numpy(logits).to(DEV), topk)
+    assert set(np.unique(sel.cpu().numpy())) == set(hot)
+    sel[::97, 0] = e + 1  # no such expert: the entry contributes nothing
+    xd = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    y = layer.process(xd, sel, wts).float().cpu().numpy()
+    sel_h, wts_h = sel.cpu().numpy(), wts.cpu().numpy().copy()
+    w_live = np.where(sel_h < e, wts_h, 0.0).astype(np.float32)
+    truth = oracle.moe_forward(xf, w_gu, w_dn, np.where(sel_h < e, sel_h, 0), w_live, act_bf16=True)
+    assert norm_err(y, truth) < 4e-3
+    assert np.isfinite(y).all()
+
+
 def test_moe_activation_split_is_exact_on_wide_dynamic_range(oracle):
     # activations spanning many binades inside one 32-block: the hi/lo fp8 split must not lose the small ones
     e, h, i, t, topk = 2, 64, 64, 16, 1
