@@ -264,6 +264,42 @@ def test_moe_benchmark_layer(oracle, t):
     assert np.isfinite(y).all()
 
 
+@pytest.mark.parametrize("t", [64, 1024])
+def test_moe_benchmark_layer_properties(t):
+    """At the benchmark sizes, what holds whatever the numbers are: the same call twice gives the same bits (the
+    order of the rows inside an expert's range is left to atomics, and no result depends on it); permuting the tokens
+    permutes the output rows, bit for bit (another plan, other tiles, the same arithmetic per row); doubling the
+    routing weights doubles the output exactly; a token routed to one expert in all four entries, with weights
+    (1/2, 1/2, 0, 0), gives what weights (1, 0, 0, 0) give."""
+    e, h, i, topk = synth.MOE_EXPERTS, synth.MOE_HIDDEN, synth.MOE_INTER, synth.MOE_TOPK
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(31 + t)
+
+    def weight(n, k):
+        nb = n * k // 32
+        raw = torch.empty((nb, 17), dtype=torch.uint8, device=DEV)
+        raw[:, :16] = torch.randint(0, 256, (nb, 16), dtype=torch.uint8, device=DEV, generator=gen)
+        raw[:, 16] = torch.randint(119, 128, (nb,), dtype=torch.uint8, device=DEV, generator=gen)
+        return Mxfp4Weight.from_raw(raw, n, k, DEV)
+
+    layer = MoEExperts(weight(e * 2 * i, h), weight(e * h, i), e, h, i)
+    x = torch.randn((t, h), device=DEV, generator=gen).to(torch.bfloat16)
+    sel, wts = route_topk(torch.randn((t, e), device=DEV, generator=gen), topk)
+    y = layer.process(x, sel, wts).clone()
+    assert torch.equal(layer.process(x, sel, wts), y)
+    perm = torch.randperm(t, device=DEV, generator=gen)
+    assert torch.equal(layer.process(x[perm].contiguous(), sel[perm].contiguous(), wts[perm].contiguous()), y[perm])
+    assert torch.equal(layer.process(x, sel, (2.0 * wts).contiguous()).float(), 2.0 * y.float())
+    # four equal rows of one expert: r/2 + r/2 + 0 + 0 = r exactly in f32
+    one = sel[:, :1].expand(t, topk).contiguous()
+    halves = torch.zeros((t, topk), dtype=torch.float32, device=DEV)
+    halves[:, :2] = 0.5
+    single = torch.zeros((t, topk), dtype=torch.float32, device=DEV)
+    single[:, 0] = 1.0
+    assert torch.equal(layer.process(x, one, halves), layer.process(x, one, single))
+    assert bool(torch.isfinite(y.float()).all())
+
+
 def test_moe_argument_errors():
     lib = capi.load_library()
     p = 0x1000
