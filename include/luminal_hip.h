@@ -267,6 +267,11 @@ lhip_status lhip_mxfp4_repack(const void *raw_dev, void *planar_dev, int64_t n, 
 lhip_status lhip_mxfp4_unpack(const void *planar_dev, void *raw_dev, int64_t n, int64_t k, void *stream);
 /* Exact dequantisation to f32[N][K] (every e8m0 code, 0xff gives NaN). */
 lhip_status lhip_mxfp4_dequant_f32(const void *planar_dev, float *out_dev, int64_t n, int64_t k, void *stream);
+/* Dequantisation to bf16[N][K] (out 16-byte aligned) with the conversion instruction the expert GEMMs use
+ * (v_cvt_scalef32_pk_bf16_fp4): e2m1 * 2^(e-127) has two significant bits and bf16 has f32's exponent range, so the
+ * result equals lhip_mxfp4_dequant_f32's wherever that is a normal number (e8m0 codes 2..252 for every e2m1 value).
+ * No counterpart in the reference; it is what pins the matrix path's weight values bit for bit. */
+lhip_status lhip_mxfp4_dequant_bf16(const void *planar_dev, void *out_bf16_dev, int64_t n, int64_t k, void *stream);
 
 /* Router: for each of t tokens, the topk largest of its e logits (ties to the
  * lower index) into sel[t][topk], and softmax over those k into wts[t][topk]. */
@@ -276,14 +281,30 @@ lhip_status lhip_moe_route_topk(const float *logits_dev, int32_t *sel_dev, float
 /* Expert layer: y[t] = sum_s wts[t][s] * down_e( up_e(x[t]) * swish(gate_e(x[t])) ), e = sel[t][s].
  *   w_gate_up_planar : planar MXFP4 of shape (e*2*i, h): expert-major, rows [0,i) of an expert = gate, [i,2i) = up
  *   w_down_planar    : planar MXFP4 of shape (e*h, i)
- *   x, y             : bf16 (t, h); accumulation in f32 on the block-scaled matrix instruction
+ *   x, y             : bf16 (t, h); accumulation in f32; the SwiGLU result is rounded to bf16 between the two matmuls
  *   sel, wts         : routing as produced by lhip_moe_route_topk (an id outside [0,e) drops that term)
  *   workspace_dev    : lhip_mxfp4_moe_workspace_nbytes(...) bytes, 256-byte aligned; contents are scratch
- * h and i must be multiples of 32, e <= 1024.  e8m0 codes 0xff (NaN) in the weights are not supported here. */
+ * h and i must be multiples of 32, e <= 1024.  e8m0 codes 0xff (NaN) in the weights are not supported here.
+ *
+ * Two forms of the matmuls (lhip_mxfp4_moe_bf16 is LHIP_MOE_EXACT):
+ *   LHIP_MOE_EXACT  weights expanded exactly to bf16 in registers (lhip_mxfp4_dequant_bf16's values), bf16 matrix
+ *                   instruction, f32 accumulation: every product is exact and every matmul output lies within the
+ *                   f32 accumulation error of the exact product of its inputs (the reference's "dequantise exactly,
+ *                   then multiply", examples/llama/src/loader.rs:227-241).
+ *   LHIP_MOE_FAST   the block-scaled f8f6f4 matrix instruction on the raw fp4 codes, each bf16 activation split
+ *                   exactly into two fp8 numbers.  The instruction aligns the 128 products of a step to the largest
+ *                   and drops what lies 2^-13 below it, so an output carries an absolute error of up to about
+ *                   2^-11 * sum over 128-wide chunks of max |a_k w_k|: small against typical outputs, unbounded
+ *                   relative to outputs that cancel. */
+#define LHIP_MOE_EXACT 0
+#define LHIP_MOE_FAST 1
 size_t lhip_mxfp4_moe_workspace_nbytes(int64_t t, int64_t h, int64_t i, int64_t e, int64_t topk);
 lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
                                 const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                 int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream);
+lhip_status lhip_mxfp4_moe_bf16_mode(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                     const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                     int64_t i, int64_t e, int64_t topk, int32_t mode, void *workspace_dev, void *stream);
 
 /* lhip_mxfp4_moe_bf16 for callers that cannot allocate a workspace (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc): no counterpart in the reference.  The workspace is a scratch array inside the
@@ -298,14 +319,18 @@ lhip_status lhip_mxfp4_moe_bf16_static(const void *w_gate_up_planar, const void 
                                        const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                        int64_t i, int64_t e, int64_t topk, void *stream);
 
-/* The intermediates of the last lhip_mxfp4_moe_bf16 call that used this workspace with the same (t, h, i, e, topk),
+/* The intermediates of the last layer call that used this workspace with the same (t, h, i, e, topk) and mode
+ * (lhip_mxfp4_moe_read_intermediates: LHIP_MOE_EXACT, the mode of lhip_mxfp4_moe_bf16 and _static),
  * per routed entry r = t*topk + s: act_dev (t*topk, i) f32 = up * swish(gate) as the down projection consumed it
- * (a bf16 value, held in the workspace as two fp8 numbers and a block scale: decoded exactly), down_dev (t*topk, h)
+ * (a bf16 value; the fast form holds it as two fp8 numbers and a block scale, decoded exactly), down_dev (t*topk, h)
  * f32 = that entry's down projection before the weighted sum.  Either pointer may be NULL.  No counterpart in the
  * reference; it lets a caller check each of the layer's two matmuls against its own inputs, since the rounding of
  * the activations to bf16 between them makes the end-to-end result a discontinuous function of the first one. */
 lhip_status lhip_mxfp4_moe_read_intermediates(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
                                               int64_t h, int64_t i, int64_t e, int64_t topk, void *stream);
+lhip_status lhip_mxfp4_moe_read_intermediates_mode(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
+                                                   int64_t h, int64_t i, int64_t e, int64_t topk, int32_t mode,
+                                                   void *stream);
 
 /* ---- the operators around the matmuls in the Llama-3 decode loop (f32) --------
  * What the reference assembles from primitive ops in examples/llama/src/model.rs,

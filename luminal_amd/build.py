@@ -16,6 +16,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libluminal_hip.so")
+OBJ_DIR = os.path.join(HERE, "build")  # objects, one per source (not tracked)
 # Code object with the matvec kernels under C names, for hosts that launch through hipModule* themselves.
 MODULE_SRC = os.path.join(CSRC, "module", "q8_gemv_module.hip")
 MODULE = os.path.join(HERE, "luminal_hip_kernels.hsaco")
@@ -47,15 +48,40 @@ def _run(cmd: list[str]) -> None:
         print(out, file=sys.stderr)
 
 
-def build(verbose: bool = True) -> str:
+def _object_path(src: str) -> str:
+    return os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(src))[0] + ".o")
+
+
+def _headers() -> list[str]:
+    return glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(os.path.dirname(HERE), "include", "*.h"))
+
+
+def build(verbose: bool = True, incremental: bool = False, jobs: int | None = None) -> str:
+    """Compile every source to an object (in parallel), then link.  ``incremental`` skips a source whose object is
+    newer than it and than every header; the default recompiles everything."""
+    from concurrent.futures import ThreadPoolExecutor
+
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no HIP sources under {CSRC}")
     cc = hipcc()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    newest_header = max((os.path.getmtime(h) for h in _headers()), default=0.0)
+
+    def stale(src: str) -> bool:
+        obj = _object_path(src)
+        return not (incremental and os.path.exists(obj) and
+                    os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header))
+
+    todo = [s for s in srcs if stale(s)]
     if verbose:
-        print(f"[luminal_amd.build] {cc} -> {LIB}", file=sys.stderr)
-    _run([cc, *COMMON, *DEVICE_FLAGS, "-shared", "-o", LIB, *srcs])
-    build_module(verbose)
+        print(f"[luminal_amd.build] {cc}: {len(todo)} of {len(srcs)} sources -> {LIB}", file=sys.stderr)
+    jobs = jobs or min(8, os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "8")))
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        list(pool.map(lambda s: _run([cc, *COMMON, *DEVICE_FLAGS, "-c", "-o", _object_path(s), s]), todo))
+    _run([cc, *COMMON, "-shared", "-o", LIB, *[_object_path(s) for s in srcs]])
+    if todo or not os.path.exists(MODULE):
+        build_module(verbose)
     return LIB
 
 
@@ -87,5 +113,5 @@ def build_host_test(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv)
     build_host_test()

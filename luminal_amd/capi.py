@@ -14,6 +14,8 @@ LHIP_ERR_MISALIGNED = 3
 LHIP_ERR_HIP = 4
 LHIP_ERR_UNSUPPORTED = 5
 
+LHIP_MOE_EXACT, LHIP_MOE_FAST = 0, 1
+
 _vp, _i64, _sz, _int = C.c_void_p, C.c_int64, C.c_size_t, C.c_int
 
 # name -> (restype, argtypes); one entry per declaration in include/luminal_hip.h
@@ -67,6 +69,9 @@ SIGNATURES = {
     "lhip_moe_route_topk": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "lhip_mxfp4_moe_workspace_nbytes": (_sz, [_i64] * 5),
     "lhip_mxfp4_moe_bf16": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp, _vp]),
+    "lhip_mxfp4_moe_bf16_mode": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [C.c_int32, _vp, _vp]),
+    "lhip_mxfp4_moe_read_intermediates_mode": (C.c_int32, [_vp] * 3 + [_i64] * 5 + [C.c_int32, _vp]),
+    "lhip_mxfp4_dequant_bf16": (C.c_int32, [_vp, _vp, _i64, _i64, _vp]),
     "lhip_mxfp4_moe_bf16_static": (C.c_int32, [_vp] * 6 + [_i64] * 5 + [_vp]),
     "lhip_mxfp4_moe_read_intermediates": (C.c_int32, [_vp] * 3 + [_i64] * 5 + [_vp]),
     "lhip_gather_rows_f32": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

@@ -22,6 +22,27 @@ lhip_status hip_failed(hipError_t e);
 // Kernel launches report configuration errors through hipGetLastError.
 #define LHIP_CHECK_LAUNCH() LHIP_HIP_TRY(hipGetLastError())
 
+// Kernels that use more than 64 KiB of dynamic LDS have to be told so once (per device); remembered here so that a
+// launch costs no hipFuncSetAttribute call after the first.  One object per kernel (a function-local static of its
+// launcher).
+struct LdsOptIn {
+    size_t bytes[64] = {};  // largest size set so far, per device
+};
+static inline lhip_status lds_opt_in(LdsOptIn &st, const void *kernel, size_t lds_bytes, bool needed) {
+    if (!needed) return LHIP_OK;
+    int dev = 0;
+    LHIP_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return LHIP_ERR_UNSUPPORTED;
+    if (__atomic_load_n(&st.bytes[dev], __ATOMIC_RELAXED) >= lds_bytes) return LHIP_OK;
+    LHIP_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    __atomic_store_n(&st.bytes[dev], lds_bytes, __ATOMIC_RELAXED);
+    return LHIP_OK;
+}
+
+static inline lhip_status lds_opt_in(LdsOptIn &st, const void *kernel, size_t lds_bytes) {
+    return lds_opt_in(st, kernel, lds_bytes, lds_bytes > 64 * 1024);
+}
+
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 static inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }

@@ -462,9 +462,8 @@ struct Program {
 template <int G, int HD>
 static lhip_status launch_program(const Program &pr, hipStream_t s) {
     auto kernel = decode_program_kernel<G, HD>;
-    if (pr.lds_bytes > 48 * 1024)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(pr.lds_bytes)));
+    static LdsOptIn opt;
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kernel), pr.lds_bytes, pr.lds_bytes > 48 * 1024)) return st;
     hipLaunchKernelGGL(decode_program_begin_kernel, dim3(1), dim3(64), 0, s, pr.sync_dev);
     LHIP_CHECK_LAUNCH();
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pr.grid)), dim3(kProgThreads), pr.lds_bytes, s, pr.ops_dev,

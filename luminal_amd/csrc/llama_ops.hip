@@ -527,10 +527,10 @@ lhip_status lhip_attention_f32(const float *qkv_dev, const float *k_cache_dev, c
         return LHIP_OK;
     }
     // the score row is dynamic LDS on top of 32.1 KiB of static arrays: past 64 KiB in all the kernel has to opt in
-    if (static_cast<size_t>(max_seq) * sizeof(float) + sizeof(float4) * 32 * 64 + 64 > 64 * 1024)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(static_cast<size_t>(max_seq) * sizeof(float))));
+    static LdsOptIn opt;
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(attention_kernel), static_cast<size_t>(max_seq) * sizeof(float),
+                                    static_cast<size_t>(max_seq) * sizeof(float) + sizeof(float4) * 32 * 64 + 64 > 64 * 1024))
+        return st;
     hipLaunchKernelGGL(attention_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(q_heads)),
                        dim3(kAttnThreads),
                        static_cast<size_t>(max_seq) * sizeof(float), as_stream(stream), qkv_dev, k_cache_dev,

@@ -27,28 +27,9 @@
 // which shows on elements far below the block's scale).  Two MFMAs (hi, lo) per
 // weight fragment then give the exact sum of exact products in f32, which is
 // closer to the f32 semantics than a bf16 MFMA over rounded weights would be.
-#include "common.h"
-
-#include <type_traits>
-#include <utility>
+#include "mxfp4_moe_device.h"
 
 namespace lhip {
-
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef uint32_t mu32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int kChunk = 128;      // K elements per MFMA
-constexpr int kLoShift = 5;      // the lo plane of an activation is held times 2^5 and multiplied with block scale - 5
-constexpr float kLoGain = 32.f;
-constexpr int kARow = 160;       // LDS bytes per activation row of a chunk: 128 fp8 + 32 padding (with 16 the fragment reads,
-                                 // lane (r, g) at r * pitch + 16 g, take twice as long: measured 8.0 against 4.3 cycles per read)
-
-static inline int64_t pad128(int64_t k) { return (k + 127) / 128 * 128; }
-// Row pitch of a whole quantised activation row in LDS (Kp a multiple of 128): the row plus padding that makes the
-// pitch 160 mod 256, the residue measured free of bank conflicts for the fragment reads.
-__host__ __device__ static inline int moe_small_pitch(int Kp) { return Kp + ((Kp & 255) ? 32 : 160); }
-
 // ---------------------------------------------------------------------------
 // Router: top-k of the logits (ties to the lower index), softmax over the k.
 // ---------------------------------------------------------------------------
@@ -116,94 +97,6 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(const float *__rest
         if (lane == bi) avail = false;
     }
     if (lane < topk) wts[static_cast<size_t>(t) * topk + lane] = mine * (1.0f / sum);
-}
-
-// ---------------------------------------------------------------------------
-// Plan: group the R = T*topk routed entries by expert and cut each expert's rows
-// into tiles of BM.  One workgroup; E <= 1024.
-// ---------------------------------------------------------------------------
-struct MoePlan {
-    int *offsets;      // [E+1] first slot of each expert
-    int *slot_src;     // [R]   slot -> routed entry r = t*topk + s
-    int *slot_of;      // [R]   routed entry -> slot (-1 if its expert id is invalid)
-    int *tile_expert;  // [max_tiles]
-    int *tile_row0;    // [max_tiles] first slot of the tile
-    int *tile_rows;    // [max_tiles] valid rows in the tile (0 = unused entry)
-    int *n_tiles;      // [1]
-    int max_tiles;     // entries of the three tile arrays
-    // 0: tiles are listed in expert order from entry 0.  Otherwise the list is cut into eight ranges of this many
-    // entries, one per XCD (range x is read by the workgroups whose dispatch number is x modulo 8), and the
-    // tiles, still in expert order, are dealt to the ranges in eight contiguous, equal shares: the tiles of an
-    // expert, and all column blocks of a tile, then run on one XCD and find each other's weights and
-    // activation rows in its L2.
-    int tiles_per_xcd;
-};
-
-__device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int R, int E, int BM, const MoePlan &p) {
-    __shared__ int cnt[1024], off[1025], cur[1024];
-    for (int e = threadIdx.x; e < E; e += 1024) {
-        cnt[e] = 0;
-        cur[e] = 0;
-    }
-    for (int t = threadIdx.x; t < p.max_tiles; t += 1024) {  // entries no tile is written to stay marked unused
-        p.tile_expert[t] = 0;
-        p.tile_row0[t] = 0;
-        p.tile_rows[t] = 0;
-    }
-    __syncthreads();
-    for (int r = threadIdx.x; r < R; r += 1024) {
-        const int e = sel[r];
-        if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
-    }
-    __syncthreads();
-    // Thread e lays out expert e: its first slot and first tile are prefix sums over the experts before it
-    // (E <= 1024 broadcast reads from LDS), then it writes its own tiles.
-    // ceil(cnt / BM) tiles of equal height (a multiple of 16 rows): 140 rows with BM = 128 become 80 + 60 rather
-    // than 128 + 12, and the GEMM skips the row fragments a tile does not have.
-    for (int e = threadIdx.x; e < E; e += 1024) {
-        int o = 0, nt = 0, total = 0;
-        for (int q = 0; q < E; ++q) {
-            const int tq = (cnt[q] + BM - 1) / BM;  // equals the number of tiles written for q below
-            if (q < e) {
-                o += cnt[q];
-                nt += tq;
-            }
-            total += tq;
-        }
-        off[e] = o;
-        p.offsets[e] = o;
-        const int tiles_e = (cnt[e] + BM - 1) / BM;
-        const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
-        for (int m0 = 0; m0 < cnt[e]; m0 += per) {
-            int at = nt;
-            if (p.tiles_per_xcd) {  // tile nt of `total` goes to range x = floor(8 nt / total), behind that range's earlier tiles
-                const int x = nt * 8 / total;
-                at = x * p.tiles_per_xcd + nt - (x * total + 7) / 8;
-            }
-            p.tile_expert[at] = e;
-            p.tile_row0[at] = o + m0;
-            p.tile_rows[at] = min(per, cnt[e] - m0);
-            ++nt;
-        }
-        if (e == E - 1) {
-            off[E] = o + cnt[e];
-            p.offsets[E] = o + cnt[e];
-            *p.n_tiles = nt;
-        }
-    }
-    __syncthreads();
-    // Order inside an expert's range is arbitrary (atomic): every row is computed
-    // independently, and slot_of lets the combine step find it again.
-    for (int r = threadIdx.x; r < R; r += 1024) {
-        const int e = sel[r];
-        if (e >= 0 && e < E) {
-            const int pos = off[e] + atomicAdd(&cur[e], 1);
-            p.slot_src[pos] = r;
-            p.slot_of[r] = pos;
-        } else {
-            p.slot_of[r] = -1;
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------
@@ -301,32 +194,6 @@ struct MoeGemmArgs {
     int n_experts, direct_rows;
 };
 
-// Maximum over the 16 lanes of a DPP row, in every lane of the row (quad swaps, then the two mirrors): register
-// moves only, where a shuffle would go through the LDS pipeline.
-__device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)));
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)));
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)));
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)));
-    return v;
-}
-
-// f(integral_constant<int, 1>) ... f(integral_constant<int, N-1>), expanded at compile time.
-template <class F, int... Is>
-__device__ __forceinline__ void static_for_from1_impl(F &&f, std::integer_sequence<int, Is...>) {
-    (f(std::integral_constant<int, Is + 1>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for_from1(F &&f) {
-    static_for_from1_impl(static_cast<F &&>(f), std::make_integer_sequence<int, (N > 1 ? N - 1 : 0)>{});
-}
-
-template <int MT, int NT>
-struct BSet {
-    mu32x4 q[NT];
-    uint32_t s[NT];
-    bool valid;  // wave-uniform: false for a dead chunk past the padded K
-};
 
 // WR = 1: 4 waves, each all MT row fragments x its NT column fragments.  WR = 2: 8 waves, the upper four
 // take the odd row fragments, so every SIMD holds two waves with half the accumulators each
@@ -865,7 +732,6 @@ __global__ __launch_bounds__(256) void mx_moe_gemm_small_kernel(MoeGemmArgs g) {
 // order.  The rows' quantised activations (all of K) are staged in LDS once; a wave requests its whole share of
 // the weights (all routed rows, K up to 4096) before anything else and holds it in registers.
 // ---------------------------------------------------------------------------
-constexpr int kDirectRows = 4;
 
 struct MoeDownDirectArgs {
     const uint8_t *a_hi, *a_lo, *a_sc;  // quantised activations: R rows of Kp / Kp/32 bytes, row = routed entry
@@ -1057,71 +923,26 @@ __global__ __launch_bounds__(256) void moe_read_intermediates_kernel(const int *
             down[static_cast<size_t>(r) * H + h] = slot >= 0 ? out[static_cast<size_t>(slot) * H + h] : 0.f;
 }
 
-// ---------------------------------------------------------------------------
-// Workspace carving (256-byte aligned pieces, in this order).
-// ---------------------------------------------------------------------------
-struct MoeWorkspace {
-    MoePlan plan;
-    uint8_t *x_hi, *x_lo, *x_sc;  // quantised x, T rows of Kp(H)
-    __bf16 *act;                  // [R][I]
-    uint8_t *a_hi, *a_lo, *a_sc;  // quantised act, R rows of Kp(I)
-    float *out;                   // [R][H]
-    size_t total;
-};
-
-static MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
-    MoeWorkspace w{};
-    const int64_t R = T * topk;
-    const int64_t max_tiles = R / 16 + E + 8;  // tiles of at least 16 rows, one partial tile per expert, rounded up to eight
-    size_t off = 0;
-    auto take = [&](size_t bytes) {
-        uint8_t *p = base ? static_cast<uint8_t *>(base) + off : nullptr;
-        off += (bytes + 255) & ~size_t{255};
-        return p;
-    };
-    w.plan.offsets = reinterpret_cast<int *>(take((E + 1) * 4));
-    w.plan.slot_src = reinterpret_cast<int *>(take(R * 4));
-    w.plan.slot_of = reinterpret_cast<int *>(take(R * 4));
-    w.plan.tile_expert = reinterpret_cast<int *>(take(max_tiles * 4));
-    w.plan.tile_row0 = reinterpret_cast<int *>(take(max_tiles * 4));
-    w.plan.tile_rows = reinterpret_cast<int *>(take(max_tiles * 4));
-    w.plan.n_tiles = reinterpret_cast<int *>(take(4));
-    const int64_t Hp = pad128(H), Ip = pad128(I);
-    w.x_hi = take(T * Hp);
-    w.x_lo = take(T * Hp);
-    w.x_sc = take(T * (Hp / 32));
-    w.act = reinterpret_cast<__bf16 *>(take(R * I * 2));
-    w.a_hi = take(R * Ip);
-    w.a_lo = take(R * Ip);
-    w.a_sc = take(R * (Ip / 32));
-    w.out = reinterpret_cast<float *>(take(R * H * 4));
-    w.total = off;
-    return w;
-}
-
 template <int MT, int NT, bool GATED, int WR = 1, int D = 4>
 static lhip_status launch_moe_gemm(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
     constexpr int BM = 16 * MT;
     const size_t lds_bytes = 3 * (2 * static_cast<size_t>(BM) * kARow + BM * 4);
     auto kern = mx_moe_gemm_kernel<MT, NT, GATED, WR, D>;
-    if (lds_bytes > 64 * 1024)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    static LdsOptIn opt;
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256 * WR),
                        lds_bytes, s, a);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
-static inline size_t moe_small_lds_bytes(int Kp) { return 2 * 16 * static_cast<size_t>(moe_small_pitch(Kp)) + 16 * (Kp / 32); }
 
 template <int NT, bool GATED>
 static lhip_status launch_moe_gemm_small(const MoeGemmArgs &a, int col_blocks, int max_tiles, hipStream_t s) {
     const size_t lds_bytes = moe_small_lds_bytes(a.Kp);
     auto kern = mx_moe_gemm_small_kernel<NT, GATED>;
-    if (lds_bytes > 64 * 1024)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    static LdsOptIn opt;
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(max_tiles)), dim3(256),
                        lds_bytes, s, a);
     LHIP_CHECK_LAUNCH();
@@ -1154,6 +975,15 @@ static lhip_status moe_scratch_address(unsigned char **out) {
 lhip_status moe_static_setup() {
     unsigned char *p = nullptr;
     return moe_scratch_address(&p);
+}
+
+lhip_status moe_launch_combine(const float *out, const int *slot_of, const float *wts, __bf16 *y, int T, int H, int topk,
+                               hipStream_t s) {
+    const size_t threads = static_cast<size_t>(T) * (H / 4);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s, out, slot_of,
+                       wts, y, T, H, topk);
+    LHIP_CHECK_LAUNCH();
+    return LHIP_OK;
 }
 
 static lhip_status check_moe_shape(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk) {
@@ -1193,10 +1023,18 @@ size_t lhip_mxfp4_moe_workspace_nbytes(int64_t t, int64_t h, int64_t i, int64_t 
 lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
                                 const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
                                 int64_t i, int64_t e, int64_t topk, void *workspace_dev, void *stream) {
+    return lhip_mxfp4_moe_bf16_mode(w_gate_up_planar, w_down_planar, x_dev, sel_dev, wts_dev, y_dev, t, h, i, e, topk,
+                                    LHIP_MOE_EXACT, workspace_dev, stream);
+}
+
+lhip_status lhip_mxfp4_moe_bf16_mode(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
+                                     const int32_t *sel_dev, const float *wts_dev, void *y_dev, int64_t t, int64_t h,
+                                     int64_t i, int64_t e, int64_t topk, int32_t mode, void *workspace_dev, void *stream) {
     if (!w_gate_up_planar || !w_down_planar || !x_dev || !sel_dev || !wts_dev || !y_dev || !workspace_dev)
         return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_moe_shape(t, h, i, e, topk)) return s;
     if (h % 4 != 0) return LHIP_ERR_INVALID_SHAPE;
+    if (mode != LHIP_MOE_EXACT && mode != LHIP_MOE_FAST) return LHIP_ERR_UNSUPPORTED;
     if (!aligned(w_gate_up_planar, 256) || !aligned(w_down_planar, 256) || !aligned(x_dev, 16) ||
         !aligned(workspace_dev, 256) || !aligned(y_dev, 2))
         return LHIP_ERR_MISALIGNED;
@@ -1204,6 +1042,10 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
     const int T = static_cast<int>(t), H = static_cast<int>(h), I = static_cast<int>(i), E = static_cast<int>(e);
     const int topk_i = static_cast<int>(topk), R = T * topk_i;
     MoeWorkspace w = carve(workspace_dev, t, h, i, e, topk);
+    if (mode == LHIP_MOE_EXACT)
+        return moe_exact_forward(static_cast<const uint8_t *>(w_gate_up_planar), static_cast<const uint8_t *>(w_down_planar),
+                                 static_cast<const __bf16 *>(x_dev), sel_dev, wts_dev, static_cast<__bf16 *>(y_dev), T, H, I,
+                                 E, topk_i, w, s);
     const int Hp = static_cast<int>(pad128(h)), Ip = static_cast<int>(pad128(i));
 
     // Row tile.  Up to 128 rows: the smallest height that holds an expert with two standard deviations more rows
@@ -1241,9 +1083,8 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         {
             const size_t lds_bytes = moe_small_lds_bytes(Hp);
             auto kern = mx_moe_gemm_small_kernel<2, true, true>;
-            if (lds_bytes > 64 * 1024)
-                LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            static LdsOptIn opt;
+            if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
             hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((I + 63) / 64), static_cast<unsigned>(R)), dim3(256), lds_bytes, s, a1);
             LHIP_CHECK_LAUNCH();
         }
@@ -1255,9 +1096,8 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         a2.out = w.out; a2.y = static_cast<__bf16 *>(y_dev);
         {
             const size_t lds_bytes = moe_small_lds_bytes(Ip);
-            if (lds_bytes > 64 * 1024)
-                LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(mx_moe_down_direct_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            static LdsOptIn opt;
+            if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(mx_moe_down_direct_kernel), lds_bytes)) return st;
             hipLaunchKernelGGL(mx_moe_down_direct_kernel, dim3(static_cast<unsigned>(H / 16)), dim3(256), lds_bytes, s, a2);
             LHIP_CHECK_LAUNCH();
         }
@@ -1319,13 +1159,7 @@ lhip_status lhip_mxfp4_moe_bf16(const void *w_gate_up_planar, const void *w_down
         }
     }
     if (st) return st;
-    {
-        const size_t threads = static_cast<size_t>(T) * (H / 4);
-        hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, s, w.out,
-                           w.plan.slot_of, wts_dev, static_cast<__bf16 *>(y_dev), T, H, topk_i);
-        LHIP_CHECK_LAUNCH();
-    }
-    return LHIP_OK;
+    return moe_launch_combine(w.out, w.plan.slot_of, wts_dev, static_cast<__bf16 *>(y_dev), T, H, topk_i, s);
 }
 
 lhip_status lhip_mxfp4_moe_bf16_static(const void *w_gate_up_planar, const void *w_down_planar, const void *x_dev,
@@ -1341,12 +1175,21 @@ lhip_status lhip_mxfp4_moe_bf16_static(const void *w_gate_up_planar, const void 
 
 lhip_status lhip_mxfp4_moe_read_intermediates(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
                                               int64_t h, int64_t i, int64_t e, int64_t topk, void *stream) {
+    return lhip_mxfp4_moe_read_intermediates_mode(workspace_dev, act_dev, down_dev, t, h, i, e, topk, LHIP_MOE_EXACT, stream);
+}
+
+lhip_status lhip_mxfp4_moe_read_intermediates_mode(const void *workspace_dev, float *act_dev, float *down_dev, int64_t t,
+                                                   int64_t h, int64_t i, int64_t e, int64_t topk, int32_t mode,
+                                                   void *stream) {
     if (!workspace_dev) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_moe_shape(t, h, i, e, topk)) return s;
+    if (mode != LHIP_MOE_EXACT && mode != LHIP_MOE_FAST) return LHIP_ERR_UNSUPPORTED;
     if (!aligned(workspace_dev, 256) || !aligned(act_dev, 4) || !aligned(down_dev, 4)) return LHIP_ERR_MISALIGNED;
     if (!act_dev && !down_dev) return LHIP_OK;
     MoeWorkspace w = carve(const_cast<void *>(workspace_dev), t, h, i, e, topk);
     const int R = static_cast<int>(t * topk);
+    if (mode == LHIP_MOE_EXACT)
+        return moe_exact_read_intermediates(w, act_dev, down_dev, R, static_cast<int>(i), static_cast<int>(h), as_stream(stream));
     hipLaunchKernelGGL(moe_read_intermediates_kernel, dim3(static_cast<unsigned>(R)), dim3(256), 0, as_stream(stream),
                        w.plan.slot_of, w.a_hi, w.a_lo, w.a_sc, w.out, act_dev, down_dev, R, static_cast<int>(i),
                        static_cast<int>(pad128(i)), static_cast<int>(h));

@@ -342,10 +342,8 @@ static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void 
     if (static_cast<int64_t>(m_tiles) * n_tiles_pad > 0x7fffffff) return LHIP_ERR_INVALID_SHAPE;  // the grid's x extent
     const size_t lds_bytes = 2 * (static_cast<size_t>(BM + BN) * kRowBytes + static_cast<size_t>(BN) * 8);
     auto kern = q8_gemm_bf16_kernel<BM, BN, WM, WN, D, OutT>;
-    if (lds_bytes > 64 * 1024) {
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-    }
+    static LdsOptIn opt;
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
     const int kt_slice = slices > 1 ? (k / kBK + slices - 1) / slices : 0;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad), static_cast<unsigned>(slices)),
                        dim3(WM * WN * 64), lds_bytes, s, qs, ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m,

@@ -447,9 +447,8 @@ static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const XT *x, 
                                int k, int splits, int passes, hipStream_t s) {
     auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, XT>;
     constexpr size_t lds_bytes = SkShape<MT, sk_limbs<XT>()>::LDS;
-    if (lds_bytes > 64 * 1024)  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds_bytes)));
+    static LdsOptIn opt;  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
     const int units = k / kSkUnit, per = (units + splits - 1) / splits;
     hipLaunchKernelGGL(kern,
                        dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits),

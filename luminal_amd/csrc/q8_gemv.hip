@@ -368,9 +368,10 @@ static lhip_status launch_fused(const GemvGroup &p, const GemvFuse &f, const flo
     const int cap = kNumCUs * blocks_per_cu;
     if (grid > cap) grid = cap;
     const size_t lds_bytes = static_cast<size_t>(k) * sizeof(float);
-    if (lds_bytes + W * sizeof(float) > 64 * 1024)  // with the static reduction array: beyond the default limit (K = 16384)
-        LHIP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_fused_kernel<R, S, W, NORM, EPI>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+    static LdsOptIn opt;  // with the static reduction array: beyond the default limit (K = 16384)
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(q8_gemv_fused_kernel<R, S, W, NORM, EPI>), lds_bytes,
+                                    lds_bytes + W * sizeof(float) > 64 * 1024))
+        return st;
     hipLaunchKernelGGL((q8_gemv_fused_kernel<R, S, W, NORM, EPI>), dim3(static_cast<unsigned>(grid)), dim3(W * 64),
                        lds_bytes, s, p, f, x, k, n_groups);
     LHIP_CHECK_LAUNCH();

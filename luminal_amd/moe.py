@@ -45,6 +45,15 @@ class Mxfp4Weight:
                        "lhip_mxfp4_unpack")
         return raw
 
+    def dequantize_bf16(self) -> torch.Tensor:
+        """The weight as the bf16 numbers the exact expert GEMMs multiply (lhip_mxfp4_dequant_bf16)."""
+        lib = capi.load_library()
+        out = torch.empty((self.n, self.k), dtype=torch.bfloat16, device=self.planar.device)
+        with torch.cuda.device(out.device):
+            capi.check(lib.lhip_mxfp4_dequant_bf16(self.planar.data_ptr(), out.data_ptr(), self.n, self.k, _stream()),
+                       "lhip_mxfp4_dequant_bf16")
+        return out
+
     def dequantize(self) -> torch.Tensor:
         lib = capi.load_library()
         out = torch.empty((self.n, self.k), dtype=torch.float32, device=self.planar.device)
@@ -76,7 +85,9 @@ class MoEExperts:
         self.gu, self.dn, self.e, self.h, self.i = w_gate_up, w_down, experts, hidden, inter
         self._ws = None
 
-    def process(self, x: torch.Tensor, sel: torch.Tensor, wts: torch.Tensor) -> torch.Tensor:
+    def process(self, x: torch.Tensor, sel: torch.Tensor, wts: torch.Tensor, mode: int = capi.LHIP_MOE_EXACT) -> torch.Tensor:
+        """mode: capi.LHIP_MOE_EXACT (bf16 matrix instruction on exactly expanded weights, the default) or
+        capi.LHIP_MOE_FAST (block-scaled fp4 x fp8 instruction)."""
         lib = capi.load_library()
         if x.dtype != torch.bfloat16 or not x.is_cuda:
             raise TypeError("MoEExperts expects bf16 activations on the GPU")
@@ -90,23 +101,23 @@ class MoEExperts:
             self._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
         y = torch.empty((t, self.h), dtype=torch.bfloat16, device=x.device)
         with torch.cuda.device(x.device):
-            st = lib.lhip_mxfp4_moe_bf16(self.gu.planar.data_ptr(), self.dn.planar.data_ptr(), x.data_ptr(),
-                                         sel.contiguous().data_ptr(), wts.contiguous().data_ptr(), y.data_ptr(), t,
-                                         self.h, self.i, self.e, topk, self._ws.data_ptr(), _stream())
-        capi.check(st, "lhip_mxfp4_moe_bf16")
-        self._last = (t, topk)
+            st = lib.lhip_mxfp4_moe_bf16_mode(self.gu.planar.data_ptr(), self.dn.planar.data_ptr(), x.data_ptr(),
+                                              sel.contiguous().data_ptr(), wts.contiguous().data_ptr(), y.data_ptr(), t,
+                                              self.h, self.i, self.e, topk, mode, self._ws.data_ptr(), _stream())
+        capi.check(st, "lhip_mxfp4_moe_bf16_mode")
+        self._last = (t, topk, mode)
         return y
 
     def intermediates(self):
         """(act (T*topk, I) f32, down (T*topk, H) f32) of the last `process` call: the SwiGLU activations as the down
         projection consumed them and every routed entry's down projection (lhip_mxfp4_moe_read_intermediates)."""
         lib = capi.load_library()
-        t, topk = self._last
+        t, topk, mode = self._last
         dev = self._ws.device
         act = torch.empty((t * topk, self.i), dtype=torch.float32, device=dev)
         down = torch.empty((t * topk, self.h), dtype=torch.float32, device=dev)
         with torch.cuda.device(dev):
-            st = lib.lhip_mxfp4_moe_read_intermediates(self._ws.data_ptr(), act.data_ptr(), down.data_ptr(), t, self.h,
-                                                       self.i, self.e, topk, _stream())
-        capi.check(st, "lhip_mxfp4_moe_read_intermediates")
+            st = lib.lhip_mxfp4_moe_read_intermediates_mode(self._ws.data_ptr(), act.data_ptr(), down.data_ptr(), t,
+                                                            self.h, self.i, self.e, topk, mode, _stream())
+        capi.check(st, "lhip_mxfp4_moe_read_intermediates_mode")
         return act, down

@@ -34,6 +34,20 @@ def test_static_workspace_entry_point_equals_the_workspace_one():
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), t
         assert bool(torch.isfinite(got.float()).all()) and float(got.float().abs().max()) > 0
+    # the two-launch direct form for at most four routed rows (batch-1 decode, what the entry point is aimed at): one
+    # token with top-4 and two tokens with top-2, each with one routed entry that names no expert (its activation
+    # rows in the scratch array are never written and must not be used)
+    for t, k in ((1, 4), (2, 2)):
+        x = torch.from_numpy(rng.standard_normal((t, h)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+        sel, wts = route_topk(torch.from_numpy(rng.standard_normal((t, e)).astype(np.float32)).to(DEV), k)
+        sel[0, 1] = e + 3
+        want = layer.process(x, sel, wts)
+        got = torch.full((t, h), 7.0, dtype=torch.bfloat16, device=DEV)
+        capi.check(lib.lhip_mxfp4_moe_bf16_static(gu.planar.data_ptr(), dn.planar.data_ptr(), x.data_ptr(), sel.data_ptr(),
+                                                  wts.data_ptr(), got.data_ptr(), t, h, i, e, k, st), "static")
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (t, k)
+        assert bool(torch.isfinite(got.float()).all()) and float(got.float().abs().max()) > 0
     # beyond the scratch array: refused, nothing launched
     big_t = 4096
     assert lib.lhip_mxfp4_moe_workspace_nbytes(big_t, h, i, e, topk) > 8 << 20
