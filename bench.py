@@ -418,12 +418,13 @@ def bench_moe(args, cpu_seconds=None):
             routes.append(route_topk(logits, K4))
         cases[T] = (x, routes)
     it = [0]
+    modes = {"exact": capi.LHIP_MOE_EXACT, "fast": capi.LHIP_MOE_FAST}
 
-    def run(T):
+    def run(T, mode=capi.LHIP_MOE_EXACT):
         x, routes = cases[T]
         sel, wts = routes[it[0] % 8]
         it[0] += 1
-        layer.process(x, sel, wts)
+        layer.process(x, sel, wts, mode)
 
     def step():
         for T in cases:
@@ -437,37 +438,104 @@ def bench_moe(args, cpu_seconds=None):
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    errors = _moe_strict_errors(torch, layer, cases, modes)
     per = {}
     flops_step = 0.0
     for T in cases:
-        us = _event_us(torch, lambda: run(T), 16)
         touched = E if T >= 64 else K4
         by = touched * 13219200 + 2 * 2 * T * H
         fl = T * 199065600.0
         flops_step += fl
-        per[f"T={T}"] = {"us": round(us, 1), "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
-                         "tflops": round(fl / us / 1e6, 1), "frac_mfma_fp4": round(fl / us / 1e6 / MFMA_FP4_PEAK_TFLOPS, 5),
-                         "frac_mfma_fp8_two_pass": round(2 * fl / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 5)}
-    t64, t1024 = per["T=64"], per["T=1024"]
+        for name, mode in modes.items():
+            us = _event_us(torch, lambda: run(T, mode), 16)
+            row = {"us": round(us, 1), "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
+                   "tflops": round(fl / us / 1e6, 1), "strict_err": errors[(T, name)]}
+            if name == "exact":  # one bf16 x bf16 product per multiply-add
+                row["frac_mfma_bf16"] = round(fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 5)
+            else:                # two fp8 x fp4 products per multiply-add
+                row["frac_mfma_fp4"] = round(fl / us / 1e6 / MFMA_FP4_PEAK_TFLOPS, 5)
+                row["frac_mfma_fp8_two_pass"] = round(2 * fl / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 5)
+            per[f"T={T} {name}"] = row
+    t64, t1024, f1024 = per["T=64 exact"], per["T=1024 exact"], per["T=1024 fast"]
     out = {
         "metric": "MXFP4 MoE expert layer (H=I=2880, 32 experts, top-4): GB/s and TFLOP/s, 1 GPU",
         "value": round(flops_step / (wall / args.steps) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp4 (e2m1, e8m0 block scales) weights x bf16 activations split exactly into two fp8 operands, "
-                 "f32 accumulate on v_mfma_scale_f32_16x16x128_f8f6f4, bf16 out",
-        "data": "synthetic", "config": {"workload": "gpt_oss_style_mxfp4_moe_layer", "tokens": [1, 64, 1024]},
+        "dtype": "default (exact): fp4 (e2m1, e8m0 block scales) weights expanded exactly to bf16 x bf16 activations, f32 "
+                 "accumulate on v_mfma_f32_16x16x32_bf16, bf16 out; fast: raw fp4 x two fp8 halves of each activation on "
+                 "v_mfma_scale_f32_16x16x128_f8f6f4",
+        "data": "synthetic", "config": {"workload": "gpt_oss_style_mxfp4_moe_layer", "tokens": [1, 64, 1024],
+                                        "modes": "value and roofline are the default (exact) mode; per_tokens has both"},
         "per_tokens": per,
-        "roofline": {"bound": "hbm", "kernel": "whole layer at T=64 (plan + quantise, 2 grouped GEMMs, combine)",
+        "strict_err_legend": "max |y-t| / max(|t|, 1e-3 rms(t)) against f64 on sampled tokens: act = SwiGLU activations "
+                             "(bf16) vs f64 of x; down = f32 down rows vs f64 of the activations the GPU produced; "
+                             "y_given_act = layer output vs f64 down projection + weighted sum of those activations; "
+                             "y_independent = layer output vs f64 with the intermediate rounded to bf16 on its own "
+                             "(differs wherever an activation lies within rounding error of a bf16 boundary)",
+        "roofline": {"bound": "hbm", "kernel": "whole layer at T=64, exact mode (plan, 2 grouped GEMMs, combine)",
                      "achieved": t64["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": t64["frac_hbm"],
                      "traffic": TRAFFIC["moe_t64"][0], "traffic_source": TRAFFIC["moe_t64"][1]},
-        "roofline_t1024_mfma": {"bound": "mfma", "kernel": "whole layer at T=1024",
-                                "achieved": t1024["tflops"], "peak": MFMA_FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                "frac": t1024["frac_mfma_fp4"], "frac_of_fp8_two_pass": t1024["frac_mfma_fp8_two_pass"],
-                                "traffic": None}}
+        "roofline_t1024_mfma": {"bound": "mfma", "kernel": "whole layer at T=1024, exact mode (bf16 matrix instruction)",
+                                "achieved": t1024["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                "frac": t1024["frac_mfma_bf16"], "traffic": None},
+        "roofline_t1024_mfma_fast": {"bound": "mfma", "kernel": "whole layer at T=1024, fast mode (block-scaled fp8 x fp4)",
+                                     "achieved": f1024["tflops"], "peak": MFMA_FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": f1024["frac_mfma_fp4"], "frac_of_fp8_two_pass": f1024["frac_mfma_fp8_two_pass"],
+                                     "traffic": None}}
     if cpu_seconds:
         out["cpu_baseline"] = cpu_baseline_moe(cpu_seconds)
     del layer, cases
+    torch.cuda.empty_cache()
+    return out
+
+
+def _moe_strict_errors(torch, layer, cases, modes, n_tokens=3):
+    """The layer's strict element-wise error per T and mode, each matmul against f64 arithmetic of its own inputs
+    (torch on the device; weights through lhip_mxfp4_dequant_f32, whose values are tested bit-exact) on a few tokens."""
+    e, h, i = layer.e, layer.h, layer.i
+    w_gu = layer.gu.dequantize().view(e, 2 * i, h)
+    w_dn = layer.dn.dequantize().view(e, h, i)
+
+    def rel(y, t):
+        y, t = y.double().reshape(-1), t.double().reshape(-1)
+        floor = 1e-3 * float(t.pow(2).mean().sqrt()) + 1e-300
+        return float(((y - t).abs() / t.abs().clamp_min(floor)).max())
+
+    out = {}
+    for T, (x, routes) in cases.items():
+        sel, wts = routes[0]
+        topk = sel.shape[1]
+        toks = sorted({0, T - 1, T // 2})[:n_tokens]
+        for name, mode in modes.items():
+            y = layer.process(x, sel, wts, mode)
+            act_g, down_g = layer.intermediates()
+            want_act, got_act, want_down, got_down, y_given, y_indep = [], [], [], [], [], []
+            for t in toks:
+                yg = torch.zeros(h, dtype=torch.float64, device=x.device)
+                yi = torch.zeros(h, dtype=torch.float64, device=x.device)
+                for s_ in range(topk):
+                    ex = int(sel[t, s_])
+                    r = t * topk + s_
+                    gu = w_gu[ex].double() @ x[t].double()
+                    g, u = gu[:i], gu[i:]
+                    a = u * (g / (1.0 + torch.exp(-g)))
+                    want_act.append(a)
+                    got_act.append(act_g[r])
+                    wd = w_dn[ex].double()
+                    d_own = wd @ act_g[r].double()
+                    want_down.append(d_own)
+                    got_down.append(down_g[r])
+                    yg += float(wts[t, s_]) * d_own
+                    yi += float(wts[t, s_]) * (wd @ a.float().to(torch.bfloat16).double())
+                y_given.append(yg)
+                y_indep.append(yi)
+            yt = torch.stack([y[t] for t in toks])
+            out[(T, name)] = {"act": float(f"{rel(torch.stack(got_act), torch.stack(want_act)):.3g}"),
+                              "down": float(f"{rel(torch.stack(got_down), torch.stack(want_down)):.3g}"),
+                              "y_given_act": float(f"{rel(yt, torch.stack(y_given)):.3g}"),
+                              "y_independent": float(f"{rel(yt, torch.stack(y_indep)):.3g}")}
+    del w_gu, w_dn
     torch.cuda.empty_cache()
     return out
 
