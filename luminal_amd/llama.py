@@ -328,13 +328,18 @@ class LlamaQ8:
         """Greedy decode of `steps` tokens after a prefill; returns the token ids (first = the prefill's pick)."""
         self._room(steps)
         out = torch.empty(steps, dtype=torch.int32, device=self.dev)
+        # Capturing the graph runs two real steps first (a warm-up and the captured one), which append K/V rows at
+        # pos and pos + 1 before the position is put back: with fewer than two free positions the steps that still
+        # fit run eagerly instead.
+        if use_graph and self._graph is None and self._pos_host + 2 > self.max_seq:
+            use_graph = False
         if not use_graph:
             for i in range(steps):
                 out[i:i + 1].copy_(self.tok_i)
                 self.decode_step()
+            self._check_program()
             return out
         if self._graph is None:
-            self._room(2)  # the warm-up step and the captured one
             pos0, tok0, toki0, host0 = self.pos.clone(), self.tok.clone(), self.tok_i.clone(), self._pos_host
             st = torch.cuda.Stream(device=self.dev)
             st.wait_stream(torch.cuda.current_stream())
@@ -355,7 +360,15 @@ class LlamaQ8:
             out[i:i + 1].copy_(self.tok_i)
             self._graph.replay()
         self._pos_host += steps
+        self._check_program()
         return out
+
+    def _check_program(self):
+        """With the persistent decode program, a grid-wide wait that gave up leaves the step's results meaningless by
+        design; ask (this synchronises the device) before the tokens are handed back."""
+        if self._program is not None and self._program.timed_out():
+            raise capi.LhipError(capi.LHIP_ERR_HIP, "LlamaQ8.decode",
+                                 "the persistent decode program gave up a wait: the tokens of this call are not valid")
 
 
 def fuse_rows(*raws: np.ndarray) -> np.ndarray:

@@ -656,3 +656,20 @@ def test_running_past_max_seq_is_refused_on_the_host(oracle):
     with pytest.raises(capi.LhipError):
         eng.decode(6, use_graph=False)
     assert eng.decode(5, use_graph=False).numel() == 5
+
+
+def test_decode_of_the_last_free_position(oracle):
+    """A decode of exactly the last free cache position fits and is not refused: capturing the graph needs two free
+    positions (its warm-up and captured steps write real K/V rows), so with fewer the steps run eagerly; one step
+    more is refused on the host."""
+    cfg = LlamaConfig(vocab=512, dim=1024, layers=2, q_heads=8, kv_heads=2, ffn=1024)
+    eng, _ = build_model(oracle, cfg, seed=9, max_seq=6)
+    eng.prefill([1, 2, 3, 4, 5])
+    toks = eng.decode(1, use_graph=True).cpu().numpy()
+    assert toks.shape == (1,) and eng._pos_host == 6 and int(eng.pos.item()) == 6
+    with pytest.raises(capi.LhipError):
+        eng.decode(1, use_graph=True)
+    # the same tokens as a roomier engine picks
+    eng2, _ = build_model(oracle, cfg, seed=9, max_seq=32)
+    eng2.prefill([1, 2, 3, 4, 5])
+    assert np.array_equal(eng2.decode(1, use_graph=True).cpu().numpy(), toks)
