@@ -32,6 +32,7 @@
 // the grid is one workgroup per compute unit, which the register and LDS budget of the kernel guarantees.
 #include <hip/hip_fp16.h>
 #include <limits.h>
+#include <algorithm>
 
 #include <new>
 #include <vector>
@@ -71,6 +72,7 @@ struct ProgOp {
     const float *norm_w;
     const float *residual;     // EPI_ADD: read when res_t is null
     const tagged_t *res_t;     // shadow of the residual when an earlier phase of the launch wrote it
+    int res_phase;             // ... and that phase (its tag is expected on the shadow's words)
     float *k_cache, *v_cache;
 };
 
@@ -85,6 +87,7 @@ struct Buf8 {
     u32x4 q[kProgSlots];
     unsigned d[kProgSlots];  // f16 scale code, zero-extended
     float res;               // EPI_ADD: residual of the step's row (lane < r)
+    unsigned res_tag;        // ... and the tag its word carried when it was fetched (see matvec_phase)
 };
 
 // One pipeline step of weights: slot i = slice (i / r), row (i % r).  Every step issues the same number of loads
@@ -181,25 +184,53 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
     const int nx = op.next_matvec;
     const StepGeom nxt = geom_of(ops[nx >= 0 ? nx : p]);
 
-    // Residuals of the first two steps' rows: requested now, together with the staging loads.  Whoever wrote
-    // them finished before this phase's input could be complete, so their tags need no look.
-    auto residual_of = [&](int g) -> float {
-        const int row = min(g * R + static_cast<int>(lane < static_cast<unsigned>(R) ? lane : 0u), n - 1);
-        if (op.res_t != nullptr)
-            return __uint_as_float(static_cast<unsigned>(
-                __hip_atomic_load(as_global(op.res_t) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
-        return as_global(op.residual)[row];
+    // Residuals of the first two steps' rows: requested now, together with the staging loads, and those of later
+    // steps with their weights.  A residual written by an earlier phase of this launch comes as a tagged word like
+    // every other hand-over.  Its writer need not have finished when the request goes out - nothing orders a phase
+    // that this phase's input does not depend on before it - so the tag travels with the value and is looked at
+    // where the value is used (settle_residual): in the usual case, the writer being the producer of an earlier
+    // input of this workgroup, it is there and the check costs a compare.
+    const unsigned res_tag_want = tag_base + static_cast<unsigned>(op.res_phase) + 1u;
+    auto residual_row = [&](int g) -> int {
+        return min(g * R + static_cast<int>(lane < static_cast<unsigned>(R) ? lane : 0u), n - 1);
+    };
+    auto load_residual = [&](Buf8 &buf, int g) {
+        const int row = residual_row(g);
+        if (op.res_t != nullptr) {
+            const tagged_t raw = __hip_atomic_load(as_global(op.res_t) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            buf.res = __uint_as_float(static_cast<unsigned>(raw));
+            buf.res_tag = static_cast<unsigned>(raw >> 32);
+        } else {
+            buf.res = as_global(op.residual)[row];
+            buf.res_tag = res_tag_want;
+        }
+    };
+    // The residual of row group g as fetched into buf, or - when its word did not carry the writer's tag yet -
+    // fetched again until it does (bounded like every wait of the program).
+    auto settle_residual = [&](const Buf8 &buf, int g) -> float {
+        float v = buf.res;
+        if (op.res_t == nullptr) return v;
+        bool ok = buf.res_tag == res_tag_want;
+        while (io.again(__all(ok))) {
+            const tagged_t raw = __hip_atomic_load(as_global(op.res_t) + residual_row(g), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            v = __uint_as_float(static_cast<unsigned>(raw));
+            ok = static_cast<unsigned>(raw >> 32) == res_tag_want;
+        }
+        return v;
     };
     if (epi == EPI_ADD) {
-        a.res = residual_of(T > 0 ? w.wave_global : 0);
-        b.res = residual_of(T > 1 ? w.wave_global + (chunks == 1 ? w.total_waves : 0) : 0);
+        load_residual(a, T > 0 ? w.wave_global : 0);
+        load_residual(b, T > 1 ? w.wave_global + (chunks == 1 ? w.total_waves : 0) : 0);
     }
 
     // ---- activations to LDS: float4 index slice*256 + j*64 + lane holds x[slice*1024 + lane*16 + j*4 .. +3].
     // A thread fetches up to 7 float4 per round and, when they come from an earlier phase, repeats the round
     // until every word carries that phase's tag.  With the norm, x * gain is staged and the sum of squares is
     // taken on the way by the first 256 threads in increasing index, the order of a four-wave workgroup.
-    {
+    // A workgroup none of whose waves has a row group in this phase stages nothing: it is then no reader of the
+    // phase's input at all, which the host's rule for overwriting a buffer relies on (lhip_decode_program_create).
+    if (static_cast<int>(blockIdx.x) * kProgWaves < n_groups) {
         constexpr int kBatch = 7;  // K = 14336 over 512 threads in one round
         const float4 *x4 = reinterpret_cast<const float4 *>(op.x);
         const float4 *g4 = reinterpret_cast<const float4 *>(op.norm_w);
@@ -329,12 +360,12 @@ __device__ __forceinline__ void matvec_phase(const ProgOp *__restrict__ ops, int
     };
     auto compute = [&](Buf8 &cur) {
         compute8(cur, xs4, c * S, R, S, lane, acc0, acc1);
-        if (c == chunks - 1) finish_group(g, cur.res);
+        if (c == chunks - 1) finish_group(g, epi == EPI_ADD ? settle_residual(cur, g) : 0.f);
         next(g, c);
     };
     auto refill = [&](Buf8 &cur, bool live) {  // with the step (g2, c2) of this phase
         __builtin_amdgcn_sched_barrier(0);
-        if (epi == EPI_ADD) cur.res = residual_of(live ? g2 : 0);
+        if (epi == EPI_ADD) load_residual(cur, live ? g2 : 0);
         load8(cur, op.qs, op.ds, g2 * R, n, k, c2 * S, R, S, lane, live);
         next(g2, c2);
         __builtin_amdgcn_sched_barrier(0);
@@ -484,9 +515,9 @@ static bool prog_attention_supported(int64_t g, int64_t hd) {
 // What the host knows about a caller's buffer while it lays the phases out.
 struct BufferState {
     const void *base;
-    size_t shadow_offset;  // in words, into the shadow allocation
-    int writer;            // phase that wrote the current contents, -1: the caller
-    int last_reader;       // latest phase that reads the current contents (-1: none)
+    size_t shadow_offset;      // in words, into the shadow allocation
+    int writer;                // phase that wrote the current contents, -1: the caller
+    std::vector<int> readers;  // phases that read the current contents
 };
 
 }  // namespace lhip
@@ -536,31 +567,46 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
     auto note_read = [&](const void *base, int reader, bool own, size_t *offset) -> int {
         BufferState *b = find(base);
         if (!b) {
-            buffers.push_back(BufferState{base, SIZE_MAX, -1, own ? -1 : reader});
+            buffers.push_back(BufferState{base, SIZE_MAX, -1, {}});
+            if (!own) buffers.back().readers.push_back(reader);
             return -1;
         }
-        if (!own && reader > b->last_reader) b->last_reader = reader;
+        if (!own) b->readers.push_back(reader);
         *offset = b->shadow_offset;
         return b->writer;
     };
     // A write of `words` values to `base` by phase `writer` whose own input comes from phase `input_phase`.
-    // A workgroup that writes has seen the whole output of `input_phase`: every workgroup has therefore begun
-    // that phase's arithmetic, i.e. has finished the reads of every phase up to it, and (a wave waits for its
-    // stores to be acknowledged before it stores for a later phase) the stores of every phase up to it have
-    // landed.  So the old contents may go if their writer and all their readers are phases <= input_phase.
+    // A workgroup that writes has seen the whole output of `input_phase`, so every workgroup that works in that
+    // phase has finished reading its input, has finished every earlier phase it works in (a workgroup takes the
+    // phases in order) and (a wave waits for its stores to be acknowledged before it stores for a later phase)
+    // has seen every store it issued up to then land; the same holds, step by step, for the phase that produced
+    // that input, and so on back along the chain of inputs.  The workgroups that work in a phase are the first
+    // workers[phase] of the grid, and one that does not work in a phase does not read its input either.  So a
+    // phase r that read or wrote the old contents is known to be done with them if it lies on that chain, or if
+    // some later phase on the chain employs at least as many workgroups as r does; anything else (a phase the
+    // writer's input does not depend on may still be running somewhere) is refused.
+    std::vector<ProgOp> phases;
+    std::vector<int> workers;
+    auto settled = [&](int phase, int from) -> bool {
+        for (int q = from; q >= phase; q = phases[static_cast<size_t>(q)].x_phase)
+            if (q == phase || workers[static_cast<size_t>(q)] >= workers[static_cast<size_t>(phase)]) return true;
+        return false;
+    };
     auto note_write = [&](const void *base, size_t words, int writer, int input_phase, size_t *offset) -> bool {
         BufferState *b = find(base);
         if (!b) {
-            buffers.push_back(BufferState{base, SIZE_MAX, -1, -1});
+            buffers.push_back(BufferState{base, SIZE_MAX, -1, {}});
             b = &buffers.back();
         }
-        if (b->last_reader > input_phase || b->writer > input_phase) return false;
+        if (b->writer >= 0 && !settled(b->writer, input_phase)) return false;
+        for (int r : b->readers)
+            if (r != writer && !settled(r, input_phase)) return false;
         if (b->shadow_offset == SIZE_MAX) {
             b->shadow_offset = shadow_words;
             shadow_words += (words + 31) & ~size_t{31};
         }
         b->writer = writer;
-        b->last_reader = -1;
+        b->readers.clear();
         *offset = b->shadow_offset;
         return true;
     };
@@ -568,7 +614,6 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
     struct Pending {  // offsets are turned into pointers once the shadow allocation exists
         size_t x = SIZE_MAX, y = SIZE_MAX, res = SIZE_MAX;
     };
-    std::vector<ProgOp> phases;
     std::vector<Pending> pend;
     size_t max_k = 0;
     size_t ws_ml_off = SIZE_MAX, ws_acc_off = SIZE_MAX;
@@ -618,11 +663,13 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
             ph.norm_w = o.norm_weight;
             ph.residual = o.epilogue == LHIP_FUSE_ADD ? o.residual : nullptr;
             ph.x_phase = note_read(o.x, p, false, &pe.x);
-            if (ph.residual && note_read(ph.residual, p, ph.residual == o.y, &pe.res) < 0) pe.res = SIZE_MAX;
+            ph.res_phase = ph.residual ? note_read(ph.residual, p, ph.residual == o.y, &pe.res) : -1;
+            if (ph.res_phase < 0) pe.res = SIZE_MAX;
             const size_t out_words = static_cast<size_t>(o.epilogue == LHIP_FUSE_SWIGLU ? o.n / 2 : o.n);
             if (!note_write(o.y, out_words, p, ph.x_phase, &pe.y)) return LHIP_ERR_UNSUPPORTED;
             max_k = o.k > static_cast<int64_t>(max_k) ? static_cast<size_t>(o.k) : max_k;
             phases.push_back(ph);
+            workers.push_back(std::min(grid, (ph.n_groups + kProgWaves - 1) / kProgWaves));
             pend.push_back(pe);
         } else if (o.type == LHIP_DECODE_ATTENTION) {
             if (!o.x || !o.y || !o.k_cache || !o.v_cache) return LHIP_ERR_NULL_PTR;
@@ -636,8 +683,9 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
             ph.x_phase = note_read(o.x, p, false, &pe.x);
             // the body reads its input through the tagged accessors: it must come from a phase of this program
             if (ph.x_phase < 0) return LHIP_ERR_UNSUPPORTED;
-            if (ws_last_reader > ph.x_phase) return LHIP_ERR_UNSUPPORTED;  // the previous merge may still be reading
+            if (ws_last_reader >= 0 && !settled(ws_last_reader, ph.x_phase)) return LHIP_ERR_UNSUPPORTED;  // the previous merge may still be reading
             phases.push_back(ph);
+            workers.push_back(std::min(grid, static_cast<int>(kv_heads) * splits));
             pend.push_back(pe);
             ProgOp m{};
             Pending pm;
@@ -648,6 +696,7 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
             ws_last_reader = p + 1;
             if (!note_write(o.y, static_cast<size_t>(q_heads * head_dim), p + 1, p, &pm.y)) return LHIP_ERR_UNSUPPORTED;
             phases.push_back(m);
+            workers.push_back(std::min(grid, static_cast<int>(q_heads)));
             pend.push_back(pm);
         } else {
             return LHIP_ERR_INVALID_SHAPE;

@@ -176,3 +176,62 @@ def test_create_argument_errors():
     assert handle.value is None
     assert lib.lhip_decode_program_run(None, None) == capi.LHIP_ERR_NULL_PTR
     assert lib.lhip_decode_program_destroy(None) == capi.LHIP_OK
+
+
+@pytest.mark.parametrize("same_input", [False, True], ids=["independent_input", "input_is_the_residual"])
+def test_residual_produced_by_a_phase_the_input_does_not_depend_on(same_input):
+    """y1 = W1 x, then y2 = W2 z + y1 with z written before the launch (or z = y1): nothing orders phase 0 before the
+    moment phase 1 requests its residual rows, so the residual has to travel as tagged words and be waited for like
+    an input.  Small n: most workgroups have no row group and run ahead.  Bit-equal to the two fused launches, on
+    several runs (each launch has tags of its own)."""
+    d = 1024
+    w1, w2 = weight(d, d, 41), weight(d, d, 42)
+    torch.manual_seed(5)
+    x, z = torch.randn(d, device=DEV), torch.randn(d, device=DEV)
+    pos = torch.zeros(1, dtype=torch.int32, device=DEV)
+    y1_ref, y2_ref = torch.empty(d, device=DEV), torch.empty(d, device=DEV)
+    y1, y2 = torch.full((d,), float("nan"), device=DEV), torch.full((d,), float("nan"), device=DEV)
+    prog = DecodeProgram(pos=pos).matvec(w1, x, y1)
+    prog.matvec(w2, y1 if same_input else z, y2, residual=y1, epilogue=FusedMatvec.EPI_ADD).build()
+    for run in range(4):
+        x.normal_()
+        FusedMatvec([w1], [y1_ref]).run(x)
+        FusedMatvec([w2], [y2_ref], residual=y1_ref, epilogue=FusedMatvec.EPI_ADD).run(y1_ref if same_input else z)
+        prog.run()
+        torch.cuda.synchronize()
+        assert not prog.timed_out()
+        assert torch.equal(bits(y1), bits(y1_ref)) and torch.equal(bits(y2), bits(y2_ref)), run
+
+
+def test_overwrite_is_refused_unless_its_readers_are_known_to_be_done():
+    """A buffer may be overwritten by a phase only if every phase that read or wrote its old contents either is an
+    ancestor of the overwriting phase's input or is followed, on that chain of inputs, by a phase that employs at
+    least as many workgroups (a workgroup takes the phases in order): any other phase may still be running in some
+    workgroup."""
+    d = 1024
+    w, w_tall = weight(d, d, 43), weight(4 * d, d, 44)
+    pos = torch.zeros(1, dtype=torch.int32, device=DEV)
+    a, c, e = (torch.zeros(d, device=DEV) for _ in range(3))
+    b4 = torch.zeros(4 * d, device=DEV)
+    # phase 0: a -> b4 on every workgroup of the grid; phase 1: a (before the launch) -> c on half of them; phase 2
+    # reads c and overwrites b4.  The old writer, phase 0, is no ancestor of phase 2's input (c <- phase 1 <- a) and
+    # phase 1 employs fewer workgroups than phase 0: some of phase 0's may still be storing.  Refused.
+    prog = DecodeProgram(pos=pos).matvec(w_tall, a, b4).matvec(w, a, c).matvec(w_tall, c, b4)
+    with pytest.raises(capi.LhipError) as err:
+        prog.build()
+    assert err.value.status == capi.LHIP_ERR_UNSUPPORTED
+    # phase 0: a -> b; phase 1: b -> c; phase 2: c -> e; phase 3 reads e and overwrites b: reader (1) and writer (0)
+    # of the old b are ancestors of phase 3's input.  Accepted, and equal to the fused launches.
+    b = torch.zeros(d, device=DEV)
+    torch.manual_seed(6)
+    a.normal_()
+    prog = DecodeProgram(pos=pos).matvec(w, a, b).matvec(w, b, c).matvec(w, c, e).matvec(w, e, b).build()
+    prog.run()
+    torch.cuda.synchronize()
+    assert not prog.timed_out()
+    rb, rc, re_, rb2 = (torch.empty(d, device=DEV) for _ in range(4))
+    FusedMatvec([w], [rb]).run(a)
+    FusedMatvec([w], [rc]).run(rb)
+    FusedMatvec([w], [re_]).run(rc)
+    FusedMatvec([w], [rb2]).run(re_)
+    assert torch.equal(bits(b), bits(rb2)) and torch.equal(bits(c), bits(rc)) and torch.equal(bits(e), bits(re_))
