@@ -46,7 +46,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode_projection_set",
-                    choices=["decode_projection_set", "prefill_gemm", "moe", "rows_f32"],
+                    choices=["decode_projection_set", "prefill_gemm", "moe", "rows_f32", "issue_rates"],
                     help="decode_projection_set (default, the headline metric), prefill_gemm (the Q8_0 prefill GEMM set), "
                          "moe (the MXFP4 expert layer)")
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
@@ -138,6 +138,53 @@ def _event_us(torch, fn, reps):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def bench_issue_rates(args):
+    """Issue rates of the matrix instructions the GEMMs use and of the fp4 -> bf16 conversion: register-only loops
+    (lhip_issue_rate_probe), one and two waves per SIMD; cycles per instruction from the kernel's own cycle counter,
+    the shader clock from that counter against the 100 MHz wall clock, TFLOP/s from HIP events."""
+    import torch
+
+    from luminal_amd import capi
+
+    lib = capi.load_library()
+    dev = torch.device("cuda:0")
+    capi.check(lib.lhip_init(0), "lhip_init")
+    stream = torch.cuda.current_stream().cuda_stream
+    kinds = [("v_mfma_f32_32x32x16_bf16", 0, 4, 2 * 32 * 32 * 16), ("v_mfma_f32_16x16x32_bf16", 1, 8, 2 * 16 * 16 * 32),
+             ("v_mfma_scale_f32_16x16x128_f8f6f4 fp8 x fp8", 2, 8, 2 * 16 * 16 * 128),
+             ("v_mfma_scale_f32_16x16x128_f8f6f4 fp8 x fp4", 3, 8, 2 * 16 * 16 * 128),
+             ("v_mfma_scale_f32_16x16x128_f8f6f4 fp4 x fp4", 4, 8, 2 * 16 * 16 * 128),
+             ("v_mfma_scale_f32_16x16x128_f8f6f4 fp6 x fp4", 5, 8, 2 * 16 * 16 * 128),
+             ("v_cvt_scalef32_pk_bf16_fp4", 6, 8, 0)]
+    iters = 20000
+    rows = {}
+    for name, kind, per_iter, flop in kinds:
+        for wps in (1, 2):
+            out = torch.zeros(2 * 1024 * wps, dtype=torch.int64, device=dev)
+
+            def run():
+                capi.check(lib.lhip_issue_rate_probe(kind, iters, wps, out.data_ptr(), stream), "lhip_issue_rate_probe")
+
+            us = _event_us(torch, run, 3)
+            torch.cuda.synchronize()
+            o = out.view(-1, 2).double()
+            cycles, ticks = float(o[:, 0].median()), float(o[:, 1].median())
+            n_inst = iters * per_iter  # per wave
+            clock_ghz = cycles / ticks * 0.1
+            # a SIMD's instruction stream is the wps waves' together: the launch's duration in shader cycles over the
+            # instructions the SIMD issued (the launch overhead of ~2 us in ~1 ms is inside the figure)
+            row = {"cycles_per_instruction_per_simd": round(us * 1e3 * clock_ghz / (n_inst * wps), 2),
+                   "one_wave_cycles_per_own_instruction": round(cycles / n_inst, 2),
+                   "shader_clock_ghz": round(clock_ghz, 3), "launch_us": round(us, 1)}
+            if flop:
+                row["tflops"] = round(1024.0 * wps * n_inst * flop / us / 1e6, 1)
+            rows[f"{name}, {wps} wave(s) per SIMD"] = row
+    return {"metric": "issue rates of the matrix and conversion instructions (calibration)", "unit": "cycles per instruction per SIMD",
+            "n_gpus": 1, "data": "synthetic", "config": {"workload": "issue_rates", "iters": iters,
+                                                         "independent_instructions_per_iteration": 8},
+            "rates": rows}
 
 
 def bench_rows_f32(args):
@@ -262,8 +309,9 @@ def bench_prefill_gemm(args, cpu_seconds=None):
               "lm_head": (128256, 4096)}
     ms_list = (128, 512, 2048)
     bufs, xs, ys = {}, {}, {}
+    rotate_bytes = 512 << 20  # twice the 256 MB last-level cache: every launch of a rotation streams from HBM
     for nm, (n, k) in shapes.items():
-        nbuf = 1 if nm == "lm_head" else 4
+        nbuf = max(1, -(-rotate_bytes // (n * k * 34 // 32)))
         bufs[nm] = [make_weight(torch, lib, capi, n, k, gen, dev) for _ in range(nbuf)]
     for m in ms_list:
         for k in (4096, 14336):
@@ -312,7 +360,9 @@ def bench_prefill_gemm(args, cpu_seconds=None):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 codes as exact bf16 x bf16 activations on the matrix cores, block scales and sums in f32, bf16 out",
         "data": "synthetic",
-        "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list)},
+        "config": {"workload": "llama3_8b_q8_0_prefill_gemm_set", "m": list(ms_list),
+                   "weight_rotation": "every cell is timed over distinct weight buffers of at least 512 MB in all "
+                                      f"({', '.join(f'{nm}: {len(b)}' for nm, b in bufs.items())} buffers)"},
         "per_shape": per,
         "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> (gate/up, M=2048)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -629,6 +679,8 @@ def main():
         return print(json.dumps(bench_moe(args, None if args.no_cpu_baseline else args.cpu_seconds)))
     if args.workload == "rows_f32":
         return bench_rows_f32(args)
+    if args.workload == "issue_rates":
+        return print(json.dumps(bench_issue_rates(args)))
 
     import torch
 

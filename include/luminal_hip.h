@@ -488,6 +488,21 @@ lhip_status lhip_copy_bytes(void *dst_dev, const void *src_dev, size_t nbytes, v
  * 1024 words of out_dev (4096 bytes, 4-byte aligned). */
 lhip_status lhip_read_bytes(const void *src_dev, size_t nbytes, uint32_t *out_dev, void *stream);
 
+/* Issue-rate probe (calibration, no counterpart in the reference): a register-only loop of `iters` x 8 independent
+ * instructions of one kind on every SIMD of the device, `waves_per_simd` waves on each (256 * waves_per_simd
+ * workgroups of four waves).  Lane 0 of wave w leaves out_dev[2w] = shader-clock cycles and out_dev[2w + 1] = ticks
+ * of the 100 MHz wall clock that its loop took (out_dev: 2 * 1024 * waves_per_simd words of 64 bits).  Cycles per
+ * instruction and SIMD = cycles * waves_per_simd / (8 * iters); the shader clock under that load = cycles / ticks *
+ * 100 MHz.  These are the measured ceilings the matrix-pipe rooflines are read against. */
+#define LHIP_RATE_MFMA_BF16_32X32X16 0  /* v_mfma_f32_32x32x16_bf16 (4 accumulators of 16 registers per wave) */
+#define LHIP_RATE_MFMA_BF16_16X16X32 1  /* v_mfma_f32_16x16x32_bf16 */
+#define LHIP_RATE_MFMA_SCALE_FP8_FP8 2  /* v_mfma_scale_f32_16x16x128_f8f6f4, both operands fp8 (e4m3) */
+#define LHIP_RATE_MFMA_SCALE_FP8_FP4 3  /* ... fp8 x fp4 (e2m1) */
+#define LHIP_RATE_MFMA_SCALE_FP4_FP4 4  /* ... fp4 x fp4 */
+#define LHIP_RATE_MFMA_SCALE_FP6_FP4 5  /* ... fp6 (e2m3) x fp4 */
+#define LHIP_RATE_CVT_BF16_FP4 6        /* v_cvt_scalef32_pk_bf16_fp4 */
+lhip_status lhip_issue_rate_probe(int32_t kind, int32_t iters, int32_t waves_per_simd, uint64_t *out_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

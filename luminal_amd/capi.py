@@ -91,6 +91,7 @@ SIGNATURES = {
     "lhip_argmax_f32": (C.c_int32, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _vp]),
     "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
     "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),
+    "lhip_issue_rate_probe": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, _vp, _vp]),
 }
 
 
