@@ -250,6 +250,20 @@ lhip_status lhip_q8_0_matmul_f32_ws(const void *planar_dev, const float *x_dev, 
 lhip_status lhip_q8_0_matmul_f16_ws(const void *planar_dev, const void *x_f16_dev, void *y_f16_dev, int64_t m, int64_t n,
                                     int64_t k, void *workspace_dev, size_t workspace_nbytes, void *stream);
 
+/* The bf16 prefill GEMM with the caller's workspace: lhip_q8_0_matmul_bf16 (out_form LHIP_GEMM_OUT_BF16),
+ * _bf16_f32out (LHIP_GEMM_OUT_F32) and _bf16_swiglu (LHIP_GEMM_OUT_SWIGLU) keep the partial planes of their K-sliced
+ * plans in the same per-device scratch array as the operators above and share its constraint.  This form touches no
+ * shared state: workspace_dev of lhip_q8_0_matmul_bf16_workspace_nbytes(m, n, k, out_form) bytes (256-byte aligned;
+ * 0: none is needed, NULL is fine) gives the plan, and the bits, of the plain call; a smaller one, or NULL, means fewer
+ * or no K slices (same accuracy, last bits may differ, short-and-small products leave compute units idle).  No
+ * counterpart in the reference (it has no bf16 operator). */
+#define LHIP_GEMM_OUT_BF16 0
+#define LHIP_GEMM_OUT_F32 1
+#define LHIP_GEMM_OUT_SWIGLU 2
+size_t lhip_q8_0_matmul_bf16_workspace_nbytes(int64_t m, int64_t n, int64_t k, int32_t out_form);
+lhip_status lhip_q8_0_matmul_bf16_ws(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
+                                     int32_t out_form, void *workspace_dev, size_t workspace_nbytes, void *stream);
+
 /* ---- MXFP4 weights and the mixture-of-experts layer -------------------------
  * No counterpart in the reference (it has no MXFP4 and no MoE op); built to its
  * conventions: exact dequantisation, then f32-accumulated matmul
@@ -477,6 +491,10 @@ lhip_status lhip_add_f32(float *x_dev, const float *y_dev, int64_t n, void *stre
  * array the library owns, one per device: picks that overlap in time on one device (two streams) race for it. */
 lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
                             int32_t advance, void *stream);
+/* lhip_argmax_f32 with the caller's workspace (512 bytes, 8-byte aligned) in place of the library's per-device array
+ * of partial picks: re-entrant across streams.  Same result. */
+lhip_status lhip_argmax_f32_ws(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                               int32_t advance, void *workspace_dev, void *stream);
 
 /* ---- calibration kernels ---------------------------------------------------
  * No counterpart in the reference.  A plain device-to-device copy and a

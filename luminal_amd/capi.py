@@ -89,6 +89,9 @@ SIGNATURES = {
     "lhip_cast_bf16_to_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),
     "lhip_add_f32": (C.c_int32, [_vp, _vp, _i64, _vp]),
     "lhip_argmax_f32": (C.c_int32, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _vp]),
+    "lhip_argmax_f32_ws": (C.c_int32, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _vp, _vp]),
+    "lhip_q8_0_matmul_bf16_workspace_nbytes": (_sz, [_i64, _i64, _i64, C.c_int32]),
+    "lhip_q8_0_matmul_bf16_ws": (C.c_int32, [_vp, _vp, _vp, _i64, _i64, _i64, C.c_int32, _vp, _sz, _vp]),
     "lhip_copy_bytes": (C.c_int32, [_vp, _vp, _sz, _vp]),
     "lhip_read_bytes": (C.c_int32, [_vp, _sz, _vp, _vp]),
     "lhip_issue_rate_probe": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, _vp, _vp]),

@@ -428,6 +428,9 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restric
     }
 }
 
+lhip_status argmax_impl(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                        int32_t advance, float *workspace, void *stream);
+
 static float *argmax_part_ptr() {
     static float *ptrs[64] = {};
     int dev = 0;
@@ -613,10 +616,26 @@ lhip_status lhip_cast_bf16_to_f32(const void *x_dev, float *y_dev, int64_t n, vo
 
 lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
                             int32_t advance, void *stream) {
+    return argmax_impl(x_dev, n, id_f32_dev, id_i32_dev, pos_dev, advance, nullptr, stream);
+}
+
+lhip_status lhip_argmax_f32_ws(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                               int32_t advance, void *workspace_dev, void *stream) {
+    if (!workspace_dev) return LHIP_ERR_NULL_PTR;
+    if (!aligned(workspace_dev, 8)) return LHIP_ERR_MISALIGNED;
+    return argmax_impl(x_dev, n, id_f32_dev, id_i32_dev, pos_dev, advance, static_cast<float *>(workspace_dev), stream);
+}
+
+}  // extern "C"
+
+namespace lhip {
+
+lhip_status argmax_impl(const float *x_dev, int64_t n, float *id_f32_dev, int32_t *id_i32_dev, int32_t *pos_dev,
+                        int32_t advance, float *workspace, void *stream) {
     if (!x_dev || (!id_f32_dev && !id_i32_dev)) return LHIP_ERR_NULL_PTR;
     if (n <= 0 || n > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
     if (n >= 16384 && aligned(x_dev, 16)) {  // long rows: partial picks over the chip, then one wave
-        float *part = argmax_part_ptr();
+        float *part = workspace ? workspace : argmax_part_ptr();
         if (!part) return LHIP_ERR_HIP;
         const int n4 = static_cast<int>(n >> 2);
         hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxBlocks), dim3(1024), 0, as_stream(stream),
@@ -633,4 +652,4 @@ lhip_status lhip_argmax_f32(const float *x_dev, int64_t n, float *id_f32_dev, in
     return LHIP_OK;
 }
 
-}  // extern "C"
+}  // namespace lhip

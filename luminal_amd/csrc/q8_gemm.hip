@@ -326,9 +326,22 @@ enum { kOutBf16 = 0, kOutF32 = 1, kOutSwiglu = 2 };
 
 // q8_gemm_skinny.hip: the weight-streaming kernel for at most 128 activation rows.
 bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y);
+int q8_gemm_skinny_splits(int m, int n, int k, size_t room);
 lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
-                                  int out, int splits, hipStream_t s);
+                                  int out, int splits, hipStream_t s, bool own_workspace = false, float *ws = nullptr,
+                                  size_t ws_floats = 0);
 float *q8_gemm_scratch(size_t *floats);  // the library's partial-sum array on the current device
+constexpr size_t kGemmScratchFloats = size_t{8} << 20;  // its size (q8_gemm_skinny.hip: kSkScratchFloats)
+
+// Where the partial planes of a K-sliced product go: the library's per-device scratch array (shared by every call on
+// the device), or the caller's workspace (the re-entrant entry points).  A workspace smaller than the plan of the
+// plain call needs means fewer or no slices.
+struct GemmScratch {
+    bool own = false;       // true: `ws` / `floats` below, never the library's array
+    float *ws = nullptr;
+    size_t floats = 0;
+    size_t room() const { return own ? (ws ? (floats < kGemmScratchFloats ? floats : kGemmScratchFloats) : 0) : kGemmScratchFloats; }
+};
 lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s);
 constexpr int kTileSkinny = 5;        // K slices chosen by the library
 constexpr int kTileSkinnySplit = 50;  // + number of K slices
@@ -360,7 +373,7 @@ static lhip_status launch_gemm(int out, const int8_t *qs, const __half *ds, cons
 }
 
 static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
-                                 int tile, int out, void *stream) {
+                                 int tile, int out, void *stream, const GemmScratch &scratch = GemmScratch{}) {
     if (!planar_dev || !x_dev || !y_dev) return LHIP_ERR_NULL_PTR;
     if (lhip_status s = check_q8_shape(n, k)) return s;
     if (m <= 0 || m > kMaxDim) return LHIP_ERR_INVALID_SHAPE;
@@ -374,16 +387,17 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
     hipStream_t s = as_stream(stream);
     if (tile == kTileSkinny || (tile > kTileSkinnySplit && tile <= kTileSkinnySplit + 64)) {
         if (!q8_gemm_skinny_supports(mi, ni, ki, out, y_dev)) return LHIP_ERR_UNSUPPORTED;
-        return q8_gemm_skinny_launch(qs, ds, x_dev, y_dev, mi, ni, ki, out, tile == kTileSkinny ? 0 : tile - kTileSkinnySplit, s);
+        return q8_gemm_skinny_launch(qs, ds, x_dev, y_dev, mi, ni, ki, out, tile == kTileSkinny ? 0 : tile - kTileSkinnySplit, s,
+                                     scratch.own, scratch.ws, scratch.floats);
     }
     if (tile > kTileSliced && tile <= kTileSliced + 16) {
         // Few output tiles and a long K (the down projection of a 512-token prompt: 64 tiles of 256x128): slices of K
         // fill the chip, f32 partial planes go to the scratch array and are added in slice order.
         const int slices = tile - kTileSliced;
         const int kt = ki / kBK;
-        size_t cap = 0;
-        float *part = q8_gemm_scratch(&cap);
-        if (!part) return LHIP_ERR_HIP;
+        size_t cap = scratch.room();
+        float *part = scratch.own ? scratch.ws : q8_gemm_scratch(&cap);
+        if (!part) return scratch.own ? LHIP_ERR_UNSUPPORTED : LHIP_ERR_HIP;
         if (slices < 2 || kt % slices != 0 || (kt / slices) % 4 != 0 || static_cast<size_t>(slices) * mi * ni > cap ||
             ni % 4 != 0 || !aligned(y_dev, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4)))
             return LHIP_ERR_UNSUPPORTED;
@@ -407,7 +421,7 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
 #undef LHIP_TILE
 }
 
-static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *y) {
+static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *y, size_t room = kGemmScratchFloats) {
     // Few activation rows: the product is bound by the weight stream
     if (m <= 128 && n <= kMaxDim && k <= kMaxDim &&
         q8_gemm_skinny_supports(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), out, y))
@@ -422,7 +436,7 @@ static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *
         const int64_t b0 = blocks(256, 128), kt = k / kBK;
         for (int slices = 8; slices >= 2; slices >>= 1)
             if (b0 * slices <= 256 && kt % slices == 0 && (kt / slices) % 4 == 0 &&
-                static_cast<size_t>(slices) * m * n <= (size_t{8} << 20))
+                static_cast<size_t>(slices) * m * n <= room)
                 return kTileSliced + slices;
     }
     // Otherwise the 256x128 tile from 64 workgroups on (measured faster than the smaller tiles there even with a
@@ -455,6 +469,33 @@ lhip_status lhip_q8_0_matmul_bf16_f32out(const void *planar_dev, const void *x_d
 lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_dev, void *out_dev, int64_t m, int64_t n,
                                          int64_t k, void *stream) {
     return gemm_dispatch(planar_dev, x_dev, out_dev, m, n, k, gemm_auto_tile(m, n, k, kOutSwiglu, out_dev), kOutSwiglu, stream);
+}
+
+size_t lhip_q8_0_matmul_bf16_workspace_nbytes(int64_t m, int64_t n, int64_t k, int32_t out_form) {
+    if (check_q8_shape(n, k) != LHIP_OK || m <= 0 || m > kMaxDim || k % kBK != 0) return 0;
+    if (out_form < kOutBf16 || out_form > kOutSwiglu) return 0;
+    // the plan of the plain call (an aligned output is assumed: the plain call slices K for aligned outputs only)
+    const int tile = gemm_auto_tile(m, n, k, out_form, nullptr);
+    size_t floats = 0;
+    if (tile > kTileSliced && tile <= kTileSliced + 16)
+        floats = static_cast<size_t>(tile - kTileSliced) * m * n;
+    else if (tile == kTileSkinny) {
+        const int splits = q8_gemm_skinny_splits(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), kGemmScratchFloats);
+        if (splits > 1) floats = static_cast<size_t>(splits) * m * n;
+    }
+    return floats * sizeof(float);
+}
+
+lhip_status lhip_q8_0_matmul_bf16_ws(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n, int64_t k,
+                                     int32_t out_form, void *workspace_dev, size_t workspace_nbytes, void *stream) {
+    if (out_form < kOutBf16 || out_form > kOutSwiglu) return LHIP_ERR_INVALID_SHAPE;
+    if (workspace_dev && !aligned(workspace_dev, 256)) return LHIP_ERR_MISALIGNED;
+    GemmScratch scratch;
+    scratch.own = true;
+    scratch.ws = static_cast<float *>(workspace_dev);
+    scratch.floats = workspace_dev ? workspace_nbytes / sizeof(float) : 0;
+    return gemm_dispatch(planar_dev, x_dev, y_dev, m, n, k, gemm_auto_tile(m, n, k, out_form, y_dev, scratch.room()), out_form,
+                         stream, scratch);
 }
 
 }  // extern "C"

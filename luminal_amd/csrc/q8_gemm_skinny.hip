@@ -423,12 +423,12 @@ lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int 
 
 // K slices for a product: enough workgroups for the 256 CUs, slices of whole 512-k units, partial sums within the
 // scratch array.
-int q8_gemm_skinny_splits(int m, int n, int k) {
+int q8_gemm_skinny_splits(int m, int n, int k, size_t room) {
     const int strips = (n + kSkRows - 1) / kSkRows, units = k / kSkUnit, passes = (m + 127) / 128;
     int s = 256 / (strips * passes);
     if (s < 1) s = 1;
     if (s > units) s = units;
-    while (s > 1 && static_cast<size_t>(s) * m * n > kSkScratchFloats) --s;
+    while (s > 1 && static_cast<size_t>(s) * m * n > room) --s;
     const int per = (units + s - 1) / s;
     return (units + per - 1) / per;
 }
@@ -472,10 +472,13 @@ static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, con
 }
 
 // `splits` = 0: chosen here.  The caller has checked q8_gemm_skinny_supports.
+// `own_workspace`: partial planes go to `ws` (ws_floats floats; none: no K slices) and the library's scratch array is
+// not touched.
 lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
-                                  int out, int splits, hipStream_t s) {
+                                  int out, int splits, hipStream_t s, bool own_workspace, float *ws, size_t ws_floats) {
     const int units = k / kSkUnit;
-    if (splits <= 0) splits = q8_gemm_skinny_splits(m, n, k);
+    const size_t room = own_workspace ? (ws ? std::min(ws_floats, kSkScratchFloats) : 0) : kSkScratchFloats;
+    if (splits <= 0) splits = q8_gemm_skinny_splits(m, n, k, room);
     if (splits > units) splits = units;
     {
         const int per = (units + splits - 1) / splits;
@@ -483,8 +486,8 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
     }
     float *part = nullptr;
     if (splits > 1) {
-        if (static_cast<size_t>(splits) * m * n > kSkScratchFloats) return LHIP_ERR_UNSUPPORTED;
-        part = sk_scratch_ptr();
+        if (static_cast<size_t>(splits) * m * n > room) return LHIP_ERR_UNSUPPORTED;
+        part = own_workspace ? ws : sk_scratch_ptr();
         if (!part) return LHIP_ERR_HIP;
     }
     const __bf16 *x = static_cast<const __bf16 *>(x_bf16);

@@ -673,3 +673,25 @@ def test_decode_of_the_last_free_position(oracle):
     eng2, _ = build_model(oracle, cfg, seed=9, max_seq=32)
     eng2.prefill([1, 2, 3, 4, 5])
     assert np.array_equal(eng2.decode(1, use_graph=True).cpu().numpy(), toks)
+
+
+def test_argmax_with_the_callers_workspace():
+    """lhip_argmax_f32_ws: the same pick as lhip_argmax_f32 with the partial picks in the caller's 512 bytes."""
+    lib = capi.load_library()
+    torch.manual_seed(3)
+    x = torch.randn(128256, device=DEV)
+    x[77777] = x.max() + 1.0
+    x[99999] = x[77777]  # an exact tie: the last index wins
+    ws = torch.zeros(512, dtype=torch.uint8, device=DEV)
+    outs = []
+    for use_ws in (False, True):
+        f, i, pos = torch.zeros(1, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV)
+        if use_ws:
+            capi.check(lib.lhip_argmax_f32_ws(x.data_ptr(), x.numel(), f.data_ptr(), i.data_ptr(), pos.data_ptr(), 2, ws.data_ptr(), s()), "ws")
+        else:
+            capi.check(lib.lhip_argmax_f32(x.data_ptr(), x.numel(), f.data_ptr(), i.data_ptr(), pos.data_ptr(), 2, s()), "plain")
+        torch.cuda.synchronize()
+        outs.append((float(f.item()), int(i.item()), int(pos.item())))
+    assert outs[0] == outs[1] == (99999.0, 99999, 2)
+    assert lib.lhip_argmax_f32_ws(x.data_ptr(), x.numel(), None, None, None, 0, ws.data_ptr(), s()) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_argmax_f32_ws(x.data_ptr(), x.numel(), ws.data_ptr(), None, None, 0, None, s()) == capi.LHIP_ERR_NULL_PTR

@@ -333,3 +333,101 @@ def test_swiglu_epilogue_equals_gemm_then_swiglu(m, n, k):
     # pairs are stored two at a time: N must be a multiple of 4
     assert lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), got.data_ptr(), m, n - 2, k, s) \
         == capi.LHIP_ERR_INVALID_SHAPE
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 4096, 4096), (128, 1024, 4096), (512, 4096, 4096), (512, 1024, 4096),
+                                   (300, 600, 2048)])
+def test_bf16_workspace_form_gives_the_plain_calls_bits_and_overlaps_safely(oracle, m, n, k):
+    """lhip_q8_0_matmul_bf16_ws keeps the partial planes of a K-sliced plan in the caller's workspace: with the
+    recommended size it gives the bits of the plain call for every output form (weight-streaming kernel with K
+    slices, tiled kernel with K slices, plans without slices); without a workspace K is not sliced and the bar still
+    holds; two streams with a workspace each run interleaved and each gets its own result."""
+    lib = capi.load_library()
+    qs, d = synth.q8_0_random(n, k, seed=m + n + k)
+    w = upload(qs, d)
+    xfs, xds = [], []
+    for seed in (1, 2):
+        xf, bits = bf16_activations(oracle, m, k, seed=seed)
+        xfs.append(xf)
+        xds.append(torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16))
+    forms = [(capi_form, plain, dtype, cols) for capi_form, plain, dtype, cols in
+             ((0, lib.lhip_q8_0_matmul_bf16, torch.bfloat16, n), (1, lib.lhip_q8_0_matmul_bf16_f32out, torch.float32, n),
+              (2, lib.lhip_q8_0_matmul_bf16_swiglu, torch.bfloat16, n // 2))]
+    sliced = False
+    for form, plain_fn, dtype, cols in forms:
+        nbytes = lib.lhip_q8_0_matmul_bf16_workspace_nbytes(m, n, k, form)
+        sliced = sliced or nbytes > 0
+        assert nbytes % 4 == 0 and nbytes <= 32 << 20
+        spaces = [torch.empty(max(nbytes, 256), dtype=torch.uint8, device=DEV) for _ in xds]
+        plain = []
+        for x in xds:
+            y = torch.empty((m, cols), dtype=dtype, device=DEV)
+            capi.check(plain_fn(w.planar.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, _stream()), "plain")
+            plain.append(y)
+        y_ws = torch.empty((m, cols), dtype=dtype, device=DEV)
+        capi.check(lib.lhip_q8_0_matmul_bf16_ws(w.planar.data_ptr(), xds[0].data_ptr(), y_ws.data_ptr(), m, n, k, form,
+                                                spaces[0].data_ptr() if nbytes else None, nbytes, _stream()), "ws")
+        y_none = torch.empty((m, cols), dtype=dtype, device=DEV)
+        capi.check(lib.lhip_q8_0_matmul_bf16_ws(w.planar.data_ptr(), xds[0].data_ptr(), y_none.data_ptr(), m, n, k, form,
+                                                None, 0, _stream()), "ws none")
+        torch.cuda.synchronize()
+        assert torch.equal(y_ws.view(torch.uint8), plain[0].view(torch.uint8)), form
+        if form != 2:
+            truth = truth_for(oracle, qs, d, xfs[0])
+            assert rel_err(y_none.float().cpu().numpy(), truth) < (TOL if form == 0 else TOL_F32), form
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        outs = [torch.empty((m, cols), dtype=dtype, device=DEV) for _ in xds]
+        torch.cuda.synchronize()
+        for _ in range(10):
+            for i, st in enumerate(streams):
+                capi.check(lib.lhip_q8_0_matmul_bf16_ws(w.planar.data_ptr(), xds[i].data_ptr(), outs[i].data_ptr(), m, n, k,
+                                                        form, spaces[i].data_ptr() if nbytes else None, nbytes,
+                                                        st.cuda_stream), "ws 2")
+        torch.cuda.synchronize()
+        for i in range(2):
+            assert torch.equal(outs[i].view(torch.uint8), plain[i].view(torch.uint8)), (form, i)
+    assert sliced  # every shape here has a K-sliced plan in at least one output form
+
+
+def test_bf16_workspace_form_argument_checks():
+    lib = capi.load_library()
+    w = upload(*synth.q8_0_random(1024, 1024, seed=3))
+    x = torch.zeros((8, 1024), device=DEV, dtype=torch.bfloat16)
+    y = torch.empty((8, 1024), device=DEV, dtype=torch.bfloat16)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    p, xp, yp = w.planar.data_ptr(), x.data_ptr(), y.data_ptr()
+    assert lib.lhip_q8_0_matmul_bf16_workspace_nbytes(8, 1024, 1000, 0) == 0   # invalid shape
+    assert lib.lhip_q8_0_matmul_bf16_workspace_nbytes(8, 1024, 1024, 3) == 0   # no such output form
+    assert lib.lhip_q8_0_matmul_bf16_ws(p, xp, yp, 8, 1024, 1024, 3, None, 0, _stream()) == capi.LHIP_ERR_INVALID_SHAPE
+    assert lib.lhip_q8_0_matmul_bf16_ws(p, xp, yp, 8, 1024, 1024, 0, ws.data_ptr() + 64, 1 << 19, _stream()) == capi.LHIP_ERR_MISALIGNED
+    assert lib.lhip_q8_0_matmul_bf16_ws(None, xp, yp, 8, 1024, 1024, 0, None, 0, _stream()) == capi.LHIP_ERR_NULL_PTR
+
+
+def test_result_of_a_row_depends_on_the_row_count_only_through_the_plan(oracle):
+    """The contract on M: a row's result does not depend on the other rows of the call (equal bits whatever they
+    hold), calls with the same M take the same plan (equal bits), and calls whose M selects another plan - the
+    weight-streaming kernel up to 128 rows, K slices of the tiled kernel, the tiled kernel - agree within the
+    operator's tolerance, not bit for bit (another order of the f32 additions)."""
+    n, k = 4096, 4096
+    qs, d = synth.q8_0_random(n, k, seed=77)
+    w = upload(qs, d)
+    xf, bits = bf16_activations(oracle, 2048, k, seed=5)
+    truth0 = truth_for(oracle, qs, d, xf[:1])
+    x_all = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    row0 = {}
+    for m in (1, 16, 128, 512, 2048):
+        y = QuantizedMatmulBf16().process(x_all[:m].contiguous(), w)
+        other = x_all[:m].clone()
+        if m > 1:
+            other[1:] = torch.flip(other[1:], dims=[0]) * 3.0  # the same first row among different rows
+        y2 = QuantizedMatmulBf16().process(other, w)
+        torch.cuda.synchronize()
+        assert torch.equal(y[0].view(torch.int16), y2[0].view(torch.int16)), m
+        row0[m] = y[0].float().cpu().numpy()
+        assert rel_err(row0[m][None, :], truth0) < TOL, m
+    differing = sum(not np.array_equal(row0[a], row0[b]) for a, b in ((1, 16), (16, 128), (128, 512), (512, 2048)))
+    print(f"[M contract] pairs of neighbouring plans whose first rows differ in some bit: {differing} of 4")
