@@ -569,11 +569,15 @@ static lhip_status launch_exact_gemm(const MoeExactArgs &a, int col_blocks, int 
 
 // Tile height of the exact form for R routed rows over E experts: the smallest of 16, 32, 64 rows that holds an
 // expert with two standard deviations more rows than the average (so that nearly every expert is one tile and its
-// weights are read and expanded once), else 128-row tiles (experts with more rows are cut into equal tiles).
+// weights are read and expanded once); experts with more than 64 rows are cut into equal tiles of at most 64, whose
+// later reads of the weights come out of the XCD's L2.  Measured on the benchmark layer (us per layer, 64-row tiles as
+// four-wave workgroups two to a CU / 128-row tiles as eight-wave workgroups): T = 256 134 / 194, T = 512 187 / 207,
+// T = 1024 274 / 342, T = 2048 458 / 530; and 16- / 32- / 64-row tiles: T = 32 87 / 94 / 110, T = 64 90 / 95 / 110,
+// T = 128 132 / 99 / 114.
 static inline int exact_tile_fragments(int R, int E) {
     const int avg = (R + E - 1) / E;
     const int need = avg + 2 * static_cast<int>(sqrtf(static_cast<float>(avg)) + 0.5f);
-    return need <= 16 ? 1 : need <= 32 ? 2 : need <= 64 ? 4 : 8;
+    return need <= 16 ? 1 : need <= 32 ? 2 : 4;
 }
 
 lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16 *x, const int32_t *sel_dev,
@@ -632,8 +636,7 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
     switch (mt) {
         case 1: st = launch_exact_gemm<1, 4, true, 1, 4>(a1, cb1, max_tiles, s); break;
         case 2: st = launch_exact_gemm<2, 4, true, 1, 4>(a1, cb1, max_tiles, s); break;
-        case 4: st = launch_exact_gemm<4, 4, true, 1, 2>(a1, cb1, max_tiles, s); break;
-        default: st = launch_exact_gemm<8, 4, true, 2, 2>(a1, cb1, max_tiles, s); break;
+        default: st = launch_exact_gemm<4, 4, true, 1, 2>(a1, cb1, max_tiles, s); break;
     }
     if (st) return st;
     MoeExactArgs a2{};
@@ -646,8 +649,7 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
     switch (mt) {
         case 1: st = launch_exact_gemm<1, 2, false, 1, 4>(a2, cb2, max_tiles, s); break;
         case 2: st = launch_exact_gemm<2, 2, false, 1, 4>(a2, cb2, max_tiles, s); break;
-        case 4: st = launch_exact_gemm<4, 4, false, 1, 2>(a2, cb2w, max_tiles, s); break;
-        default: st = launch_exact_gemm<8, 4, false, 2, 2>(a2, cb2w, max_tiles, s); break;
+        default: st = launch_exact_gemm<4, 4, false, 1, 2>(a2, cb2w, max_tiles, s); break;
     }
     if (st) return st;
     return moe_launch_combine(w.out, w.plan.slot_of, wts_dev, y, T, H, topk, s);
