@@ -388,6 +388,33 @@ size_t lhip_attention_decode_workspace_nbytes(int64_t q_heads, int64_t kv_heads,
 lhip_status lhip_attention_decode_f32(const float *qkv_dev, float *k_cache_dev, float *v_cache_dev, float *out_dev,
                                       const int32_t *pos_dev, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
                                       int64_t max_seq, float theta, void *workspace_dev, void *stream);
+/* The same operator over FEW key ranges (one per 64-key tile up to eight for contexts of at most 2048 keys, sixteen
+ * beyond) instead of all the workspace has room for: with its merge launch (_few_ranges_f32; same semantics, other
+ * partial sums, so last bits differ from lhip_attention_decode_f32), and without it (_partial_f32: the ranges' partial
+ * states stay in workspace_dev for lhip_q8_0_matvec_attn_merge_f32, which merges them while it stages its
+ * activations).  Measured on MI355X at 512-768 keys: 9.5 us against 6.6 us for the many-range kernel - a range is
+ * then two tiles of dependent trips to memory instead of one. */
+lhip_status lhip_attention_decode_few_ranges_f32(const float *qkv_dev, float *k_cache_dev, float *v_cache_dev,
+                                                 float *out_dev, const int32_t *pos_dev, int64_t q_heads, int64_t kv_heads,
+                                                 int64_t head_dim, int64_t max_seq, float theta, void *workspace_dev,
+                                                 void *stream);
+lhip_status lhip_attention_decode_partial_f32(const float *qkv_dev, float *k_cache_dev, float *v_cache_dev,
+                                              const int32_t *pos_dev, int64_t q_heads, int64_t kv_heads, int64_t head_dim,
+                                              int64_t max_seq, float theta, void *workspace_dev, void *stream);
+/* y = W att (+ residual), att = the attention output that lhip_attention_decode_few_ranges_f32 would have written for
+ * the partial states lhip_attention_decode_partial_f32 left in attn_workspace_dev at position *pos_dev: the output
+ * projection of model.rs:137-139 with the merge of the key ranges folded into its staging prologue (every workgroup
+ * forms the q_heads * head_dim activations itself, with the merge kernel's arithmetic in the merge kernel's order, so
+ * y equals lhip_attention_decode_few_ranges_f32 followed by lhip_q8_0_matvec_fused_f32 bit for bit), which takes one
+ * launch out of a decoder layer.  k must equal q_heads * head_dim and be a multiple of 2048; residual_dev may be NULL
+ * or equal y_dev.  Contexts beyond 2048 keys (more than eight ranges) are merged correctly but with a dependent trip
+ * to memory per further range.  A measured alternative, not what the Llama engine uses by default: on MI355X the
+ * pair (few-range attention 9.5 us, this call 11.5 us) takes 21.0 us per layer where many-range attention, its merge
+ * launch and the plain output projection take 6.6 + 4.7 + 6.3 = 17.6 us. */
+lhip_status lhip_q8_0_matvec_attn_merge_f32(const void *planar_dev, float *y_dev, int64_t n, int64_t k,
+                                            const void *attn_workspace_dev, const int32_t *pos_dev, int64_t q_heads,
+                                            int64_t kv_heads, int64_t head_dim, int64_t max_seq, const float *residual_dev,
+                                            void *stream);
 /* out[r][j] = up * swish(gate) (model.rs:24-32) with gate = gate_up[r][j], up = gate_up[r][f + j], or, with
  * interleaved != 0, gate = gate_up[r][2j], up = gate_up[r][2j + 1] (the row order the fused matvec epilogue uses). */
 lhip_status lhip_swiglu_f32(const float *gate_up_dev, float *out_dev, int64_t rows, int64_t f, int interleaved,

@@ -83,6 +83,9 @@ SIGNATURES = {
     "lhip_attention_bf16": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lhip_attention_decode_workspace_nbytes": (C.c_size_t, [_i64, _i64, _i64]),
     "lhip_attention_decode_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp]),
+    "lhip_attention_decode_few_ranges_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp]),
+    "lhip_attention_decode_partial_f32": (C.c_int32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_float, _vp, _vp]),
+    "lhip_q8_0_matvec_attn_merge_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "lhip_swiglu_f32": (C.c_int32, [_vp, _vp, _i64, _i64, _int, _vp]),
     "lhip_swiglu_f32_bf16out": (C.c_int32, [_vp, _vp, _i64, _i64, _int, _vp]),
     "lhip_cast_f32_to_bf16": (C.c_int32, [_vp, _vp, _i64, _vp]),

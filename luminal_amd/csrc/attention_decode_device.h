@@ -171,6 +171,23 @@ static inline int dec_splits(int64_t kv_heads) {
     int64_t s = 256 / kv_heads;
     return static_cast<int>(s < 1 ? 1 : (s > 64 ? 64 : s));
 }
+// Key ranges a step's attention is cut into, of the n_splits the workspace has room for.  Normally all of them: at
+// batch 1 the kernel is a handful of dependent trips to memory, and the shorter the ranges the fewer trips (32 ranges
+// of one tile each at 512-768 keys: 6.6 us; 8 ranges of two tiles: 9.5 us).  `few`: one range per 64-key tile up to
+// eight (contexts up to 2048 keys), sixteen beyond - few enough partial states for a consumer to merge them itself
+// (lhip_q8_0_matvec_attn_merge_f32).  Workgroups of ranges that hold no keys leave at once.
+constexpr int kDecMaxActive = 16;
+__host__ __device__ inline int dec_active_splits(int n_keys, int n_splits, bool few) {
+    if (!few) return n_splits;
+    int eff = n_keys <= 2048 ? (n_keys + 63) / 64 : kDecMaxActive;
+    eff = eff > 8 && n_keys <= 2048 ? 8 : eff;
+    eff = eff < 1 ? 1 : eff;
+    return eff < n_splits ? eff : n_splits;
+}
+// Weight of a key range's partial state in the merge, exp(its maximum - the overall maximum).  Out of line: the merge
+// kernel and the matvec prologue that merges on its own must round alike, and inlined copies of the library routine
+// need not.
+__device__ __noinline__ float dec_merge_weight(float m, float mx) { return expf(m - mx); }
 
 // LDS of one workgroup in the attention body.
 template <int G, int HD>
@@ -198,7 +215,7 @@ __device__ __forceinline__ void attention_decode_body(IO io, AttnShared<G, HD> &
                                                       const float *__restrict__ qkv, float *__restrict__ k_cache,
                                                       float *__restrict__ v_cache, int pos, int hkv, int max_seq,
                                                       float theta, int n_splits, float *__restrict__ ws_ml,
-                                                      float4 *__restrict__ ws_acc) {
+                                                      float4 *__restrict__ ws_acc, bool few_ranges = false) {
     constexpr int C4 = HD / 4;
     constexpr int KG = kDecThreads / C4;     // key groups in P.V
     constexpr int KPG = kDecTile / KG;       // keys per group and tile
@@ -210,8 +227,10 @@ __device__ __forceinline__ void attention_decode_body(IO io, AttnShared<G, HD> &
     const bool on = THREADS == kDecThreads || tid < kDecThreads;  // wave-uniform
     const int hq = hkv * G;
     const int n_keys = min(pos + 1, max_seq);
-    const int chunk = (n_keys + n_splits - 1) / n_splits;
+    const int eff_splits = dec_active_splits(n_keys, n_splits, few_ranges);
+    const int chunk = (n_keys + eff_splits - 1) / eff_splits;
     const int k0 = split * chunk, k1 = min(n_keys, k0 + chunk);
+    if (k0 >= k1) return;  // uniform over the workgroup: a range without keys has nothing to do, not even the append
     const float inv_sqrt = 1.0f / sqrtf(static_cast<float>(HD));
     const float4 *kc4 = reinterpret_cast<const float4 *>(k_cache) + static_cast<size_t>(kvh) * max_seq * C4;
     const float4 *vc4 = reinterpret_cast<const float4 *>(v_cache) + static_cast<size_t>(kvh) * max_seq * C4;
@@ -393,14 +412,15 @@ template <int G, int HD, int THREADS, typename IO>
 __device__ __forceinline__ void attention_merge_body(IO io, MergeShared &sh, int head, float *__restrict__ out, int pos,
                                                      int max_seq, int n_splits, const float *__restrict__ ws_ml,
                                                      const float4 *__restrict__ ws_acc,
-                                                     float *__restrict__ out_copy = nullptr) {
+                                                     float *__restrict__ out_copy = nullptr, bool few_ranges = false) {
     constexpr int C4 = HD / 4;
     constexpr int SG = kDecThreads / C4;  // sub-groups: 8 (HD 128) or 16 (HD 64)
     const int tid = threadIdx.x;
     const bool on = THREADS == kDecThreads || tid < kDecThreads;
     const int kvh = head / G, g = head - kvh * G;
     const int n_keys = min(pos + 1, max_seq);
-    const int chunk = (n_keys + n_splits - 1) / n_splits;
+    const int eff_splits = dec_active_splits(n_keys, n_splits, few_ranges);
+    const int chunk = (n_keys + eff_splits - 1) / eff_splits;
     const int n_active = (n_keys + chunk - 1) / chunk;  // ranges that held keys (<= 64)
     const size_t base = static_cast<size_t>(kvh) * n_splits;
     const int c = tid % C4, sg = (tid / C4) % SG;
@@ -438,7 +458,7 @@ __device__ __forceinline__ void attention_merge_body(IO io, MergeShared &sh, int
                 const int sidx = s0 + u * SG;
                 const bool live = sidx < n_active;
                 const float2 v = sh.ml_s[live ? sidx : 0];
-                const float wgt = live ? expf(v.x - mx) : 0.f;
+                const float wgt = live ? dec_merge_weight(v.x, mx) : 0.f;
                 den = fmaf(v.y, wgt, den);
                 num.x = fmaf(a[u].x, wgt, num.x); num.y = fmaf(a[u].y, wgt, num.y);
                 num.z = fmaf(a[u].z, wgt, num.z); num.w = fmaf(a[u].w, wgt, num.w);

@@ -588,8 +588,14 @@ lhip_status lhip_decode_program_create(const lhip_decode_op *ops, int n_ops, int
     std::vector<ProgOp> phases;
     std::vector<int> workers;
     auto settled = [&](int phase, int from) -> bool {
-        for (int q = from; q >= phase; q = phases[static_cast<size_t>(q)].x_phase)
-            if (q == phase || workers[static_cast<size_t>(q)] >= workers[static_cast<size_t>(phase)]) return true;
+        for (int q = from; q >= phase; q = phases[static_cast<size_t>(q)].x_phase) {
+            if (q == phase) return true;
+            // every one of a matvec's or a merge's first workers[q] workgroups does work in it; of an attention
+            // phase's only those whose key range holds keys at the current position
+            if (phases[static_cast<size_t>(q)].type != PHASE_ATTENTION &&
+                workers[static_cast<size_t>(q)] >= workers[static_cast<size_t>(phase)])
+                return true;
+        }
         return false;
     };
     auto note_write = [&](const void *base, size_t words, int writer, int input_phase, size_t *offset) -> bool {

@@ -45,6 +45,7 @@ static int split_min_rows(int64_t n, int64_t k) {
 }  // namespace lhip
 
 #include "q8_gemv_device.h"
+#include "attention_decode_device.h"
 
 namespace lhip {
 
@@ -73,12 +74,89 @@ struct GemvGroup {
 };
 
 struct GemvFuse {
-    const float *norm_w;    // NORM: gain of the RMS norm, K floats
+    const float *norm_w;    // PRO_NORM: gain of the RMS norm, K floats
     float eps;
     const float *residual;  // EPI_ADD: N floats (single weight only)
+    // PRO_MERGE: the activations are the output of decode attention, formed here from the partial states its key
+    // ranges left in the attention workspace (lhip_attention_decode_partial_f32) instead of being read from x
+    const float *ws_ml;
+    const float4 *ws_acc;
+    const int *pos;
+    int hkv, g, c4, n_splits, max_seq;  // KV heads, query heads per KV head, head_dim / 4, ranges of the workspace
 };
 
 enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+enum { PRO_NONE = 0, PRO_NORM = 1, PRO_MERGE = 2 };
+
+// PRO_MERGE: float4 `src` of the attention output (head = src / c4, column src % c4) from the partial states, with
+// the arithmetic and the order of additions of attention_merge_body: its SG = 256 / c4 sub-groups take the ranges
+// sg, sg + SG, ... in a chain of fused multiply-adds each, and their sums are added in sub-group order (a sub-group
+// without ranges adds zeros).  Up to eight ranges - every context of at most 2048 keys - are requested at once and
+// cost one trip to memory; more than eight take a loop of dependent trips, which is correct and slow: callers that
+// serve longer contexts keep the merge launch.
+__device__ __forceinline__ float4 merged_attention_piece(const GemvFuse &f, int src, int n_active) {
+    const int head = src / f.c4, c = src - head * f.c4;
+    const int kvh = head / f.g, gq = head - kvh * f.g;
+    const size_t base = static_cast<size_t>(kvh) * f.n_splits;
+    auto slot_of = [&](int s) { return (base + min(s, n_active - 1)) * f.g + gq; };  // ranges past the last re-read it
+    float4 a[8];
+    float2 ml[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {  // every request before the first use
+        const size_t slot = slot_of(s);
+        ml[s] = *reinterpret_cast<const float2 *>(f.ws_ml + slot * 2);
+        a[s] = f.ws_acc[slot * f.c4 + c];
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        if (s < n_active) mx = fmaxf(mx, ml[s].x);
+    for (int s = 8; s < n_active; ++s) mx = fmaxf(mx, f.ws_ml[slot_of(s) * 2]);
+    float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+    float den = 0.f;
+    const int sgn = kDecThreads / f.c4;  // the merge kernel's sub-groups: 8 (head_dim 128) or 16 (head_dim 64)
+#pragma unroll
+    for (int sg = 0; sg < 8; ++sg) {
+        const float w = sg < n_active ? dec_merge_weight(ml[sg].x, mx) : 0.f;
+        float4 p = make_float4(fmaf(a[sg].x, w, 0.f), fmaf(a[sg].y, w, 0.f), fmaf(a[sg].z, w, 0.f), fmaf(a[sg].w, w, 0.f));
+        float d = fmaf(ml[sg].y, w, 0.f);
+        if (sgn == 8) {  // this sub-group's further ranges sg + 8, sg + 16, ... continue its chain
+            for (int s = sg + 8; s < n_active; s += 8) {
+                const size_t slot = slot_of(s);
+                const float2 m2 = *reinterpret_cast<const float2 *>(f.ws_ml + slot * 2);
+                const float4 a2 = f.ws_acc[slot * f.c4 + c];
+                const float w2 = dec_merge_weight(m2.x, mx);
+                d = fmaf(m2.y, w2, d);
+                p.x = fmaf(a2.x, w2, p.x); p.y = fmaf(a2.y, w2, p.y); p.z = fmaf(a2.z, w2, p.z); p.w = fmaf(a2.w, w2, p.w);
+            }
+        }
+        if (sg == 0) {
+            num = p;
+            den = d;
+        } else {
+            num.x += p.x; num.y += p.y; num.z += p.z; num.w += p.w;
+            den += d;
+        }
+    }
+    if (sgn == 16) {  // sub-groups 8..15 hold one range each
+        for (int s = 8; s < 16; ++s) {
+            float4 p = make_float4(0.f, 0.f, 0.f, 0.f);
+            float d = 0.f;
+            if (s < n_active) {
+                const size_t slot = slot_of(s);
+                const float2 m2 = *reinterpret_cast<const float2 *>(f.ws_ml + slot * 2);
+                const float4 a2 = f.ws_acc[slot * f.c4 + c];
+                const float w2 = dec_merge_weight(m2.x, mx);
+                d = fmaf(m2.y, w2, 0.f);
+                p = make_float4(fmaf(a2.x, w2, 0.f), fmaf(a2.y, w2, 0.f), fmaf(a2.z, w2, 0.f), fmaf(a2.w, w2, 0.f));
+            }
+            num.x += p.x; num.y += p.y; num.z += p.z; num.w += p.w;
+            den += d;
+        }
+    }
+    const float inv = 1.0f / den;
+    return make_float4(num.x * inv, num.y * inv, num.z * inv, num.w * inv);
+}
 
 struct Located {
     const int8_t *qs;
@@ -105,10 +183,11 @@ __device__ __forceinline__ Located locate(const GemvGroup &p, int gg) {
     return o;
 }
 
-template <int R, int S, int W, bool NORM, int EPI>
+template <int R, int S, int W, int PRO, int EPI>
 __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p, const GemvFuse f,
                                                                const float *__restrict__ x, int k, int n_groups) {
     static_assert(EPI != EPI_SWIGLU || R % 2 == 0, "SwiGLU pairs live in one wave");
+    constexpr bool NORM = PRO == PRO_NORM;
     extern __shared__ float4 xs4[];
     __shared__ float red[W];
     const unsigned lane = threadIdx.x & 63u;
@@ -144,10 +223,21 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
         const float4 *g4 = reinterpret_cast<const float4 *>(f.norm_w);
         const int k4 = k >> 2;
         float ss = 0.f;
+        int n_active = 0;
+        if (PRO == PRO_MERGE) {  // the key ranges the attention launch cut this position's context into
+            const int n_keys = min(*f.pos + 1, f.max_seq);
+            const int eff = dec_active_splits(n_keys, f.n_splits, true);
+            const int chunk = (n_keys + eff - 1) / eff;
+            n_active = (n_keys + chunk - 1) / chunk;
+        }
 #pragma unroll 4
         for (int i = threadIdx.x; i < k4; i += W * 64) {
             const int src = (i & ~255) | ((i & 63) << 2) | ((i >> 6) & 3);
-            float4 v = x4[src];
+            float4 v;
+            if (PRO == PRO_MERGE)
+                v = merged_attention_piece(f, src, n_active);
+            else
+                v = x4[src];
             if (NORM) {
                 const float4 g = g4[src];
                 // spelled out, so that every kernel that takes this sum rounds it the same way
@@ -361,7 +451,7 @@ static void choose(int n, int k, int *rows_per_wave, int *k_unroll, int *blocks_
     }
 }
 
-template <int R, int S, int W, bool NORM, int EPI>
+template <int R, int S, int W, int PRO, int EPI>
 static lhip_status launch_fused(const GemvGroup &p, const GemvFuse &f, const float *x, int k, int n_groups,
                                 int blocks_per_cu, hipStream_t s) {
     int grid = (n_groups + W - 1) / W;
@@ -369,10 +459,10 @@ static lhip_status launch_fused(const GemvGroup &p, const GemvFuse &f, const flo
     if (grid > cap) grid = cap;
     const size_t lds_bytes = static_cast<size_t>(k) * sizeof(float);
     static LdsOptIn opt;  // with the static reduction array: beyond the default limit (K = 16384)
-    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(q8_gemv_fused_kernel<R, S, W, NORM, EPI>), lds_bytes,
+    if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(q8_gemv_fused_kernel<R, S, W, PRO, EPI>), lds_bytes,
                                     lds_bytes + W * sizeof(float) > 64 * 1024))
         return st;
-    hipLaunchKernelGGL((q8_gemv_fused_kernel<R, S, W, NORM, EPI>), dim3(static_cast<unsigned>(grid)), dim3(W * 64),
+    hipLaunchKernelGGL((q8_gemv_fused_kernel<R, S, W, PRO, EPI>), dim3(static_cast<unsigned>(grid)), dim3(W * 64),
                        lds_bytes, s, p, f, x, k, n_groups);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
@@ -383,17 +473,17 @@ static lhip_status launch_fused_variant(bool norm, int epi, const GemvGroup &p, 
                                         int n_groups, int blocks_per_cu, hipStream_t s) {
     if (epi == EPI_SWIGLU) {
         if constexpr (R % 2 == 0) {
-            return norm ? launch_fused<R, S, W, true, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s)
-                        : launch_fused<R, S, W, false, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s);
+            return norm ? launch_fused<R, S, W, PRO_NORM, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s)
+                        : launch_fused<R, S, W, PRO_NONE, EPI_SWIGLU>(p, f, x, k, n_groups, blocks_per_cu, s);
         } else {
             return LHIP_ERR_UNSUPPORTED;
         }
     }
     if (epi == EPI_ADD)
-        return norm ? launch_fused<R, S, W, true, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s)
-                    : launch_fused<R, S, W, false, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s);
-    return norm ? launch_fused<R, S, W, true, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s)
-                : launch_fused<R, S, W, false, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s);
+        return norm ? launch_fused<R, S, W, PRO_NORM, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s)
+                    : launch_fused<R, S, W, PRO_NONE, EPI_ADD>(p, f, x, k, n_groups, blocks_per_cu, s);
+    return norm ? launch_fused<R, S, W, PRO_NORM, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s)
+                : launch_fused<R, S, W, PRO_NONE, EPI_NONE>(p, f, x, k, n_groups, blocks_per_cu, s);
 }
 
 // Launch shapes of the fused kernel: (rows per wave, slices per step, waves per workgroup, workgroups per CU).
@@ -612,9 +702,55 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
             p.group_end[i] = INT_MAX;
         }
     }
-    const GemvFuse f{norm_weight_dev, eps, residual_dev};
+    GemvFuse f{};
+    f.norm_w = norm_weight_dev;
+    f.eps = eps;
+    f.residual = residual_dev;
     return dispatch_fused(rows_per_wave, k_unroll, waves_per_block, blocks_per_cu, norm_weight_dev != nullptr, epilogue,
                           p, f, x_dev, static_cast<int>(k), static_cast<int>(groups), as_stream(stream));
+}
+
+lhip_status lhip_q8_0_matvec_attn_merge_f32(const void *planar_dev, float *y_dev, int64_t n, int64_t k,
+                                            const void *attn_workspace_dev, const int32_t *pos_dev, int64_t q_heads,
+                                            int64_t kv_heads, int64_t head_dim, int64_t max_seq, const float *residual_dev,
+                                            void *stream) {
+    if (!planar_dev || !y_dev || !attn_workspace_dev || !pos_dev) return LHIP_ERR_NULL_PTR;
+    if (lhip_status st = check_q8_shape(n, k)) return st;
+    if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_seq <= 0 || q_heads % kv_heads != 0 || max_seq > kMaxDim ||
+        kv_heads > 65535 || k != q_heads * head_dim)
+        return LHIP_ERR_INVALID_SHAPE;
+    const int64_t gq = q_heads / kv_heads;
+    if (!(gq == 1 || gq == 2 || gq == 4 || gq == 8) || !(head_dim == 64 || head_dim == 128)) return LHIP_ERR_UNSUPPORTED;
+    // one 16-wave workgroup per CU shares a single merged copy of the activations; slices of 2048
+    if (k % 2048 != 0 || k > kMaxLdsK) return LHIP_ERR_UNSUPPORTED;
+    if (!aligned(planar_dev, 256) || !aligned(y_dev, 4) || !aligned(attn_workspace_dev, 256) ||
+        (residual_dev && !aligned(residual_dev, 4)))
+        return LHIP_ERR_MISALIGNED;
+    auto *base = static_cast<const uint8_t *>(planar_dev);
+    GemvGroup p;
+    for (int i = 0; i < kMaxGroup; ++i) {
+        p.qs[i] = reinterpret_cast<const int8_t *>(base);
+        p.ds[i] = reinterpret_cast<const unsigned short *>(base + q8_scale_offset(n, k));
+        p.y[i] = y_dev;
+        p.n[i] = static_cast<int>(n);
+        p.group_end[i] = i == 0 ? static_cast<int>(n) : INT_MAX;
+    }
+    const int splits = dec_splits(kv_heads);
+    auto *ws = static_cast<const uint8_t *>(attn_workspace_dev);
+    GemvFuse f{};
+    f.residual = residual_dev;
+    f.ws_ml = reinterpret_cast<const float *>(ws);
+    f.ws_acc = reinterpret_cast<const float4 *>(ws + dec_ml_bytes(kv_heads, splits, gq));
+    f.pos = pos_dev;
+    f.hkv = static_cast<int>(kv_heads);
+    f.g = static_cast<int>(gq);
+    f.c4 = static_cast<int>(head_dim / 4);
+    f.n_splits = splits;
+    f.max_seq = static_cast<int>(max_seq);
+    hipStream_t s = as_stream(stream);
+    const int ki = static_cast<int>(k), groups = static_cast<int>(n);
+    return residual_dev ? launch_fused<1, 2, 16, PRO_MERGE, EPI_ADD>(p, f, nullptr, ki, groups, 1, s)
+                        : launch_fused<1, 2, 16, PRO_MERGE, EPI_NONE>(p, f, nullptr, ki, groups, 1, s);
 }
 
 lhip_status lhip_q8_0_matvec_fused_f32(const void *const *planar_dev, float *const *y_dev, const int64_t *n, int count,

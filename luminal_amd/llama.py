@@ -75,6 +75,14 @@ class LlamaQ8:
         self._program = None
         ws = self.lib.lhip_attention_decode_workspace_nbytes(cfg.q_heads, cfg.kv_heads, cfg.head_dim)
         self._attn_ws = torch.empty(ws, dtype=torch.uint8, device=self.dev) if ws else None
+        # merge_in_o_proj = True lets the output projection merge the attention's key ranges while it stages its
+        # activations (lhip_attention_decode_partial_f32 + lhip_q8_0_matvec_attn_merge_f32: one launch fewer per
+        # layer).  Measured slower on MI355X than the three launches (21.0 against 17.6 us per layer at 512-768
+        # keys: with few key ranges the attention kernel takes two tiles of dependent memory trips per range, and
+        # the merge inside the projection's prologue delays its weight stream), so it is off unless asked for.
+        self.merge_in_o_proj = False
+        self._can_merge_in_o_proj = (self._attn_ws is not None and cfg.dim % 2048 == 0 and cfg.dim <= 16384
+                                     and max_seq <= 2048)
 
     # ---- buffers -----------------------------------------------------------
     def _buf(self, name, shape, dtype=torch.float32):
@@ -283,12 +291,30 @@ class LlamaQ8:
             return logits
         for i, (p_qkv, p_o, p_gu, p_down) in enumerate(plans):
             p_qkv.run(h)                                   # qkv = Wqkv norm(h)
-            self._attend_one(i, qkv, att)
-            p_o.run(att)                                   # h += Wo att
+            if self.merge_in_o_proj and self._can_merge_in_o_proj:
+                self._attend_partial(i, qkv)
+                w_o = self.w[f"{i}.o"]
+                capi.check(lib.lhip_q8_0_matvec_attn_merge_f32(w_o.planar.data_ptr(), h.data_ptr(), w_o.n, w_o.k,
+                                                               self._attn_ws.data_ptr(), self.pos.data_ptr(), cfg.q_heads,
+                                                               cfg.kv_heads, cfg.head_dim, self.max_seq, h.data_ptr(), _s()),
+                           "lhip_q8_0_matvec_attn_merge_f32")  # h += Wo merge(partial states)
+            else:
+                self._attend_one(i, qkv, att)
+                p_o.run(att)                               # h += Wo att
             p_gu.run(h)                                    # act = up * swish(gate) of Wgu norm(h)
             p_down.run(act)                                # h += Wdown act
         head.run(h)                                        # logits = Wout norm(h)
         return logits
+
+    def _attend_partial(self, i, qkv):
+        """Rotary, cache append and attention over the key ranges for one new token of layer i; the ranges' partial
+        states stay in the workspace."""
+        cfg = self.cfg
+        capi.check(self.lib.lhip_attention_decode_partial_f32(qkv.data_ptr(), self.k_cache[i].data_ptr(),
+                                                              self.v_cache[i].data_ptr(), self.pos.data_ptr(), cfg.q_heads,
+                                                              cfg.kv_heads, cfg.head_dim, self.max_seq, cfg.theta,
+                                                              self._attn_ws.data_ptr(), _s()),
+                   "lhip_attention_decode_partial_f32")
 
     def _attend_one(self, i, qkv, att):
         """Rotary, cache append and attention for one new token of layer i."""

@@ -695,3 +695,87 @@ def test_argmax_with_the_callers_workspace():
     assert outs[0] == outs[1] == (99999.0, 99999, 2)
     assert lib.lhip_argmax_f32_ws(x.data_ptr(), x.numel(), None, None, None, 0, ws.data_ptr(), s()) == capi.LHIP_ERR_NULL_PTR
     assert lib.lhip_argmax_f32_ws(x.data_ptr(), x.numel(), ws.data_ptr(), None, None, 0, None, s()) == capi.LHIP_ERR_NULL_PTR
+
+
+@pytest.mark.parametrize("hq,hkv,hd", [(32, 8, 128), (16, 2, 128), (32, 32, 64), (16, 8, 128)])
+def test_output_projection_that_merges_the_key_ranges_itself(hq, hkv, hd):
+    """lhip_attention_decode_partial_f32 + lhip_q8_0_matvec_attn_merge_f32 against lhip_attention_decode_few_ranges_f32
+    followed by the fused matvec with the residual: the same bits, at positions that give one key range, a ragged last
+    range, eight ranges and (beyond 2048 keys) sixteen; the caches are appended to alike.  The few-range attention
+    itself against the many-range one: the operator's tolerance (other partial sums)."""
+    lib = capi.load_library()
+    dim = hq * hd
+    max_seq = 2600
+    rng = np.random.default_rng(hq + hkv)
+    qs, d = synth.q8_0_random(dim, dim, seed=hq * hd, scale_sigma=float(np.sqrt(3.0 / dim) / 0.8))
+    w = Q8Weight.from_raw(synth.q8_0_raw_blocks(qs, d), dim, dim, DEV)
+    ws_n = lib.lhip_attention_decode_workspace_nbytes(hq, hkv, hd)
+    assert ws_n > 0
+    kc0 = torch.from_numpy(rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)).to(DEV)
+    vc0 = torch.from_numpy(rng.standard_normal((hkv, max_seq, hd)).astype(np.float32)).to(DEV)
+    for p in (0, 5, 63, 64, 200, 511, 700, 2047, 2048, 2599):
+        qkv = torch.from_numpy(rng.standard_normal((hq + 2 * hkv) * hd).astype(np.float32)).to(DEV)
+        res = torch.from_numpy(rng.standard_normal(dim).astype(np.float32)).to(DEV)
+        pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+        # reference: attention with its merge launch, then y = res + W att
+        kc, vc = kc0.clone(), vc0.clone()
+        ws = torch.zeros(ws_n, dtype=torch.uint8, device=DEV)
+        att = torch.empty(dim, device=DEV)
+        capi.check(lib.lhip_attention_decode_few_ranges_f32(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), att.data_ptr(),
+                                                            pos.data_ptr(), hq, hkv, hd, max_seq, 500000.0, ws.data_ptr(),
+                                                            s()), "decode, few ranges")
+        kc3, vc3, att3 = kc0.clone(), vc0.clone(), torch.empty(dim, device=DEV)
+        capi.check(lib.lhip_attention_decode_f32(qkv.data_ptr(), kc3.data_ptr(), vc3.data_ptr(), att3.data_ptr(),
+                                                 pos.data_ptr(), hq, hkv, hd, max_seq, 500000.0, ws.data_ptr(), s()), "decode")
+        torch.cuda.synchronize()
+        assert rel_err(att.cpu().numpy(), att3.cpu().numpy().astype(np.float64)) < 2e-3, p  # two f32 paths, other partial sums
+        assert torch.equal(kc3, kc) and torch.equal(vc3, vc), p
+        y_ref = res.clone()
+        from luminal_amd.quantized import FusedMatvec
+        FusedMatvec([w], [y_ref], residual=y_ref, epilogue=FusedMatvec.EPI_ADD).run(att)
+        # the folded form
+        kc2, vc2 = kc0.clone(), vc0.clone()
+        ws2 = torch.full((ws_n,), 0xFF, dtype=torch.uint8, device=DEV)  # stale contents: NaN patterns
+        capi.check(lib.lhip_attention_decode_partial_f32(qkv.data_ptr(), kc2.data_ptr(), vc2.data_ptr(), pos.data_ptr(), hq,
+                                                         hkv, hd, max_seq, 500000.0, ws2.data_ptr(), s()), "partial")
+        y = res.clone()
+        capi.check(lib.lhip_q8_0_matvec_attn_merge_f32(w.planar.data_ptr(), y.data_ptr(), dim, dim, ws2.data_ptr(),
+                                                       pos.data_ptr(), hq, hkv, hd, max_seq, y.data_ptr(), s()), "merge")
+        y_plain = torch.empty(dim, device=DEV)
+        capi.check(lib.lhip_q8_0_matvec_attn_merge_f32(w.planar.data_ptr(), y_plain.data_ptr(), dim, dim, ws2.data_ptr(),
+                                                       pos.data_ptr(), hq, hkv, hd, max_seq, None, s()), "merge, no residual")
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int32), y_ref.view(torch.int32)), p
+        assert torch.equal((y_plain + res).view(torch.int32), y_ref.view(torch.int32)) or torch.allclose(y_plain + res, y_ref), p
+        assert torch.equal(kc2, kc) and torch.equal(vc2, vc), p
+    p8 = w.planar.data_ptr()
+    assert lib.lhip_q8_0_matvec_attn_merge_f32(p8, y.data_ptr(), dim, dim, None, pos.data_ptr(), hq, hkv, hd, max_seq, None, s()) == capi.LHIP_ERR_NULL_PTR
+    assert lib.lhip_q8_0_matvec_attn_merge_f32(p8, y.data_ptr(), dim, dim, ws2.data_ptr(), pos.data_ptr(), hq, hkv, hd + 64, max_seq, None, s()) == capi.LHIP_ERR_INVALID_SHAPE
+
+
+def test_engine_with_the_merge_inside_the_output_projection(oracle):
+    """LlamaQ8.merge_in_o_proj: decode steps through lhip_attention_decode_partial_f32 and
+    lhip_q8_0_matvec_attn_merge_f32 against the oracle, and graph replay against eager stepping."""
+    cfg = LlamaConfig(vocab=1000, dim=2048, layers=2, q_heads=16, kv_heads=4, ffn=2048)
+    eng, wf = build_model(oracle, cfg, seed=77, max_seq=128)
+    eng.merge_in_o_proj = True
+    assert eng.fused_decode and eng._can_merge_in_o_proj
+    prompt = [int(t) for t in np.random.default_rng(2).integers(0, cfg.vocab, 70)]
+    kc, vc = empty_cache(cfg), empty_cache(cfg)
+    want = lo.forward(cfg, wf, prompt, kc, vc, 0)
+    eng.prefill(prompt)
+    tok = lo.argmax_last(want[-1])
+    assert int(eng.tok_i.item()) == tok
+    for step in range(4):
+        want_step = lo.forward(cfg, wf, [tok], kc, vc, len(prompt) + step)[0]
+        logits = eng.decode_step()
+        assert rel_err(logits.cpu().numpy(), want_step) < 2e-3, step
+        tok = lo.argmax_last(want_step)
+        eng.tok.fill_(float(tok))
+        eng.tok_i.fill_(tok)
+    eng.reset()
+    eng.prefill(prompt)
+    eager = eng.decode(6, use_graph=False).cpu().numpy()
+    eng.reset()
+    eng.prefill(prompt)
+    assert np.array_equal(eng.decode(6, use_graph=True).cpu().numpy(), eager)
