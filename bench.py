@@ -31,12 +31,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (FETCH_SIZE scaled by the copy-kernel factor 2.0, plus WRITE_SIZE) of each section's dominant
-# kernel, copied from the committed rocprofv3 counter summaries named beside them; printed with the figure so a
-# reader can tell where it came from (they go stale when a kernel changes and the profile is not refreshed).
+# kernel (for the MoE layer: of the layer's launches at T = 64), copied from the committed rocprofv3 counter
+# summaries named beside them, where the figure is written with its digits in groups of three followed by " B";
+# tests/test_bench_cli.py checks that each file still holds its figure, so a refreshed profile and this table cannot
+# drift apart unnoticed.
 TRAFFIC = {
     "gemv": (138310222, "profiles/q8_gemv_decode_projection_set.md"),
-    "gemm": (694005145, "profiles/q8_gemm_prefill_set.md"),
-    "moe_t64": (2 * (158755 + 82880) * 1024, "profiles/mxfp4_moe_layer.md"),
+    "gemm": (682674278, "profiles/q8_gemm_prefill_set.md"),
+    "moe_t64": (487359283, "profiles/mxfp4_moe_layer.md"),
 }
 
 

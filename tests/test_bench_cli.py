@@ -23,3 +23,16 @@ def test_help_lists_the_driver_flags():
     assert proc.returncode == 0
     for flag in ("--gpus", "--steps", "--warmup", "--workload", "--no-cpu-baseline"):
         assert flag in proc.stdout
+
+
+def test_traffic_figures_are_the_ones_in_the_committed_profiles():
+    """bench.py prints `roofline.traffic` from a table of constants; each must be the figure the rocprofv3 summary it
+    names arrives at (written there as digits in groups of three, then " B")."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_for_traffic", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert set(bench.TRAFFIC) == {"gemv", "gemm", "moe_t64"}
+    for key, (nbytes, source) in bench.TRAFFIC.items():
+        text = open(os.path.join(ROOT, source)).read()
+        assert f"{nbytes:,}".replace(",", " ") + " B" in text, (key, nbytes, source)
