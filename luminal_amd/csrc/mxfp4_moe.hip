@@ -180,6 +180,7 @@ struct MoeGemmArgs {
     int K, Kp;
     int N;                              // output columns per expert (I or H)
     const int *tile_expert, *tile_row0, *tile_rows, *n_tiles;
+    const int *tile_run0, *tile_runlen; // runs of tiles of one expert (MoePlan)
     int tiles_per_xcd;                  // layout of the tile list (MoePlan::tiles_per_xcd)
     void *out;                          // bf16 [R][N] (gated) or f32 [R][N]
     // Gated GEMM with NT == 4 only: when q_hi is set, the epilogue quantises its bf16 result for the next GEMM
@@ -216,21 +217,40 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
     // Which tile and which column block.  Workgroups are dispatched in the order of their linear number
     // (x fastest) and dealt to the eight XCDs in turn, so the workgroups with the same number modulo 8 share an L2.
     // With a tile list laid out per XCD, those take the entries of their XCD's range in order, all column blocks
-    // of one tile after another: the tile's activation rows, which every column block reads, and the weights
-    // of an expert cut into several tiles then come out of that L2 after their first use.  Entries without a
-    // tile have no rows.
+    // of one tile after another: the tile's activation rows, which every column block reads, come out of that L2
+    // after their first use.  Where an expert was cut into a run of several tiles, the run is walked column block
+    // by column block instead (all tiles of the run for one block, then the next block): the workgroups that read
+    // the same weights are dispatched next to each other and share one fetch of them.  Entries without a tile have
+    // no rows.
     int tile = blockIdx.y, cb = blockIdx.x;
+    int expert, row0, rows;
     if (g.tiles_per_xcd) {
         const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-        const int turn = linear >> 3;
-        const int entry = turn / static_cast<int>(gridDim.x);  // < gridDim.y / 8 = tiles_per_xcd
-        cb = turn - entry * static_cast<int>(gridDim.x);
-        tile = (linear & 7) * g.tiles_per_xcd + entry;
+        const int turn = linear >> 3, cols = static_cast<int>(gridDim.x);
+        const int base = (linear & 7) * g.tiles_per_xcd;
+        const int entry = turn / cols;  // < gridDim.y / 8 = tiles_per_xcd
+        cb = turn - entry * cols;
+        tile = base + entry;
+        // (the entry's own tile is read in the same trip to memory; only a workgroup inside a run pays a second one,
+        // and not for the expert, which the run shares)
+        expert = g.tile_expert[tile];
+        row0 = g.tile_row0[tile];
+        rows = g.tile_rows[tile];
+        const int run0 = g.tile_run0[tile], runlen = g.tile_runlen[tile];
+        if (runlen > 1) {
+            const int local = turn - (run0 - base) * cols;  // position among the run's runlen * cols workgroups
+            cb = local / runlen;
+            tile = run0 + (local - cb * runlen);
+            row0 = g.tile_row0[tile];
+            rows = g.tile_rows[tile];
+        }
+    } else {
+        expert = g.tile_expert[tile];
+        row0 = g.tile_row0[tile];
+        rows = g.tile_rows[tile];
     }
-    const int expert = g.tile_expert[tile];
-    const int row0 = g.tile_row0[tile];
-    const int rows = g.tile_rows[tile];
     if (rows == 0) return;
+
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1119,6 +1139,7 @@ lhip_status lhip_mxfp4_moe_bf16_mode(const void *w_gate_up_planar, const void *w
     a1.w_nib = gu; a1.w_sc = gu + mx_scale_offset(e * 2 * i, h);
     a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
+    a1.tile_run0 = w.plan.tile_run0; a1.tile_runlen = w.plan.tile_runlen;
     a1.n_tiles = w.plan.n_tiles; a1.tiles_per_xcd = w.plan.tiles_per_xcd; a1.out = w.act;
     const bool whole_rows = mt == 1 && decode_sized && moe_small_lds_bytes(Hp) <= 150 * 1024;
     // Every gated kernel launched below quantises its result for the down GEMM in its epilogue.
@@ -1144,6 +1165,7 @@ lhip_status lhip_mxfp4_moe_bf16_mode(const void *w_gate_up_planar, const void *w
     a2.w_nib = dn; a2.w_sc = dn + mx_scale_offset(e * h, i);
     a2.rows_per_expert = H; a2.K = I; a2.Kp = Ip; a2.N = H;
     a2.tile_expert = w.plan.tile_expert; a2.tile_row0 = w.plan.tile_row0; a2.tile_rows = w.plan.tile_rows;
+    a2.tile_run0 = w.plan.tile_run0; a2.tile_runlen = w.plan.tile_runlen;
     a2.n_tiles = w.plan.n_tiles; a2.tiles_per_xcd = w.plan.tiles_per_xcd; a2.out = w.out;
     if (mt == 1) {
         st = decode_sized && moe_small_lds_bytes(Ip) <= 150 * 1024

@@ -36,6 +36,10 @@ struct MoePlan {
     int *tile_expert;  // [max_tiles]
     int *tile_row0;    // [max_tiles] first slot of the tile
     int *tile_rows;    // [max_tiles] valid rows in the tile (0 = unused entry)
+    // [max_tiles] the run of a tile: the consecutive list entries that hold tiles of the same expert (on the same XCD,
+    // when the list is cut per XCD) start at entry tile_run0 and number tile_runlen (0 = unused entry).  The exact
+    // GEMMs walk a run column block by column block, so that the workgroups that read the same weights run together.
+    int *tile_run0, *tile_runlen;
     int *n_tiles;      // [1]
     int max_tiles;     // entries of the three tile arrays
     // 0: tiles are listed in expert order from entry 0.  Otherwise the list is cut into eight ranges of this many
@@ -56,6 +60,8 @@ __device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int 
         p.tile_expert[t] = 0;
         p.tile_row0[t] = 0;
         p.tile_rows[t] = 0;
+        p.tile_run0[t] = t;
+        p.tile_runlen[t] = 0;
     }
     __syncthreads();
     for (int r = threadIdx.x; r < R; r += 1024) {
@@ -81,15 +87,21 @@ __device__ __forceinline__ void moe_plan_block(const int *__restrict__ sel, int 
         p.offsets[e] = o;
         const int tiles_e = (cnt[e] + BM - 1) / BM;
         const int per = tiles_e ? ((cnt[e] + tiles_e - 1) / tiles_e + 15) / 16 * 16 : 0;
+        const int nt_first = nt, nt_end = nt + tiles_e;
         for (int m0 = 0; m0 < cnt[e]; m0 += per) {
-            int at = nt;
+            int at = nt, run_first = nt_first, run_end = nt_end;
             if (p.tiles_per_xcd) {  // tile nt of `total` goes to range x = floor(8 nt / total), behind that range's earlier tiles
                 const int x = nt * 8 / total;
-                at = x * p.tiles_per_xcd + nt - (x * total + 7) / 8;
+                const int x_first = (x * total + 7) / 8, x_end = ((x + 1) * total + 7) / 8;  // the tiles of range x
+                at = x * p.tiles_per_xcd + nt - x_first;
+                run_first = max(nt_first, x_first);
+                run_end = min(nt_end, x_end);
             }
             p.tile_expert[at] = e;
             p.tile_row0[at] = o + m0;
             p.tile_rows[at] = min(per, cnt[e] - m0);
+            p.tile_run0[at] = at - (nt - run_first);
+            p.tile_runlen[at] = run_end - run_first;
             ++nt;
         }
         if (e == E - 1) {
@@ -178,6 +190,8 @@ static inline MoeWorkspace carve(void *base, int64_t T, int64_t H, int64_t I, in
     w.plan.tile_expert = reinterpret_cast<int *>(take(max_tiles * 4));
     w.plan.tile_row0 = reinterpret_cast<int *>(take(max_tiles * 4));
     w.plan.tile_rows = reinterpret_cast<int *>(take(max_tiles * 4));
+    w.plan.tile_run0 = reinterpret_cast<int *>(take(max_tiles * 4));
+    w.plan.tile_runlen = reinterpret_cast<int *>(take(max_tiles * 4));
     w.plan.n_tiles = reinterpret_cast<int *>(take(4));
     const int64_t Hp = pad128(H), Ip = pad128(I);
     w.x_hi = take(T * Hp);

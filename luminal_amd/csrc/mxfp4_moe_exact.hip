@@ -92,6 +92,7 @@ struct MoeExactArgs {
     int K, Kp;
     int N;
     const int *tile_expert, *tile_row0, *tile_rows, *n_tiles;
+    const int *tile_run0, *tile_runlen;
     int tiles_per_xcd;
     void *out;            // bf16 [R][N] (gated) or f32 [R][N]
 };
@@ -110,18 +111,37 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_exact_kernel(MoeExactArg
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 3 x A_BUF
 
     // Tile and column block of this workgroup (see MoePlan::tiles_per_xcd for the per-XCD list).
+    // Within a run of tiles of one expert the workgroups are ordered column block by column block: the tiles that
+    // read the same weights are dispatched next to each other and share one fetch of them out of the XCD's L2.
     int tile = blockIdx.y, cb = blockIdx.x;
+    int expert, row0, rows;
     if (g.tiles_per_xcd) {
         const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-        const int turn = linear >> 3;
-        const int entry = turn / static_cast<int>(gridDim.x);
-        cb = turn - entry * static_cast<int>(gridDim.x);
-        tile = (linear & 7) * g.tiles_per_xcd + entry;
+        const int turn = linear >> 3, cols = static_cast<int>(gridDim.x);
+        const int base = (linear & 7) * g.tiles_per_xcd;
+        const int entry = turn / cols;
+        cb = turn - entry * cols;
+        tile = base + entry;
+        // (the entry's own tile is read in the same trip to memory; only a workgroup inside a run pays a second one,
+        // and not for the expert, which the run shares)
+        expert = g.tile_expert[tile];
+        row0 = g.tile_row0[tile];
+        rows = g.tile_rows[tile];
+        const int run0 = g.tile_run0[tile], runlen = g.tile_runlen[tile];
+        if (runlen > 1) {
+            const int local = turn - (run0 - base) * cols;  // position among the run's runlen * cols workgroups
+            cb = local / runlen;
+            tile = run0 + (local - cb * runlen);
+            row0 = g.tile_row0[tile];
+            rows = g.tile_rows[tile];
+        }
+    } else {
+        expert = g.tile_expert[tile];
+        row0 = g.tile_row0[tile];
+        rows = g.tile_rows[tile];
     }
-    const int expert = g.tile_expert[tile];
-    const int row0 = g.tile_row0[tile];
-    const int rows = g.tile_rows[tile];
     if (rows == 0) return;
+
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -631,6 +651,7 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
     a1.rows_per_expert = 2 * I; a1.K = H; a1.Kp = Hp; a1.N = I;
     a1.tile_expert = w.plan.tile_expert; a1.tile_row0 = w.plan.tile_row0; a1.tile_rows = w.plan.tile_rows;
     a1.n_tiles = w.plan.n_tiles; a1.tiles_per_xcd = w.plan.tiles_per_xcd; a1.out = w.act;
+    a1.tile_run0 = w.plan.tile_run0; a1.tile_runlen = w.plan.tile_runlen;
     const int cb1 = (I + 127) / 128;  // 4 waves x two (gate, up) pairs of 16 columns
     lhip_status st;
     switch (mt) {
@@ -645,6 +666,7 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
     a2.rows_per_expert = H; a2.K = I; a2.Kp = Ip; a2.N = H;
     a2.tile_expert = w.plan.tile_expert; a2.tile_row0 = w.plan.tile_row0; a2.tile_rows = w.plan.tile_rows;
     a2.n_tiles = w.plan.n_tiles; a2.tiles_per_xcd = w.plan.tiles_per_xcd; a2.out = w.out;
+    a2.tile_run0 = w.plan.tile_run0; a2.tile_runlen = w.plan.tile_runlen;
     const int cb2 = (H + 127) / 128, cb2w = (H + 255) / 256;
     switch (mt) {
         case 1: st = launch_exact_gemm<1, 2, false, 1, 4>(a2, cb2, max_tiles, s); break;
