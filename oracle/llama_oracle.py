@@ -12,6 +12,12 @@ times V, merge heads, output projection (:112-139); residuals and SwiGLU MLP dow
 Pinned by: the closed forms above checked piecewise in tests/test_llama_oracle.py (norm and softmax against
 direct formulas, rotary embedding against complex multiplication, prefill-vs-incremental consistency of the
 KV cache).  The reference holds no stored vectors for this path.
+
+forward_prompt_bf16 is the same pass with round-to-nearest-even roundings to bfloat16 placed where a prompt pass on
+bf16 matrix-core operands places them (the operands of every linear layer and of the attention products); it has no
+counterpart in the reference, whose graph runs in one dtype throughout, and exists so that such a pass can be held
+to a tight bar against a restatement with its own roundings and, separately, to the distance of that restatement
+from the unrounded truth.
 """
 from __future__ import annotations
 
@@ -94,6 +100,88 @@ def forward(cfg, w, tokens, k_cache, v_cache, pos0):
         x, k_cache[i], v_cache[i] = layer_forward(cfg, wl, x, k_cache[i], v_cache[i], pos0)
     n = rms_norm(x, w["out_norm"], cfg.eps)
     return n @ w["lm_head"].astype(np.float64).T
+
+
+def bf16_round(x):
+    """Round to bfloat16, ties to even, returned as float64 (finite inputs)."""
+    a = np.ascontiguousarray(x, dtype=np.float32)
+    u = a.view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).astype(np.float64).reshape(a.shape)
+
+
+def attention_bf16_operands(q, k_all, v_all, pos0, tile=32):
+    """Causal grouped-query attention with bf16 operands for both products: q / sqrt(head_dim), K and V rounded once;
+    per tile of `tile` keys the weights exp(s - running max) rounded and the running sum taken over the rounded
+    weights (so a result is a convex combination of V rows); the quotient rounded.  q: (s, hq, hd) after the rotary
+    embedding, k_all / v_all: (hkv, n_keys, hd).  Returns (s, hq * hd) in float64."""
+    s, hq, hd = q.shape
+    grp = hq // k_all.shape[0]
+    n_keys = k_all.shape[1]
+    qb = bf16_round(q.astype(np.float32) * (np.float32(1.0) / np.sqrt(np.float32(hd))))
+    kb, vb = bf16_round(k_all), bf16_round(v_all)
+    visible = np.arange(n_keys)[None, :] <= (pos0 + np.arange(s))[:, None]
+    out = np.empty((s, hq, hd))
+    for h in range(hq):
+        sc = np.where(visible, qb[:, h] @ kb[h // grp].T, -np.inf)
+        m = np.full(s, -np.inf)
+        l, acc = np.zeros(s), np.zeros((s, hd))
+        for k0 in range(0, n_keys, tile):  # key 0 is visible to every row, so every running maximum is finite
+            t = sc[:, k0:k0 + tile]
+            m_new = np.maximum(m, t.max(axis=1))
+            corr = np.exp(m - m_new)
+            wgt = bf16_round(np.exp(t - m_new[:, None]))
+            l = l * corr + wgt.sum(axis=1)
+            acc = acc * corr[:, None] + wgt @ vb[h // grp, k0:k0 + tile]
+            m = m_new
+        out[:, h] = bf16_round(acc / l[:, None])
+    return out.reshape(s, hq * hd)
+
+
+def forward_prompt_bf16(cfg, w, tokens, bf16_attention=True, all_logits=True):
+    """The prompt pass (positions 0 .. len(tokens) - 1, empty caches) with the roundings of a pass whose linear layers
+    and attention products take bf16 operands and accumulate in f32: the RMS norms in front of q/k/v, gate/up and (for
+    all_logits) the lm_head write bf16; q/k/v come back unrounded (they feed the rotary embedding and the f32
+    caches); attention as attention_bf16_operands, or, with bf16_attention False, in full precision with only its
+    result rounded; up * swish(gate) is rounded where it is formed; the o and down products join the residual
+    stream unrounded.  With all_logits False the last norm and the lm_head stay unrounded and only the last position
+    is returned, as the generation loop needs it.  Arithmetic between the roundings is float64.  w as in forward().
+    Returns (logits, k_cache, v_cache) with the caches as lists of (kv_heads, s, hd) arrays."""
+    hd, hq, hkv = cfg.head_dim, cfg.q_heads, cfg.kv_heads
+    x = w["embed"][np.asarray(tokens, dtype=np.int64)].astype(np.float64)
+    s = x.shape[0]
+    kcs, vcs = [], []
+    for i in range(cfg.layers):
+        f = lambda key: w[f"{i}.{key}"].astype(np.float64)
+        n = bf16_round(rms_norm(x, w[f"{i}.attn_norm"], cfg.eps))
+        q = rope((n @ f("q").T).reshape(s, hq, hd), 0, cfg.theta)
+        k = rope((n @ f("k").T).reshape(s, hkv, hd), 0, cfg.theta)
+        v = (n @ f("v").T).reshape(s, hkv, hd)
+        # the caches hold f32 rows
+        k_all = k.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
+        v_all = v.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
+        kcs.append(k_all)
+        vcs.append(v_all)
+        if bf16_attention:
+            att = attention_bf16_operands(q.astype(np.float32).astype(np.float64), k_all, v_all, 0)
+        else:
+            grp = hq // hkv
+            att = np.empty((s, hq, hd))
+            mask = np.triu(np.ones((s, s)), 1) * F16_MIN
+            for h in range(hq):
+                sc = q[:, h, :] @ k_all[h // grp].T / np.sqrt(hd) + mask
+                e = np.exp(sc - sc.max(axis=1, keepdims=True))
+                att[:, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v_all[h // grp]
+            att = bf16_round(att.reshape(s, hq * hd))
+        x = x + att @ f("o").T
+        n = bf16_round(rms_norm(x, w[f"{i}.ffn_norm"], cfg.eps))
+        act = bf16_round((n @ f("up").T) * swish(n @ f("gate").T))
+        x = x + act @ f("down").T
+    if all_logits:
+        n = bf16_round(rms_norm(x, w["out_norm"], cfg.eps))
+        return n @ w["lm_head"].astype(np.float64).T, kcs, vcs
+    n = rms_norm(x[-1:], w["out_norm"], cfg.eps)
+    return (n @ w["lm_head"].astype(np.float64).T)[0], kcs, vcs
 
 
 def argmax_last(v):

@@ -1,7 +1,8 @@
 """The Llama-3 decode loop through the C ABI against the numpy oracle, on small
 configurations of the same architecture (the oracle cannot run 8B parameters in
 test time): single operators, f32 prefill + decode logits within 2e-3, graph
-replay equal to eager stepping, bf16 prefill within the bf16 bar."""
+replay equal to eager stepping, bf16 prefill within what its own roundings cost (measured in the test against a
+restatement with the same roundings)."""
 import numpy as np
 import pytest
 
@@ -272,6 +273,42 @@ def test_prompt_attention_on_matrix_cores(hq, hkv, hd, S, pos0):
     assert err < 1e-5, err
 
 
+# ---- the bf16 prompt pass through a whole stack.
+# oracle.llama_oracle.forward_prompt_bf16 is the pass in f64 with the bf16 roundings in the engine's places.  Its
+# distance from the exact f64 pass is what bf16 operands cost (unit roundoff 2^-9 on every operand of every product:
+# about 1.1e-3 of a product's rms each, nine per layer, added in quadrature along the residual stream, the maximum
+# over a few thousand logits four to five deviations out: 1e-2 to 3e-2 of the logits' rms on these two-layer stacks),
+# and the tests compute it.  The engine cannot be held to a tighter bar against that restatement than against the
+# truth: measured stage by stage on the 4096 / 14336 layer, q, k and v of the first layer agree to 3e-4 of their rms
+# (one element of the normed input lands on the other side of a rounding boundary under f32 arithmetic and moves a
+# whole row by that), the attention given the engine's own q, k, v agrees bit for bit, but that 3e-4 flips 2 % of the
+# attention's output roundings by one bf16 ulp each, those flip 38 % of the SwiGLU roundings, and after one layer two
+# faithful implementations differ by about as much as either differs from the truth.  (Where no rounding tips - most of
+# the small stacks below - the engine agrees with the restatement to 3e-7 ... 1.5e-6 of the logits' rms, which is what
+# shows the restatement to be the engine's arithmetic; one tip and the figure is 7e-3 to 2e-2.)  Every operator is held tightly
+# on its own inputs elsewhere in this file and in test_q8_gemm_gpu.py; the stack is held to: no further from the truth,
+# and from the restatement, than 1.5 times what the roundings themselves cost.
+BF16_STACK_FACTOR = 1.5
+
+
+def uses_bf16_attention(cfg):
+    """Head shapes for which the prompt pass takes lhip_attention_bf16 (else attention in f32, result rounded)."""
+    return cfg.head_dim in (64, 128) and cfg.q_heads // cfg.kv_heads in (2, 4, 8)
+
+
+def check_bf16_stack(got, exact, rounded, what=""):
+    """got: the engine's logits; exact: the f64 pass; rounded: the f64 pass with the engine's bf16 roundings."""
+    rms = float(np.sqrt(np.mean(exact * exact)))
+    to_rounded = float(np.max(np.abs(got - rounded))) / rms
+    budget = float(np.max(np.abs(rounded - exact))) / rms
+    to_exact = float(np.max(np.abs(got - exact))) / rms
+    print(f"[bf16 stack{what}] engine vs exact {to_exact:.2e}, restatement with the same roundings vs exact {budget:.2e}, "
+          f"engine vs restatement {to_rounded:.2e} (of the logits' rms)")
+    assert 1e-4 < budget < 5e-2, (what, budget)
+    assert to_exact < BF16_STACK_FACTOR * budget, (what, to_exact, budget)
+    assert to_rounded < BF16_STACK_FACTOR * budget, (what, to_rounded, budget)
+
+
 def _bf16(x):
     """Round to bfloat16 (nearest even) and return as float64."""
     return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).bfloat16().double().numpy()
@@ -429,9 +466,9 @@ def test_llama3_8b_layer_dimensions_vs_oracle(oracle):
     want = lo.forward(cfg, wf, prompt, kc, vc, 0)
     got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
     assert rel_err(got.cpu().numpy(), want) < 2e-3
-    rms = float(np.sqrt(np.mean(want * want)))
     gotb = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True, all_logits=True)
-    assert np.max(np.abs(gotb.cpu().numpy() - want)) / rms < 5e-2  # bf16 activations through the whole stack
+    assert uses_bf16_attention(cfg)
+    check_bf16_stack(gotb.cpu().numpy(), want, lo.forward_prompt_bf16(cfg, wf, prompt)[0], " 4096/14336, 2 layers")
     eng.reset()
     eng.prefill(prompt)
     tok = lo.argmax_last(want[-1])
@@ -479,21 +516,24 @@ def test_bf16_prefill_then_f32_decode(oracle, cfg):
     prompt = [int(t) for t in np.random.default_rng(4).integers(0, cfg.vocab, 20)]
     kc, vc = empty_cache(cfg), empty_cache(cfg)
     want = lo.forward(cfg, wf, prompt, kc, vc, 0)
-    t = np.asarray(want[-1])
+    bfa = uses_bf16_attention(cfg)
+    assert bfa == (cfg.q_heads // cfg.kv_heads != 3)
     got = eng.prefill(prompt, bf16=True).cpu().numpy()
-    assert np.max(np.abs(got - t)) / np.sqrt(np.mean(t * t)) < 5e-2  # bf16 matmuls through the whole stack
+    last_rounded, kcb, vcb = lo.forward_prompt_bf16(cfg, wf, prompt, bf16_attention=bfa, all_logits=False)
+    check_bf16_stack(got, np.asarray(want[-1]), last_rounded, " last position")
     eng.reset()
     allpos = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True,
                          all_logits=True).cpu().numpy()
-    assert np.max(np.abs(allpos - want)) / np.sqrt(np.mean(want * want)) < 5e-2
-    # the f32 decode step continues from the cache the bf16 pass wrote
+    check_bf16_stack(allpos, want, lo.forward_prompt_bf16(cfg, wf, prompt, bf16_attention=bfa)[0], " all positions")
+    # the f32 decode step continues from the cache the bf16 pass wrote: against the f32 oracle step over the exact
+    # caches (the budget of the bf16 pass) and over the caches of the rounded restatement (the f32 tolerance)
     eng.reset()
     eng.prefill(prompt, bf16=True)
     tok = lo.argmax_last(want[-1])
     eng.tok.fill_(float(tok))
     step = lo.forward(cfg, wf, [tok], kc, vc, len(prompt))[0]
-    got_step = eng.decode_step().cpu().numpy()
-    assert np.max(np.abs(got_step - step)) / np.sqrt(np.mean(step * step)) < 5e-2
+    step_rounded = lo.forward(cfg, wf, [tok], kcb, vcb, len(prompt))[0]
+    check_bf16_stack(eng.decode_step().cpu().numpy(), step, step_rounded, " f32 step after the bf16 prompt")
 
 
 def test_bf16_output_forms_equal_the_rounded_f32_forms():
@@ -630,7 +670,8 @@ def test_gguf_loader_gives_the_same_model(oracle, tmp_path, embed_dtype):
     got = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), all_logits=True)
     assert rel_err(got.cpu().numpy(), want) < 2e-3
     gotb = eng.forward(torch.tensor(prompt, dtype=torch.float32, device=DEV), len(prompt), bf16=True, all_logits=True)
-    assert np.max(np.abs(gotb.cpu().numpy() - want)) / np.sqrt(np.mean(want * want)) < 5e-2
+    check_bf16_stack(gotb.cpu().numpy(), want, lo.forward_prompt_bf16(cfg, ow, prompt, bf16_attention=uses_bf16_attention(cfg))[0],
+                     " model read from GGUF")
     eng.prefill(prompt)
     tok = lo.argmax_last(want[-1])
     assert int(eng.tok_i.item()) == tok
