@@ -138,6 +138,35 @@ def attention_bf16_operands(q, k_all, v_all, pos0, tile=32):
     return out.reshape(s, hq * hd)
 
 
+def layer_forward_bf16(cfg, wl, x, bf16_attention=True):
+    """One decoder layer of the prompt pass with bf16 operands (see forward_prompt_bf16), positions 0 .. s - 1 on empty
+    caches.  wl as in layer_forward.  Returns (x, k_all, v_all), the caches as the f32 rows a device would hold."""
+    hd, hq, hkv = cfg.head_dim, cfg.q_heads, cfg.kv_heads
+    s = x.shape[0]
+    f = lambda key: wl[key].astype(np.float64)
+    n = bf16_round(rms_norm(x, wl["attn_norm"], cfg.eps))
+    q = rope((n @ f("q").T).reshape(s, hq, hd), 0, cfg.theta)
+    k = rope((n @ f("k").T).reshape(s, hkv, hd), 0, cfg.theta)
+    v = (n @ f("v").T).reshape(s, hkv, hd)
+    k_all = k.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
+    v_all = v.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
+    if bf16_attention:
+        att = attention_bf16_operands(q.astype(np.float32).astype(np.float64), k_all, v_all, 0)
+    else:
+        grp = hq // hkv
+        att = np.empty((s, hq, hd))
+        mask = np.triu(np.ones((s, s)), 1) * F16_MIN
+        for h in range(hq):
+            sc = q[:, h, :] @ k_all[h // grp].T / np.sqrt(hd) + mask
+            e = np.exp(sc - sc.max(axis=1, keepdims=True))
+            att[:, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v_all[h // grp]
+        att = bf16_round(att.reshape(s, hq * hd))
+    x = x + att @ f("o").T
+    n = bf16_round(rms_norm(x, wl["ffn_norm"], cfg.eps))
+    act = bf16_round((n @ f("up").T) * swish(n @ f("gate").T))
+    return x + act @ f("down").T, k_all, v_all
+
+
 def forward_prompt_bf16(cfg, w, tokens, bf16_attention=True, all_logits=True):
     """The prompt pass (positions 0 .. len(tokens) - 1, empty caches) with the roundings of a pass whose linear layers
     and attention products take bf16 operands and accumulate in f32: the RMS norms in front of q/k/v, gate/up and (for
@@ -147,36 +176,13 @@ def forward_prompt_bf16(cfg, w, tokens, bf16_attention=True, all_logits=True):
     stream unrounded.  With all_logits False the last norm and the lm_head stay unrounded and only the last position
     is returned, as the generation loop needs it.  Arithmetic between the roundings is float64.  w as in forward().
     Returns (logits, k_cache, v_cache) with the caches as lists of (kv_heads, s, hd) arrays."""
-    hd, hq, hkv = cfg.head_dim, cfg.q_heads, cfg.kv_heads
     x = w["embed"][np.asarray(tokens, dtype=np.int64)].astype(np.float64)
-    s = x.shape[0]
     kcs, vcs = [], []
     for i in range(cfg.layers):
-        f = lambda key: w[f"{i}.{key}"].astype(np.float64)
-        n = bf16_round(rms_norm(x, w[f"{i}.attn_norm"], cfg.eps))
-        q = rope((n @ f("q").T).reshape(s, hq, hd), 0, cfg.theta)
-        k = rope((n @ f("k").T).reshape(s, hkv, hd), 0, cfg.theta)
-        v = (n @ f("v").T).reshape(s, hkv, hd)
-        # the caches hold f32 rows
-        k_all = k.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
-        v_all = v.transpose(1, 0, 2).astype(np.float32).astype(np.float64)
+        wl = {key: w[f"{i}.{key}"] for key in LAYER_KEYS}
+        x, k_all, v_all = layer_forward_bf16(cfg, wl, x, bf16_attention)
         kcs.append(k_all)
         vcs.append(v_all)
-        if bf16_attention:
-            att = attention_bf16_operands(q.astype(np.float32).astype(np.float64), k_all, v_all, 0)
-        else:
-            grp = hq // hkv
-            att = np.empty((s, hq, hd))
-            mask = np.triu(np.ones((s, s)), 1) * F16_MIN
-            for h in range(hq):
-                sc = q[:, h, :] @ k_all[h // grp].T / np.sqrt(hd) + mask
-                e = np.exp(sc - sc.max(axis=1, keepdims=True))
-                att[:, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v_all[h // grp]
-            att = bf16_round(att.reshape(s, hq * hd))
-        x = x + att @ f("o").T
-        n = bf16_round(rms_norm(x, w[f"{i}.ffn_norm"], cfg.eps))
-        act = bf16_round((n @ f("up").T) * swish(n @ f("gate").T))
-        x = x + act @ f("down").T
     if all_logits:
         n = bf16_round(rms_norm(x, w["out_norm"], cfg.eps))
         return n @ w["lm_head"].astype(np.float64).T, kcs, vcs

@@ -10,8 +10,10 @@ dequantised by the C oracle and dropped after use (about 1 GB of f32 per layer, 
 the lm_head in slices).  The decode steps are teacher-forced with fixed token ids, so the oracle needs ONE causal pass
 over prompt + forced tokens (its prefill-equals-incremental-decode property is pinned in tests/test_llama_oracle.py):
 row t of that pass is what the engine must produce at position t, by the prompt pass for t < 8 and by a decode step
-after it.  Measured: 13 s of CPU time for the two oracle passes (f64 and f32) on the GPU box's host cores, 2 s of
-GPU time.
+after it.  The prompt pass on bf16 matrix-core operands (what a long prompt runs on, and what the benchmark's 512-token
+prefill uses) is checked in the same walk: the oracle restates it with the engine's bf16 roundings
+(llama_oracle.layer_forward_bf16) over the 8 prompt positions.  Measured: about 20 s of CPU time for the three oracle
+passes (f64, f32, f64 with bf16 roundings) on the GPU box's host cores, 2 s of GPU time.
 """
 import time
 
@@ -67,6 +69,9 @@ def test_llama3_8b_full_depth_vs_oracle(oracle):
         got.append(eng.decode_step().cpu().numpy()[None, :])
     got = np.concatenate(got)
     assert got.shape == (n_prompt + n_forced, cfg.vocab)
+    eng.reset()
+    got_bf16 = eng.forward(prompt, n_prompt, bf16=True, all_logits=True).cpu().numpy()
+    eng.reset()
 
     # ---- oracle: one causal pass over all the tokens, one layer's weights on the host at a time
     t0 = time.perf_counter()
@@ -74,6 +79,7 @@ def test_llama3_8b_full_depth_vs_oracle(oracle):
     ids = torch.tensor(tokens, dtype=torch.int64, device=DEV)
     x = w["embed"][ids].cpu().numpy().astype(np.float64)
     x32 = x.astype(np.float32)  # the same pass in f32 arithmetic, the reference's own (its CPU path is f32 throughout)
+    xb = x[:n_prompt].copy()    # the prompt positions through the pass with bf16 operands
     empty = np.zeros((cfg.kv_heads, 0, hd))
     for i in range(cfg.layers):
         qkv = host_f32(oracle, w[f"{i}.qkv"])          # q rows, then k rows, then v rows
@@ -84,11 +90,14 @@ def test_llama3_8b_full_depth_vs_oracle(oracle):
               "down": host_f32(oracle, w[f"{i}.down"])}
         x, _, _ = lo.layer_forward(cfg, wl, x, empty, empty, 0)
         x32, _, _ = lo.layer_forward(cfg, wl, x32, empty, empty, 0, dtype=np.float32)
+        xb, _, _ = lo.layer_forward_bf16(cfg, wl, xb)
         del qkv, gu, wl
     n = lo.rms_norm(x, w["out_norm"].cpu().numpy(), cfg.eps)
     n32 = lo.rms_norm(x32, w["out_norm"].cpu().numpy(), cfg.eps, np.float32)
+    nb = lo.bf16_round(lo.rms_norm(xb, w["out_norm"].cpu().numpy(), cfg.eps))
     want = np.empty((len(tokens), cfg.vocab))
     cpu32 = np.empty((len(tokens), cfg.vocab), np.float32)
+    rounded = np.empty((n_prompt, cfg.vocab))
     head = w["lm_head"]
     raw = head.to_raw().view(cfg.vocab, -1)
     step = 16032  # 8 slices of the vocabulary
@@ -97,6 +106,7 @@ def test_llama3_8b_full_depth_vs_oracle(oracle):
         wf = oracle.q8_0_dequant(raw[r0:r1].contiguous().cpu().numpy(), (r1 - r0) * cfg.dim).reshape(r1 - r0, cfg.dim)
         want[:, r0:r1] = n @ wf.astype(np.float64).T
         cpu32[:, r0:r1] = n32 @ wf.T
+        rounded[:, r0:r1] = nb @ wf.astype(np.float64).T
     cpu_s = time.perf_counter() - t0
     print(f"[full depth] oracle pass over {len(tokens)} tokens: {cpu_s:.1f} s")
 
@@ -114,6 +124,20 @@ def test_llama3_8b_full_depth_vs_oracle(oracle):
     for t in range(len(tokens)):
         assert errs[t] < FULL_DEPTH_TOL, t
         assert lo.argmax_last(got[t]) == lo.argmax_last(want[t]), t
+
+    # ---- the prompt pass on bf16 operands: no further from the truth, and from the restatement with its own roundings,
+    # than 1.5 times what those roundings cost (tests/test_llama_gpu.py derives the rule: after the first operand that
+    # lands on the other side of a rounding boundary two faithful implementations drift apart by the rounding noise)
+    wp = want[:n_prompt]
+    budget = float(np.max(np.abs(rounded - wp))) / rms
+    to_exact = float(np.max(np.abs(got_bf16 - wp))) / rms
+    to_rounded = float(np.max(np.abs(got_bf16 - rounded))) / rms
+    print(f"[full depth] bf16 prompt pass: engine vs exact {to_exact:.2e}, restatement with the same roundings vs exact "
+          f"{budget:.2e}, engine vs restatement {to_rounded:.2e} (of the logits' rms)")
+    assert 1e-4 < budget < 0.2
+    assert to_exact < 1.5 * budget and to_rounded < 1.5 * budget
+    agree = sum(lo.argmax_last(got_bf16[t]) == lo.argmax_last(wp[t]) for t in range(n_prompt))
+    print(f"[full depth] bf16 prompt pass: greedy pick equal to the exact pass's at {agree} of {n_prompt} positions")
 
     # ---- the generation loop at full depth: graph replay picks the tokens eager stepping picks, and its first
     # decode step's pick is the oracle's for the prompt followed by its own greedy token
