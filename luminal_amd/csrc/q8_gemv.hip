@@ -184,8 +184,18 @@ __device__ __forceinline__ Located locate(const GemvGroup &p, int gg) {
 }
 
 template <int R, int S, int W, int PRO, int EPI>
-__global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p, const GemvFuse f,
-                                                               const float *__restrict__ x, int k, int n_groups) {
+__global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const int8_t *qs0, const unsigned short *ds0,
+                                                               const float *__restrict__ x, const float *aux, int n0,
+                                                               int end0, int k, int n_groups, int grid_blocks, float eps,
+                                                               const GemvGroup p, const GemvFuse f) {
+    // The scalar arguments in front (the first weight of the group, the activations and the sizes) reach the wave in
+    // registers; the two structs are read from the argument buffer by the wave itself.  A wave whose first row group
+    // lies in the first weight - every wave of a single-weight launch - requests its first weights without waiting
+    // for that read, nor does the staging of the activations (grid_blocks is gridDim.x, which otherwise comes out of
+    // the same buffer; eps repeats f.eps; aux is f.norm_w for a kernel with the norm prologue, else f.residual).
+    // Fourteen dwords: what the hardware preloads.
+    const float *norm_w = PRO == PRO_NORM ? aux : f.norm_w;
+    const float *residual = PRO == PRO_NORM ? f.residual : aux;
     static_assert(EPI != EPI_SWIGLU || R % 2 == 0, "SwiGLU pairs live in one wave");
     constexpr bool NORM = PRO == PRO_NORM;
     extern __shared__ float4 xs4[];
@@ -193,7 +203,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
     const unsigned lane = threadIdx.x & 63u;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wave_global = blockIdx.x * W + wave;
-    const int total_waves = gridDim.x * W;
+    const int total_waves = grid_blocks * W;
 
     const int chunks = k / (S * 1024);
     const int my_groups = wave_global < n_groups ? (n_groups - wave_global + total_waves - 1) / total_waves : 0;
@@ -204,15 +214,21 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
     // flight and waiting for it would drain the prefetched next step every time (wait counts retire in order).
     auto residual_of = [&](const Located &l, bool live) -> float {
         const int row = l.row0 + static_cast<int>(lane);
-        return (EPI == EPI_ADD && live && lane < static_cast<unsigned>(R) && row < l.n) ? f.residual[row] : 0.f;
+        return (EPI == EPI_ADD && live && lane < static_cast<unsigned>(R) && row < l.n) ? residual[row] : 0.f;
     };
     float res_cur = 0.f, res_next = 0.f;
 
     StepBuf<R, S> a, b;
     {
-        const Located l = locate<R>(p, wave_global < n_groups ? wave_global : 0);
-        res_cur = residual_of(l, T > 0);
-        load_step(a, l.qs, l.ds, l.row0, l.n, k, 0, lane, T > 0);
+        const int g0 = wave_global < n_groups ? wave_global : 0;
+        if (g0 < end0) {  // wave-uniform
+            load_step(a, qs0, ds0, g0 * R, n0, k, 0, lane, T > 0);
+            asm volatile("" ::: "memory");  // keeps the two arms apart: merged, the loads would wait for the structs
+        } else {
+            const Located l = locate<R>(p, g0);
+            load_step(a, l.qs, l.ds, l.row0, l.n, k, 0, lane, T > 0);
+        }
+        res_cur = residual_of(locate<R>(p, g0), T > 0);
     }
 
     // The norm's scalar factor commutes with the matrix product, so x * g is staged at once and the row sums
@@ -220,7 +236,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
     // is published by the staging barrier.
     {
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
-        const float4 *g4 = reinterpret_cast<const float4 *>(f.norm_w);
+        const float4 *g4 = reinterpret_cast<const float4 *>(norm_w);
         const int k4 = k >> 2;
         float ss = 0.f;
         int n_active = 0;
@@ -254,6 +270,9 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
             if (lane == 0) red[wave] = ss;
         }
     }
+    // The structs are read here, behind the first weight loads and the staging loads: left to their first use inside
+    // the pipeline loop, the read would stall the second step of every wave.
+    asm volatile("" ::"s"(p.group_end[1]), "s"(p.group_end[2]), "s"(p.n[1]));
     __syncthreads();
     if (T == 0) return;
     float scale = 1.f;
@@ -261,7 +280,7 @@ __global__ __launch_bounds__(W * 64) void q8_gemv_fused_kernel(const GemvGroup p
         float total = 0.f;
 #pragma unroll
         for (int w = 0; w < W; ++w) total += red[w];
-        scale = 1.0f / sqrtf(total / static_cast<float>(k) + f.eps);
+        scale = 1.0f / sqrtf(total / static_cast<float>(k) + eps);
     }
 
     float acc[R];
@@ -463,7 +482,8 @@ static lhip_status launch_fused(const GemvGroup &p, const GemvFuse &f, const flo
                                     lds_bytes + W * sizeof(float) > 64 * 1024))
         return st;
     hipLaunchKernelGGL((q8_gemv_fused_kernel<R, S, W, PRO, EPI>), dim3(static_cast<unsigned>(grid)), dim3(W * 64),
-                       lds_bytes, s, p, f, x, k, n_groups);
+                       lds_bytes, s, p.qs[0], p.ds[0], x, PRO == PRO_NORM ? f.norm_w : f.residual, p.n[0], p.group_end[0], k, n_groups,
+                       grid, f.eps, p, f);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
