@@ -169,18 +169,12 @@ struct Located {
 // Row group -> (weight, first row).  All operands are wave-uniform.
 template <int R>
 __device__ __forceinline__ Located locate(const GemvGroup &p, int gg) {
-    Located o{p.qs[0], p.ds[0], p.y[0], p.n[0], gg * R};
-#pragma unroll
-    for (int i = 1; i < kMaxGroup; ++i) {
-        if (gg >= p.group_end[i - 1]) {
-            o.qs = p.qs[i];
-            o.ds = p.ds[i];
-            o.y = p.y[i];
-            o.n = p.n[i];
-            o.row0 = (gg - p.group_end[i - 1]) * R;
-        }
-    }
-    return o;
+    // Two dependent reads of the argument buffer: the three boundaries at once, then the entries of the weight they
+    // select (written as a chain of comparisons, this compiled to a branch and a one-word read per boundary).
+    const int e0 = p.group_end[0], e1 = p.group_end[1], e2 = p.group_end[2];
+    const int w = (gg >= e0) + (gg >= e1) + (gg >= e2);  // boundaries ascend; unused ones are INT_MAX
+    const int before = w == 0 ? 0 : (w == 1 ? e0 : (w == 2 ? e1 : e2));
+    return Located{p.qs[w], p.ds[w], p.y[w], p.n[w], (gg - before) * R};
 }
 
 template <int R, int S, int W, int PRO, int EPI>
