@@ -356,8 +356,16 @@ __device__ __forceinline__ void exact_stage_rows(unsigned char *lds, const __bf1
     }
 }
 
+// The leading arguments are what stands between the launch and the first weight load (sel[tile] -> expert -> address):
+// as scalars they reach the wave in registers, where a by-value struct is read from the argument buffer first.
 template <int D>
-__global__ __launch_bounds__(256) void mx_moe_gateup_direct_exact_kernel(MoeDirectExactArgs g) {
+__global__ __launch_bounds__(256) void mx_moe_gateup_direct_exact_kernel(const int *sel, const uint8_t *w_nib, const uint8_t *w_sc,
+                                                                         const __bf16 *x, int rows_per_expert, int k_in,
+                                                                         int k_padded, int n_out, int n_experts,
+                                                                         int direct_rows, MoeDirectExactArgs rest) {
+    MoeDirectExactArgs g = rest;
+    g.sel = sel; g.w_nib = w_nib; g.w_sc = w_sc; g.x = x;
+    g.rows_per_expert = rows_per_expert; g.K = k_in; g.Kp = k_padded; g.N = n_out; g.n_experts = n_experts; g.direct_rows = direct_rows;
     constexpr int NT = 2;  // a gate fragment and its up fragment
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tile = blockIdx.y;
@@ -458,7 +466,13 @@ struct MoeDownDirectExactArgs {
     __bf16 *y;            // [R / topk][N]
 };
 
-__global__ __launch_bounds__(256) void mx_moe_down_direct_exact_kernel(MoeDownDirectExactArgs g) {
+__global__ __launch_bounds__(256) void mx_moe_down_direct_exact_kernel(const int *sel, const uint8_t *w_nib, const uint8_t *w_sc,
+                                                                       const __bf16 *act, int rows_per_expert, int k_in,
+                                                                       int k_padded, int n_out, int n_experts, int n_rows,
+                                                                       MoeDownDirectExactArgs rest) {
+    MoeDownDirectExactArgs g = rest;  // (leading scalars as in the gate/up kernel)
+    g.sel = sel; g.w_nib = w_nib; g.w_sc = w_sc; g.act = act;
+    g.rows_per_expert = rows_per_expert; g.K = k_in; g.Kp = k_padded; g.N = n_out; g.n_experts = n_experts; g.R = n_rows;
     constexpr int D = 8;  // chunks of a routed row per wave: K up to 4 * D * kChunk
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x;
@@ -619,7 +633,8 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
             auto kern = mx_moe_gateup_direct_exact_kernel<8>;
             static LdsOptIn opt;
             if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
-            hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((I + 63) / 64), static_cast<unsigned>(R)), dim3(256), lds_bytes, s, a1);
+            hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((I + 63) / 64), static_cast<unsigned>(R)), dim3(256), lds_bytes, s,
+                               a1.sel, a1.w_nib, a1.w_sc, a1.x, a1.rows_per_expert, a1.K, a1.Kp, a1.N, a1.n_experts, a1.direct_rows, a1);
             LHIP_CHECK_LAUNCH();
         }
         MoeDownDirectExactArgs a2{};
@@ -631,7 +646,8 @@ lhip_status moe_exact_forward(const uint8_t *gu, const uint8_t *dn, const __bf16
             const size_t lds_bytes = moe_small_lds_bytes(Ip);
             static LdsOptIn opt;
             if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(mx_moe_down_direct_exact_kernel), lds_bytes)) return st;
-            hipLaunchKernelGGL(mx_moe_down_direct_exact_kernel, dim3(static_cast<unsigned>(H / 16)), dim3(256), lds_bytes, s, a2);
+            hipLaunchKernelGGL(mx_moe_down_direct_exact_kernel, dim3(static_cast<unsigned>(H / 16)), dim3(256), lds_bytes, s,
+                               a2.sel, a2.w_nib, a2.w_sc, a2.act, a2.rows_per_expert, a2.K, a2.Kp, a2.N, a2.n_experts, a2.R, a2);
             LHIP_CHECK_LAUNCH();
         }
         return LHIP_OK;
