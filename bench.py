@@ -130,16 +130,24 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0
 MFMA_FP4_PEAK_TFLOPS = 10100.0
 
 
-def _event_us(torch, fn, reps):
-    fn()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
+def _event_us(torch, fn, reps, warm=1, repeats=1):
+    """Average time of one call over `reps` back-to-back calls (HIP events on torch's current stream), after `warm`
+    untimed calls; with `repeats` > 1 the best of that many such averages (the clocks of an idle GPU take a few
+    milliseconds to come up, which a cell of a few short launches otherwise pays for)."""
+    for _ in range(warm):
         fn()
-    e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / reps
+    best = None
+    for _ in range(repeats):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        best = us if best is None or us < best else best
+    return best
 
 
 def bench_issue_rates(args):
@@ -499,7 +507,7 @@ def bench_moe(args, cpu_seconds=None):
         fl = T * 199065600.0
         flops_step += fl
         for name, mode in modes.items():
-            us = _event_us(torch, lambda: run(T, mode), 16)
+            us = _event_us(torch, lambda: run(T, mode), 16, warm=4, repeats=3)
             row = {"us": round(us, 1), "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
                    "tflops": round(fl / us / 1e6, 1), "strict_err": errors[(T, name)]}
             if name == "exact":  # one bf16 x bf16 product per multiply-add
