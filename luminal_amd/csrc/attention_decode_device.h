@@ -91,6 +91,9 @@ __device__ __forceinline__ void st_agent4(float4 *p, const float4 &v) {
 // Operand access policies of the bodies below.  Addresses are given as (base, element index): a tagged array
 // has the element order of the plain one, 8 bytes per element.
 struct PlainIO {
+    // Every slot of a workspace may be read whatever it holds (plain memory: nothing waits for a value to appear), so
+    // a reader need not know which slots were written before it asks for them.
+    static constexpr bool kAnySlot = true;
     __device__ __forceinline__ float ld1(const float *b, size_t i, bool &) const { return as_global(b)[i]; }
     __device__ __forceinline__ float2 ld2(const float *b, size_t i, bool &) const {  // i even
         const lhip_f32x2 v = *as_global(reinterpret_cast<const lhip_f32x2 *>(b + i));
@@ -105,6 +108,7 @@ struct PlainIO {
 constexpr unsigned kTagSpinLimit = 1u << 20;
 
 struct TaggedIO {
+    static constexpr bool kAnySlot = false;  // a slot nobody writes this step never shows this step's tag
     unsigned in_tag, out_tag;
     unsigned *abort_flag, *sticky;  // raised when a wait is given up; seen by every other waiter
     unsigned spins = 0;
@@ -418,24 +422,38 @@ __device__ __forceinline__ void attention_merge_body(IO io, MergeShared &sh, int
     const int tid = threadIdx.x;
     const bool on = THREADS == kDecThreads || tid < kDecThreads;
     const int kvh = head / G, g = head - kvh * G;
+    const size_t base = static_cast<size_t>(kvh) * n_splits;
+    const int c = tid % C4, sg = (tid / C4) % SG;
+    float4 a[4];
+    float2 mine = make_float2(0.f, 0.f);
+    // With plain memory every range of the launch may be asked for, so the addresses of the first round do not depend
+    // on the position: its loads go out here, while the position is still on its way, instead of a trip to memory
+    // behind it; what a range without keys left in its slot is discarded below.
+    if constexpr (IO::kAnySlot) {
+        if (on) {
+            bool ok = true;
+            if (tid < n_splits) mine = io.ld2(ws_ml, ((base + tid) * G + g) * 2, ok);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                a[u] = io.ld4(ws_acc, ((base + min(sg + u * SG, n_splits - 1)) * G + g) * C4 + c, ok);
+        }
+    }
     const int n_keys = min(pos + 1, max_seq);
     const int eff_splits = dec_active_splits(n_keys, n_splits, few_ranges);
     const int chunk = (n_keys + eff_splits - 1) / eff_splits;
     const int n_active = (n_keys + chunk - 1) / chunk;  // ranges that held keys (<= 64)
-    const size_t base = static_cast<size_t>(kvh) * n_splits;
-    const int c = tid % C4, sg = (tid / C4) % SG;
     auto acc_index = [&](int sidx) { return ((base + min(sidx, n_active - 1)) * G + g) * C4 + c; };
 
-    float4 a[4];
-    float2 mine = make_float2(0.f, 0.f);
     if (on) {
-        bool ok;
-        do {
-            ok = true;
-            if (tid < n_active) mine = io.ld2(ws_ml, ((base + tid) * G + g) * 2, ok);
+        if constexpr (!IO::kAnySlot) {
+            bool ok;
+            do {
+                ok = true;
+                if (tid < n_active) mine = io.ld2(ws_ml, ((base + tid) * G + g) * 2, ok);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) a[u] = io.ld4(ws_acc, acc_index(sg + u * SG), ok);
-        } while (io.again(ok));
+                for (int u = 0; u < 4; ++u) a[u] = io.ld4(ws_acc, acc_index(sg + u * SG), ok);
+            } while (io.again(ok));
+        }
         if (tid < n_active) sh.ml_s[tid] = mine;
     }
     __syncthreads();
@@ -459,9 +477,10 @@ __device__ __forceinline__ void attention_merge_body(IO io, MergeShared &sh, int
                 const bool live = sidx < n_active;
                 const float2 v = sh.ml_s[live ? sidx : 0];
                 const float wgt = live ? dec_merge_weight(v.x, mx) : 0.f;
+                const float4 av = live ? a[u] : make_float4(0.f, 0.f, 0.f, 0.f);  // (a slot never written may hold anything)
                 den = fmaf(v.y, wgt, den);
-                num.x = fmaf(a[u].x, wgt, num.x); num.y = fmaf(a[u].y, wgt, num.y);
-                num.z = fmaf(a[u].z, wgt, num.z); num.w = fmaf(a[u].w, wgt, num.w);
+                num.x = fmaf(av.x, wgt, num.x); num.y = fmaf(av.y, wgt, num.y);
+                num.z = fmaf(av.z, wgt, num.z); num.w = fmaf(av.w, wgt, num.w);
             }
         }
         sh.num_s[sg * C4 + c] = num;
