@@ -241,7 +241,7 @@ def bench_rows_f32(args):
     per = {}
     for nm, (n, k) in shapes.items():
         for m in ms_list:
-            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3) / len(bufs[nm])
+            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3, warm=1, repeats=3) / len(bufs[nm])
             passes = (m + 63) // 64
             per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(2.0 * m * n * k / us / 1e6, 1),
                                   "weight_gbs": round(passes * n * k * 34 / 32 / us / 1e3, 1)}
@@ -352,7 +352,7 @@ def bench_prefill_gemm(args, cpu_seconds=None):
     per = {}
     for nm, (n, k) in shapes.items():
         for m in ms_list:
-            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3) / len(bufs[nm])
+            us = _event_us(torch, lambda: [run(nm, m, b) for b in bufs[nm]], 3, warm=1, repeats=3) / len(bufs[nm])
             fl = 2.0 * m * n * k
             by = n * k * 34 // 32 + 2 * m * k + 2 * m * n
             per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
@@ -360,7 +360,7 @@ def bench_prefill_gemm(args, cpu_seconds=None):
                                   "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
     # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> on the M = 2048 gate/up shape
     n, k, m = 14336, 4096, 2048
-    us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5) / len(bufs["gate/up"])
+    us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5, warm=1, repeats=3) / len(bufs["gate/up"])
     ach = 2.0 * m * n * k / us / 1e6
     value = flops_step / (wall / args.steps) / 1e12
     g128 = per["gate/up M=128"]
