@@ -215,7 +215,11 @@ lhip_status lhip_q8_0_matmul_bf16_swiglu(const void *planar_dev, const void *x_d
  * tile over S slices of K with the partial sums in the same scratch array (2 <= S <= 16,
  * K / 64 / S a whole multiple of 4, S * m * N <= 8 Mi; what the plain entry
  * points take for K >= 8192 when whole-K tiles would leave most of the chip idle, so
- * the note on overlapping calls above applies to those shapes too). */
+ * the note on overlapping calls above applies to those shapes too),
+ * 200 = the 256x128 tile in whole rounds of 256 workgroups and the column tiles left over in 2 to 8 slices of K
+ * through the same scratch array (what the plain entry points take when more than 256 tiles would end in a
+ * partly filled round: K >= 2048, the number of 256-row tiles a divisor of 256; LHIP_ERR_UNSUPPORTED where there
+ * is no such remainder). */
 lhip_status lhip_q8_0_matmul_bf16_cfg(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                       int64_t k, int tile, void *stream);
 

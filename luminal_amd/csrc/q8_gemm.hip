@@ -68,13 +68,15 @@ constexpr int kRowBytes = 144;      // 64 bf16 + 16 bytes of padding
 // The per-block fma costs one v_fma per output element and block on the vector ALU, the same number of cycles the
 // block's two MFMAs take on the matrix pipe.
 // D = register prefetch depth in K tiles (D > 1 needs K % (64*D) == 0 and D even).
+// N = weight rows of this launch; ldy = row pitch of y in weight rows (N, or more when the launch writes the leading
+// columns of a wider output; the SwiGLU form stores pairs at half that pitch).
 // OutT = __bf16 (rounded to nearest even) or float (the accumulators as they are).
 template <int BM, int BN, int WM, int WN, int D, typename OutT>
 __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t *__restrict__ qs,
                                                                  const __half *__restrict__ ds,
                                                                  const __bf16 *__restrict__ x, OutT *__restrict__ y_all,
                                                                  int M, int N, int K, int m_tiles, int n_tiles,
-                                                                 int swiglu, int kt_slice, int m_group) {
+                                                                 int swiglu, int kt_slice, int m_group, int ldy) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 accumulator tiles per wave
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
                             typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
                             const bf16x2 pk = {static_cast<__bf16>(act), static_cast<__bf16>(act2)};
                             *reinterpret_cast<bf16x2 *>(reinterpret_cast<__bf16 *>(y) +
-                                                        static_cast<size_t>(row) * (N >> 1) + (col >> 1)) = pk;
+                                                        static_cast<size_t>(row) * (ldy >> 1) + (col >> 1)) = pk;
                         }
                     }
                 }
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = static_cast<OutT>(acc[i][j][v]);
+                if (row < M && col < N) y[static_cast<size_t>(row) * ldy + col] = static_cast<OutT>(acc[i][j][v]);
             }
         }
 }
@@ -357,10 +359,42 @@ struct GemmScratch {
     size_t floats = 0;
     size_t room() const { return own ? (ws ? (floats < kGemmScratchFloats ? floats : kGemmScratchFloats) : 0) : kGemmScratchFloats; }
 };
-lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s);
+lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s, int ldy = 0);
 constexpr int kTileSkinny = 5;        // K slices chosen by the library
 constexpr int kTileSkinnySplit = 50;  // + number of K slices
 constexpr int kTileSliced = 120;      // + number of K slices: the 256x128 tile over slices of K, then a reduction
+constexpr int kTileTail = 200;        // the 256x128 tile in whole rounds of 256 workgroups, the last columns over K slices
+
+// A product of more than 256 tiles of 256x128 runs in rounds of 256 workgroups (one per CU), and a last round that
+// is partly filled takes as long as a full one: 896 tiles (gate/up at 2048 rows) are 3.5 rounds of work in the time
+// of 4.  The plan below gives the whole rounds to the plain kernel and the remaining column tiles to the K-sliced
+// form (f32 partial planes in the scratch array, added in slice order), so that the remainder fills the chip for
+// 1 / slices of a round: `n_main` leading weight rows in whole rounds, `slices` K slices for the rest (0: no such
+// plan).  Needs the M tiles to divide 256, a remainder of at most half a round, K long enough for the saving to
+// exceed the reduction launch, and room for the planes.
+struct GemmTail {
+    int n_main = 0, slices = 0;
+};
+static GemmTail gemm_tail_plan(int64_t m, int64_t n, int64_t k, int out, const void *y, size_t room) {
+    GemmTail none;
+    if (m <= 128 || k < 2048 || n % 4 != 0 || !aligned(y, out == kOutF32 ? 16 : (out == kOutBf16 ? 8 : 4))) return none;
+    const int64_t m_tiles = (m + 255) / 256, n_tiles = (n + 127) / 128;
+    if (m_tiles * n_tiles <= 256 || 256 % m_tiles != 0) return none;
+    const int64_t per_round = 256 / m_tiles;                 // column tiles of one round
+    const int64_t main_tiles = n_tiles / per_round * per_round;
+    const int64_t tail_tiles = (n_tiles - main_tiles) * m_tiles;
+    if (tail_tiles == 0) return none;
+    const int64_t n_tail = n - main_tiles * 128, kt = k / kBK;
+    for (int slices = 8; slices >= 2; slices >>= 1)
+        if (tail_tiles * slices <= 256 && kt % slices == 0 && (kt / slices) % 4 == 0 &&
+            static_cast<size_t>(slices) * m * n_tail <= room) {
+            GemmTail t;
+            t.n_main = static_cast<int>(main_tiles * 128);
+            t.slices = slices;
+            return t;
+        }
+    return none;
+}
 
 // M tiles per group of the raster (see the kernel).  Measured on the FFN, QKV and lm_head shapes: groups of 8 are
 // 5 % faster than one group of all the M tiles at M = 8192 (32 M tiles), 1 % at 4096, and the same launch at or below
@@ -370,7 +404,7 @@ static int gemm_m_group(int m_tiles) { return m_tiles < kGemmMGroup ? m_tiles : 
 
 template <int BM, int BN, int WM, int WN, int D, typename OutT>
 static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void *x, void *y, int m, int n, int k,
-                               int swiglu, hipStream_t s, int slices = 1) {
+                               int swiglu, hipStream_t s, int slices = 1, int ldy = 0) {
     const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     if (static_cast<int64_t>(m_tiles) * n_tiles_pad > 0x7fffffff) return LHIP_ERR_INVALID_SHAPE;  // the grid's x extent
@@ -381,7 +415,7 @@ static lhip_status launch_gemm_t(const int8_t *qs, const __half *ds, const void 
     const int kt_slice = slices > 1 ? (k / kBK + slices - 1) / slices : 0;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(m_tiles * n_tiles_pad), static_cast<unsigned>(slices)),
                        dim3(WM * WN * 64), lds_bytes, s, qs, ds, static_cast<const __bf16 *>(x), static_cast<OutT *>(y), m,
-                       n, k, m_tiles, n_tiles, swiglu, kt_slice, gemm_m_group(m_tiles));
+                       n, k, m_tiles, n_tiles, swiglu, kt_slice, gemm_m_group(m_tiles), ldy > 0 ? ldy : n);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
@@ -426,6 +460,29 @@ static lhip_status gemm_dispatch(const void *planar_dev, const void *x_dev, void
             return st;
         return q8_gemm_reduce_launch(part, y_dev, mi, ni, slices, out, s);
     }
+    if (tile == kTileTail) {
+        size_t cap = scratch.room();
+        float *part = scratch.own ? scratch.ws : q8_gemm_scratch(&cap);
+        if (!part) return scratch.own ? LHIP_ERR_UNSUPPORTED : LHIP_ERR_HIP;
+        const GemmTail t = gemm_tail_plan(m, n, k, out, y_dev, cap);
+        if (t.slices < 2) return LHIP_ERR_UNSUPPORTED;
+        const int n_tail = ni - t.n_main;
+        // whole rounds: the leading n_main weight rows, written into the full-width output
+        if (lhip_status st = out == kOutF32
+                                 ? launch_gemm_t<256, 128, 4, 2, 4, float>(qs, ds, x_dev, y_dev, mi, t.n_main, ki, 0, s, 1, ni)
+                                 : launch_gemm_t<256, 128, 4, 2, 4, __bf16>(qs, ds, x_dev, y_dev, mi, t.n_main, ki,
+                                                                            out == kOutSwiglu, s, 1, ni))
+            return st;
+        // the rest: K slices of the trailing weight rows into the planes, then their sum into the trailing columns
+        const int8_t *qs_tail = qs + static_cast<size_t>(t.n_main) * ki;
+        const __half *ds_tail = ds + static_cast<size_t>(t.n_main) * (ki / 32);
+        if (lhip_status st = launch_gemm_t<256, 128, 4, 2, 4, float>(qs_tail, ds_tail, x_dev, part, mi, n_tail, ki, 0, s, t.slices))
+            return st;
+        const size_t col0 = out == kOutSwiglu ? t.n_main / 2 : t.n_main;
+        void *y_tail = out == kOutF32 ? static_cast<void *>(static_cast<float *>(y_dev) + col0)
+                                      : static_cast<void *>(static_cast<__bf16 *>(y_dev) + col0);
+        return q8_gemm_reduce_launch(part, y_tail, mi, n_tail, t.slices, out, s, ni);
+    }
     // Register prefetch four (two) K tiles ahead needs K to be a whole number of 4-tile (2-tile) rounds.
     const int depth = (k % (kBK * 4)) == 0 ? 4 : ((k % (kBK * 2)) == 0 ? 2 : 1);
 #define LHIP_TILE(BM, BN, WM, WN)                                                                          \
@@ -462,6 +519,7 @@ static int gemm_auto_tile(int64_t m, int64_t n, int64_t k, int out, const void *
     }
     // Otherwise the 256x128 tile from 64 workgroups on (measured faster than the smaller tiles there even with a
     // quarter of the CUs busy: its K loop is the shortest per flop), smaller tiles for small products.
+    if (m > 128 && k % (kBK * 4) == 0 && gemm_tail_plan(m, n, k, out, y, room).slices >= 2) return kTileTail;
     if (m > 128 && blocks(256, 128) >= 64) return 0;
     return blocks(128, 64) >= 64 ? 2 : 3;
 }
@@ -500,6 +558,10 @@ size_t lhip_q8_0_matmul_bf16_workspace_nbytes(int64_t m, int64_t n, int64_t k, i
     size_t floats = 0;
     if (tile > kTileSliced && tile <= kTileSliced + 16)
         floats = static_cast<size_t>(tile - kTileSliced) * m * n;
+    else if (tile == kTileTail) {
+        const GemmTail t = gemm_tail_plan(m, n, k, out_form, nullptr, kGemmScratchFloats);
+        floats = static_cast<size_t>(t.slices) * m * (n - t.n_main);
+    }
     else if (tile == kTileSkinny) {
         const int splits = q8_gemm_skinny_splits(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k), kGemmScratchFloats);
         if (splits > 1) floats = static_cast<size_t>(splits) * m * n;

@@ -375,10 +375,11 @@ __global__ __launch_bounds__(12 * 64) void q8_gemm_skinny_kernel(const int8_t *_
 
 }
 
-// Sum of the K slices in slice order, then the output form.  One thread per four weight rows.
+// Sum of the K slices in slice order, then the output form.  One thread per four weight rows.  ldy = row pitch of y
+// in weight rows (N, or more when the planes are the trailing columns of a wider output).
 template <int OUT>
 __global__ __launch_bounds__(256) void q8_gemm_skinny_reduce_kernel(const float *__restrict__ part, void *__restrict__ y,
-                                                                    int M, int N, int splits) {
+                                                                    int M, int N, int splits, int ldy) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     const size_t quads = static_cast<size_t>(M) * (N >> 2);
     if (i >= quads) return;
@@ -386,7 +387,7 @@ __global__ __launch_bounds__(256) void q8_gemm_skinny_reduce_kernel(const float 
     sk_f32x4 v = *reinterpret_cast<const sk_f32x4 *>(part + 4 * i);
     for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const sk_f32x4 *>(part + s * plane + 4 * i);
     const int m = static_cast<int>(i / (N >> 2)), n = static_cast<int>(i % (N >> 2)) * 4;
-    sk_store4<OUT>(y, nullptr, 0, M, N, m, n, v);
+    sk_store4<OUT>(y, nullptr, 0, M, ldy, m, n, v);
 }
 
 // Scratch address per device (a __device__ array has one copy, at its own address, on every device).
@@ -408,14 +409,15 @@ float *q8_gemm_scratch(size_t *floats) {
 }
 
 // Adds `slices` f32 planes of (m, n) in order and writes the output form (as the GEMM epilogues: bf16, f32, f16, SwiGLU).
-lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s) {
+lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int slices, int out, hipStream_t s, int ldy = 0) {
+    if (ldy <= 0) ldy = n;
     const size_t quads = static_cast<size_t>(m) * (n >> 2);
     const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
     switch (out) {
-        case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
-        case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
-        case kSkOutF16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF16>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
-        default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, slices); break;
+        case kSkOutBf16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutBf16>, grid, dim3(256), 0, s, part, y, m, n, slices, ldy); break;
+        case kSkOutF32: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF32>, grid, dim3(256), 0, s, part, y, m, n, slices, ldy); break;
+        case kSkOutF16: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutF16>, grid, dim3(256), 0, s, part, y, m, n, slices, ldy); break;
+        default: hipLaunchKernelGGL(q8_gemm_skinny_reduce_kernel<kSkOutSwiglu>, grid, dim3(256), 0, s, part, y, m, n, slices, ldy); break;
     }
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;

@@ -275,6 +275,61 @@ def test_k_sliced_tiled_gemm(oracle):
                                          st) == capi.LHIP_ERR_UNSUPPORTED
 
 
+def test_whole_rounds_plus_k_sliced_remainder(oracle):
+    """More than 256 tiles of 256x128 whose last round would be partly filled: the plain entry points run the leading
+    column tiles in whole rounds with the plain kernel and the remaining ones over K slices (tile id 200).  Here 4 row
+    tiles x 81 column tiles (the last one ragged): 64 column tiles in one round, 17 over two K slices.  The leading
+    columns carry the bits of the plain tile, the others are another order of the f32 additions; every output form
+    is held to its bar against f64, the workspace form gives the same bits, and a product with no remainder
+    refuses the plan."""
+    lib = capi.load_library()
+    st = torch.cuda.current_stream().cuda_stream
+    m, n, k = 1024, 80 * 128 + 36, 2048
+    n_main = 64 * 128
+    qs, d = synth.q8_0_random(n, k, seed=51)
+    xf, bits = bf16_activations(oracle, m, k, seed=52)
+    w = upload(qs, d)
+    x = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+    truth = truth_for(oracle, qs, d, xf)
+    y32 = torch.full((m, n), float("nan"), device=DEV)
+    capi.check(lib.lhip_q8_0_matmul_bf16_f32out(w.planar.data_ptr(), x.data_ptr(), y32.data_ptr(), m, n, k, st), "f32out")
+    elem, norm = bf16_err(y32.cpu().numpy(), truth)
+    assert elem < TOL_F32 and norm < 1e-5, (elem, norm)
+    auto = run(w, bits)
+    assert bf16_err(auto, truth)[0] < TOL
+    assert np.array_equal(auto, y32.to(torch.bfloat16).float().cpu().numpy())
+    assert np.array_equal(auto, run(w, bits, 200)) and np.array_equal(auto, run(w, bits))
+    ref = run(w, bits, 0)  # the plain tile everywhere
+    assert np.array_equal(auto[:, :n_main], ref[:, :n_main])
+    tail, tail_ref = auto[:, n_main:], ref[:, n_main:]
+    step = np.abs(tail_ref) * 2.0 ** -7 + 1e-4 * float(np.sqrt(np.mean(tail_ref * tail_ref)))
+    assert np.all(np.abs(tail - tail_ref) <= step) and np.mean(tail == tail_ref) > 0.98
+    act = torch.empty(m, n // 2, device=DEV, dtype=torch.bfloat16)
+    want = torch.empty_like(act)
+    capi.check(lib.lhip_q8_0_matmul_bf16_swiglu(w.planar.data_ptr(), x.data_ptr(), act.data_ptr(), m, n, k, st), "swiglu")
+    capi.check(lib.lhip_swiglu_f32_bf16out(y32.data_ptr(), want.data_ptr(), m, n // 2, 1, st), "swiglu of f32")
+    torch.cuda.synchronize()
+    assert torch.equal(act.view(torch.int16), want.view(torch.int16))
+    # the caller's workspace instead of the library's array: two planes of the trailing columns
+    for form, dtype, cols, plain in ((0, torch.bfloat16, n, None), (1, torch.float32, n, y32), (2, torch.bfloat16, n // 2, act)):
+        nbytes = lib.lhip_q8_0_matmul_bf16_workspace_nbytes(m, n, k, form)
+        assert nbytes == 2 * m * (n - n_main) * 4
+        space = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        y_ws = torch.empty((m, cols), dtype=dtype, device=DEV)
+        capi.check(lib.lhip_q8_0_matmul_bf16_ws(w.planar.data_ptr(), x.data_ptr(), y_ws.data_ptr(), m, n, k, form,
+                                                space.data_ptr(), nbytes, st), "ws")
+        torch.cuda.synchronize()
+        if plain is None:
+            assert np.array_equal(y_ws.float().cpu().numpy(), auto)
+        else:
+            assert torch.equal(y_ws.view(torch.uint8), plain.view(torch.uint8)), form
+    # no remainder (64 column tiles are exactly one round), or a K that two slices do not cut into rounds of four tiles
+    yd = torch.empty(m, n_main, device=DEV, dtype=torch.bfloat16)
+    w2 = upload(*synth.q8_0_random(n_main, k, seed=53))
+    assert lib.lhip_q8_0_matmul_bf16_cfg(w2.planar.data_ptr(), x.data_ptr(), yd.data_ptr(), m, n_main, k, 200,
+                                         st) == capi.LHIP_ERR_UNSUPPORTED
+
+
 def test_gemm_argument_errors():
     lib = capi.load_library()
     w = upload(*synth.q8_0_random(64, 96, seed=1))
