@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # drift apart unnoticed.
 TRAFFIC = {
     "gemv": (138310222, "profiles/q8_gemv_decode_projection_set.md"),
-    "gemm": (682674278, "profiles/q8_gemm_prefill_set.md"),
+    "gemm": (757185843, "profiles/q8_gemm_prefill_set.md"),
     "moe_t64": (487359283, "profiles/mxfp4_moe_layer.md"),
 }
 
@@ -52,6 +52,8 @@ def parse():
                     help="decode_projection_set (default, the headline metric), prefill_gemm (the Q8_0 prefill GEMM set), "
                          "moe (the MXFP4 expert layer)")
     ap.add_argument("--layers", type=int, default=None, help="override the 32 layers (debug only; marks the line)")
+    ap.add_argument("--cell", default=None, help="prefill_gemm only: one cell, NAME:M (e.g. gate/up:2048), for a counter "
+                                                  "pass that must tell one call's launches apart; prints that cell only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end Llama-3-8B decode section")
     ap.add_argument("--no-sections", action="store_true", help="skip the prefill-GEMM and MoE sections of the default line")
@@ -318,6 +320,9 @@ def bench_prefill_gemm(args, cpu_seconds=None):
     shapes = {"q/o": (4096, 4096), "k/v": (1024, 4096), "gate/up": (14336, 4096), "down": (4096, 14336),
               "lm_head": (128256, 4096)}
     ms_list = (128, 512, 2048)
+    if getattr(args, "cell", None):
+        cell_name, cell_m = args.cell.rsplit(":", 1)
+        shapes, ms_list = {cell_name: shapes[cell_name]}, (int(cell_m),)
     bufs, xs, ys = {}, {}, {}
     rotate_bytes = 512 << 20  # twice the 256 MB last-level cache: every launch of a rotation streams from HBM
     for nm, (n, k) in shapes.items():
@@ -358,7 +363,11 @@ def bench_prefill_gemm(args, cpu_seconds=None):
             per[f"{nm} M={m}"] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
                                   "frac_mfma_bf16": round(fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                   "gbs": round(by / us / 1e3, 1), "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
-    # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> on the M = 2048 gate/up shape
+    if getattr(args, "cell", None):
+        return {"metric": "Q8_0 prefill GEMM TFLOP/s (MFMA utilisation), 1 GPU", "config": {"cell": args.cell},
+                "per_shape": per}
+    # dominant kernel: q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> on the M = 2048 gate/up shape (time and traffic of
+    # the whole call: the kernel's two launches and the reduction between the K slices of the second)
     n, k, m = 14336, 4096, 2048
     us = _event_us(torch, lambda: [run("gate/up", m, b) for b in bufs["gate/up"]], 5, warm=1, repeats=3) / len(bufs["gate/up"])
     ach = 2.0 * m * n * k / us / 1e6
@@ -374,7 +383,9 @@ def bench_prefill_gemm(args, cpu_seconds=None):
                    "weight_rotation": "every cell is timed over distinct weight buffers of at least 512 MB in all "
                                       f"({', '.join(f'{nm}: {len(b)}' for nm, b in bufs.items())} buffers)"},
         "per_shape": per,
-        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> (gate/up, M=2048)",
+        "roofline": {"bound": "mfma", "kernel": "lhip::q8_gemm_bf16_kernel<256, 128, 4, 2, 4, __bf16> (gate/up, M=2048: the call, "
+                                                   "i.e. this kernel over three whole rounds of column tiles, the same kernel over two K "
+                                                   "slices of the rest, and their sum)",
                      "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": TRAFFIC["gemm"][0],
                      "traffic_source": TRAFFIC["gemm"][1], "avg_launch_us": round(us, 1)},
