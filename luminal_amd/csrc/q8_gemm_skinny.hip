@@ -5,7 +5,8 @@
 // (and, when the strips alone would not fill the chip, a slice of K) and streams it from HBM straight into
 // registers in matrix-core operand order:
 //
-//   * eight compute waves of 16 weight rows each.  The int8 codes go to the matrix cores as they are (an int8 is
+//   * eight compute waves of 16 weight rows each (seven, i.e. strips of 112 rows, where that cuts N into a number
+//     of workgroups that fills the 256 CUs better: sk_plan).  The int8 codes go to the matrix cores as they are (an int8 is
 //     exact in bf16); an MFMA step (v_mfma_f32_16x16x32_bf16) is one Q8_0 block, a lane supplies eight of its
 //     codes, and the block's scale multiplies the f32 block sum: acc += d * sum, the arithmetic of the matvec
 //     kernels (crates/luminal_cuda/src/quantized.rs:93-96).  Eight groups of 64 k per row block are in flight per
@@ -39,7 +40,7 @@ typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
 
 enum { kSkOutBf16 = 0, kSkOutF32 = 1, kSkOutSwiglu = 2, kSkOutPartial = 3, kSkOutF16 = 4 };  // first three as in q8_gemm.hip
 
-constexpr int kSkRows = 128;    // weight rows per workgroup
+constexpr int kSkRows = 128;    // weight rows per workgroup of eight compute waves (seven: 112)
 constexpr int kSkPitch = 160;   // bytes per activation row of a panel in LDS
 constexpr int kSkStages = 3;    // LDS buffers
 constexpr int kSkUnit = 512;     // K slices are whole multiples of this (eight groups of 64 k)
@@ -111,21 +112,23 @@ __device__ __forceinline__ void sk_store4(void *y, float *part, int split, int M
     }
 }
 
-// grid (strips of 128 weight rows, K slices, passes of 16 * MT activation rows); eight compute waves of 16 weight
+// grid (strips of 16 * CW weight rows, K slices, passes of 16 * MT activation rows); CW compute waves of 16 weight
 // rows and four loader waves.  K % 512 == 0, N % 4 == 0.
 // A slice is `slice_groups` groups of 64 k (a multiple of 8); the last may be shorter (also a multiple of 8).
 // RING = groups in flight per wave; a slice is a multiple of RING groups.
 // XT = __bf16, __half or float: the loaders write x as NL = 1, 2 or 3 bf16 planes per tile whose sum is the value
 // exactly (an f16 has 11 significant bits, which two limbs hold; an f32's 24 take three).
-template <int MT, int OUT, int RING, typename XT>
-__global__ __launch_bounds__(12 * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
+// CW = compute waves: 8, or 7 where strips of 112 weight rows cut N into a number of workgroups that fills the chip
+// (14336 rows are 112 strips of 128 but 128 of 112: with two K slices 224 or 256 workgroups for the 256 CUs).
+template <int MT, int OUT, int RING, typename XT, int CW = 8>
+__global__ __launch_bounds__((CW + 4) * 64) void q8_gemm_skinny_kernel(const int8_t *__restrict__ qs, const __half *__restrict__ ds,
                                                              const XT *__restrict__ x, void *__restrict__ y,
                                                              float *__restrict__ part, int M, int N, int K,
                                                              int slice_groups) {
     constexpr int NL = sizeof(XT) == 4 ? 3 : (std::is_same<XT, __bf16>::value ? 1 : 2);  // bf16 limbs of an activation
     using S = SkShape<MT, NL>;
     constexpr int G = S::G;
-    constexpr int CW = 8;  // compute waves
+    static_assert(CW == 8 || CW == 7, "compute waves");
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(12 * 64) void q8_gemm_skinny_kernel(const int8_t *_
 
     // ---------------- compute waves
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = strip * kSkRows + wave * 16;
+    const int n0 = strip * (CW * 16) + wave * 16;
 
     {
         // The codes go to the matrix cores as they are (an int8 is exact in bf16) and the block scale is applied to
@@ -425,8 +428,8 @@ lhip_status q8_gemm_reduce_launch(const float *part, void *y, int m, int n, int 
 
 // K slices for a product: enough workgroups for the 256 CUs, slices of whole 512-k units, partial sums within the
 // scratch array.
-int q8_gemm_skinny_splits(int m, int n, int k, size_t room) {
-    const int strips = (n + kSkRows - 1) / kSkRows, units = k / kSkUnit, passes = (m + 127) / 128;
+static int sk_splits_for(int strips, int m, int n, int k, size_t room) {
+    const int units = k / kSkUnit, passes = (m + 127) / 128;
     int s = 256 / (strips * passes);
     if (s < 1) s = 1;
     if (s > units) s = units;
@@ -434,6 +437,33 @@ int q8_gemm_skinny_splits(int m, int n, int k, size_t room) {
     const int per = (units + s - 1) / s;
     return (units + per - 1) / per;
 }
+
+// Compute waves per workgroup (strips of 16 rows each) for `splits` K slices (0: the slices are chosen with them).
+// A workgroup's time goes with the weights it streams (rows x its share of K) and the launch takes as many rounds of
+// 256 workgroups as it has workgroups: eight waves unless seven make that product smaller.
+struct SkPlan {
+    int cw, splits;
+};
+static SkPlan sk_plan(int m, int n, int k, size_t room, int splits = 0) {
+    const int units = k / kSkUnit, passes = (m + 127) / 128;
+    SkPlan best{8, 1};
+    long best_cost = -1;
+    for (int cw = 8; cw >= 7; --cw) {
+        const int strips = (n + cw * 16 - 1) / (cw * 16);
+        int s = splits > 0 ? (splits > units ? units : splits) : sk_splits_for(strips, m, n, k, room);
+        const int per = (units + s - 1) / s;
+        s = (units + per - 1) / per;  // no empty slice
+        const long rounds = (static_cast<long>(strips) * s * passes + 255) / 256;
+        const long cost = rounds * cw * per;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = SkPlan{cw, s};
+        }
+    }
+    return best;
+}
+
+int q8_gemm_skinny_splits(int m, int n, int k, size_t room) { return sk_plan(m, n, k, room).splits; }
 
 constexpr int kSkMaxRows = 128 * 64;  // passes are the grid's z extent
 
@@ -444,33 +474,41 @@ bool q8_gemm_skinny_supports(int m, int n, int k, int out, const void *y) {
 template <typename XT>
 constexpr int sk_limbs() { return sizeof(XT) == 4 ? 3 : (std::is_same<XT, __bf16>::value ? 1 : 2); }
 
-template <int MT, int OUT, typename XT>
+template <int MT, int OUT, typename XT, int CW = 8>
 static lhip_status sk_launch_t(const int8_t *qs, const __half *ds, const XT *x, void *y, float *part, int m, int n,
                                int k, int splits, int passes, hipStream_t s) {
-    auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, XT>;
+    auto kern = q8_gemm_skinny_kernel<MT, OUT, 8, XT, CW>;
     constexpr size_t lds_bytes = SkShape<MT, sk_limbs<XT>()>::LDS;
     static LdsOptIn opt;  // opting in to more than 64 KiB of dynamic LDS is a per-function attribute
     if (lhip_status st = lds_opt_in(opt, reinterpret_cast<const void *>(kern), lds_bytes)) return st;
     const int units = k / kSkUnit, per = (units + splits - 1) / splits;
     hipLaunchKernelGGL(kern,
-                       dim3(static_cast<unsigned>((n + kSkRows - 1) / kSkRows), static_cast<unsigned>(splits),
+                       dim3(static_cast<unsigned>((n + CW * 16 - 1) / (CW * 16)), static_cast<unsigned>(splits),
                             static_cast<unsigned>(passes)),
-                       dim3(12 * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
+                       dim3((CW + 4) * 64), lds_bytes, s, qs, ds, x, y, part, m, n, k, per * 8);
     LHIP_CHECK_LAUNCH();
     return LHIP_OK;
 }
 
 // bf16 activations: passes of 16 * MT rows (one plane per tile leaves room for 128-row tiles)
-template <int MT>
+template <int MT, int CW>
 static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m,
                                 int n, int k, int splits, hipStream_t s) {
     const int passes = (m + 16 * MT - 1) / (16 * MT);
-    if (splits > 1) return sk_launch_t<MT, kSkOutPartial, __bf16>(qs, ds, x, y, part, m, n, k, splits, passes, s);
+    if (splits > 1) return sk_launch_t<MT, kSkOutPartial, __bf16, CW>(qs, ds, x, y, part, m, n, k, splits, passes, s);
     switch (out) {
-        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
-        case kSkOutF32: return sk_launch_t<MT, kSkOutF32, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
-        default: return sk_launch_t<MT, kSkOutSwiglu, __bf16>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+        case kSkOutBf16: return sk_launch_t<MT, kSkOutBf16, __bf16, CW>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+        case kSkOutF32: return sk_launch_t<MT, kSkOutF32, __bf16, CW>(qs, ds, x, y, part, m, n, k, 1, passes, s);
+        default: return sk_launch_t<MT, kSkOutSwiglu, __bf16, CW>(qs, ds, x, y, part, m, n, k, 1, passes, s);
     }
+}
+template <int CW>
+static lhip_status sk_launch_rows(int out, const int8_t *qs, const __half *ds, const __bf16 *x, void *y, float *part, int m,
+                                  int n, int k, int splits, hipStream_t s) {
+    if (m <= 16) return sk_launch_mt<1, CW>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    if (m <= 32) return sk_launch_mt<2, CW>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    if (m <= 64) return sk_launch_mt<4, CW>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    return sk_launch_mt<8, CW>(out, qs, ds, x, y, part, m, n, k, splits, s);
 }
 
 // `splits` = 0: chosen here.  The caller has checked q8_gemm_skinny_supports.
@@ -478,14 +516,9 @@ static lhip_status sk_launch_mt(int out, const int8_t *qs, const __half *ds, con
 // not touched.
 lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
                                   int out, int splits, hipStream_t s, bool own_workspace, float *ws, size_t ws_floats) {
-    const int units = k / kSkUnit;
     const size_t room = own_workspace ? (ws ? std::min(ws_floats, kSkScratchFloats) : 0) : kSkScratchFloats;
-    if (splits <= 0) splits = q8_gemm_skinny_splits(m, n, k, room);
-    if (splits > units) splits = units;
-    {
-        const int per = (units + splits - 1) / splits;
-        splits = (units + per - 1) / per;  // no empty slice
-    }
+    const SkPlan plan = sk_plan(m, n, k, room, splits);
+    splits = plan.splits;
     float *part = nullptr;
     if (splits > 1) {
         if (static_cast<size_t>(splits) * m * n > room) return LHIP_ERR_UNSUPPORTED;
@@ -493,11 +526,8 @@ lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void
         if (!part) return LHIP_ERR_HIP;
     }
     const __bf16 *x = static_cast<const __bf16 *>(x_bf16);
-    lhip_status st;
-    if (m <= 16) st = sk_launch_mt<1>(out, qs, ds, x, y, part, m, n, k, splits, s);
-    else if (m <= 32) st = sk_launch_mt<2>(out, qs, ds, x, y, part, m, n, k, splits, s);
-    else if (m <= 64) st = sk_launch_mt<4>(out, qs, ds, x, y, part, m, n, k, splits, s);
-    else st = sk_launch_mt<8>(out, qs, ds, x, y, part, m, n, k, splits, s);
+    const lhip_status st = plan.cw == 7 ? sk_launch_rows<7>(out, qs, ds, x, y, part, m, n, k, splits, s)
+                                        : sk_launch_rows<8>(out, qs, ds, x, y, part, m, n, k, splits, s);
     if (st != LHIP_OK || splits == 1) return st;
     return q8_gemm_reduce_launch(part, y, m, n, splits, out, s);
 }
