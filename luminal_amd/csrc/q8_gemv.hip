@@ -512,7 +512,7 @@ static lhip_status dispatch_fused(int r, int sl, int w, int bpc, bool norm, int 
 }
 
 // Default launch shape of the fused kernel for n_total rows (all weights together).
-static void choose_fused(int64_t n_total, int k, int epi, int *r, int *sl, int *w, int *bpc) {
+static void choose_fused(int64_t n_total, int k, int pro, int epi, int *r, int *sl, int *w, int *bpc) {
     const int slices = k % 4096 == 0 ? 4 : (k % 2048 == 0 ? 2 : 1);
     const int fit = (160 * 1024) / (k * 4);
     if (n_total >= 16384 && slices == 4 && fit >= 1) {
@@ -522,7 +522,10 @@ static void choose_fused(int64_t n_total, int k, int epi, int *r, int *sl, int *
     const bool pairs = epi == EPI_SWIGLU;
     *sl = slices >= 2 ? 2 : 1;
     if (fit >= 3) {
-        *r = pairs ? 2 : 1, *w = 4, *bpc = pairs ? 2 : 3;
+        // (measured, q|k|v = 6144 rows at K = 4096: four workgroups per CU 7.25 us against 7.55 with three when nothing
+        // precedes the products; with the norm prologue, which every workgroup pays for, three or two: decode 481 tok/s
+        // against 474 with four; the 4096 rows of o: 6.15 with three, 6.25 with four)
+        *r = pairs ? 2 : 1, *w = 4, *bpc = pairs ? 2 : (pro == PRO_NONE && n_total > 4096 ? 4 : 3);
     } else {
         *r = pairs ? 2 : 1, *w = pairs ? 8 : 16, *bpc = 1;
     }
@@ -776,7 +779,7 @@ lhip_status lhip_q8_0_matvec_fused_f32(const void *const *planar_dev, float *con
     int64_t total = 0;
     for (int i = 0; i < count; ++i) total += n[i] > 0 ? n[i] : 0;
     int r, sl, w, bpc;
-    choose_fused(total, static_cast<int>(k), epilogue, &r, &sl, &w, &bpc);
+    choose_fused(total, static_cast<int>(k), norm_weight_dev ? PRO_NORM : PRO_NONE, epilogue, &r, &sl, &w, &bpc);
     return lhip_q8_0_matvec_fused_f32_cfg(planar_dev, y_dev, n, count, x_dev, k, norm_weight_dev, eps, residual_dev,
                                           epilogue, r, sl, w, bpc, stream);
 }
