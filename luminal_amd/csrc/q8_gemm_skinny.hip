@@ -463,7 +463,15 @@ static SkPlan sk_plan(int m, int n, int k, size_t room, int splits = 0) {
     return best;
 }
 
-int q8_gemm_skinny_splits(int m, int n, int k, size_t room) { return sk_plan(m, n, k, room).splits; }
+// The plan for `room` floats of partial planes: the one the library's own array allows wherever it fits (so that a
+// caller's workspace of the recommended size gets the plain call's plan and bits), else the best within `room`.
+static SkPlan sk_plan_within(int m, int n, int k, size_t room, int splits = 0) {
+    const SkPlan plan = sk_plan(m, n, k, kSkScratchFloats, splits);
+    if (plan.splits == 1 || static_cast<size_t>(plan.splits) * m * n <= room) return plan;
+    return sk_plan(m, n, k, room, splits);
+}
+
+int q8_gemm_skinny_splits(int m, int n, int k, size_t room) { return sk_plan_within(m, n, k, room).splits; }
 
 constexpr int kSkMaxRows = 128 * 64;  // passes are the grid's z extent
 
@@ -517,7 +525,7 @@ static lhip_status sk_launch_rows(int out, const int8_t *qs, const __half *ds, c
 lhip_status q8_gemm_skinny_launch(const int8_t *qs, const __half *ds, const void *x_bf16, void *y, int m, int n, int k,
                                   int out, int splits, hipStream_t s, bool own_workspace, float *ws, size_t ws_floats) {
     const size_t room = own_workspace ? (ws ? std::min(ws_floats, kSkScratchFloats) : 0) : kSkScratchFloats;
-    const SkPlan plan = sk_plan(m, n, k, room, splits);
+    const SkPlan plan = sk_plan_within(m, n, k, room, splits);
     splits = plan.splits;
     float *part = nullptr;
     if (splits > 1) {
