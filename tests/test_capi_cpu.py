@@ -53,6 +53,31 @@ def test_size_laws():
         assert lib.lhip_q8_0_planar_nbytes(n, k) == 0
 
 
+def test_gemm_plans_show_in_the_workspace_size():
+    """lhip_q8_0_matmul_bf16_workspace_nbytes is the f32 planes of the plan the plain entry point takes (host code
+    only): K slices of the whole product, of the column tiles a last partly filled round of 256 workgroups would hold,
+    of the weight-streaming kernel, or none."""
+    lib = capi.load_library()
+    ws = lib.lhip_q8_0_matmul_bf16_workspace_nbytes
+    # 8 x 112 tiles of 256 x 128 = 3.5 rounds: 96 column tiles in whole rounds, 16 (2048 columns) in two K slices
+    assert ws(2048, 14336, 4096, 0) == 2 * 2048 * 2048 * 4
+    assert ws(2048, 14336, 4096, 2) == 2 * 2048 * 2048 * 4
+    # 8 x 1002 tiles: 992 column tiles in 31 whole rounds, the other 10 (1280 columns) in two K slices
+    assert ws(2048, 128256, 4096, 0) == 2 * 2048 * (128256 - 992 * 128) * 4
+    # 4 x 81 tiles with a ragged last one: 64 column tiles in one round, 17 (2084 columns) in two K slices
+    assert ws(1024, 80 * 128 + 36, 2048, 1) == 2 * 1024 * 2084 * 4
+    # exactly one round, or 224 tiles that K slices cannot bring to 256: one launch, no planes
+    assert ws(2048, 4096, 4096, 0) == 0
+    assert ws(512, 14336, 4096, 0) == 0
+    # fewer tiles than CUs and a long K: slices of the whole product (64 tiles x 4 slices)
+    assert ws(512, 4096, 14336, 0) == 4 * 512 * 4096 * 4
+    # at most 128 rows: the weight-streaming kernel, two K slices over strips that fill the chip
+    assert ws(128, 14336, 4096, 0) == 2 * 128 * 14336 * 4
+    assert ws(128, 128256, 4096, 0) == 0
+    # no such product
+    assert ws(128, 14336, 4100, 0) == 0 and ws(0, 14336, 4096, 0) == 0 and ws(128, 14336, 4096, 3) == 0
+
+
 def test_argument_validation_before_any_device_work():
     lib = capi.load_library()
     ok_ptr = 0x1000  # never dereferenced: validation fails first
