@@ -194,7 +194,12 @@ lhip_status lhip_q8_0_matvec_fused_f32_cfg(const void *const *planar_dev, float 
  * allocated, one copy per device) and adds them in a fixed order in a second
  * launch.  Every such call on a device shares that array: calls with m <= 128 that
  * may overlap on one device (different streams, different host threads) race on it
- * and must be ordered by the caller.  Results do not depend on timing. */
+ * and must be ordered by the caller.  Results do not depend on timing.
+ * Above 128 rows the same array holds the planes of the K-sliced plans (few 256x128 tiles and a long K; the column
+ * tiles that more than 256 tiles leave over after whole rounds of 256 workgroups: tile ids 120 + S and 200 of
+ * lhip_q8_0_matmul_bf16_cfg), so the same rule applies to every shape for which
+ * lhip_q8_0_matmul_bf16_workspace_nbytes is not zero; lhip_q8_0_matmul_bf16_ws takes the planes from the caller
+ * instead and may overlap freely. */
 lhip_status lhip_q8_0_matmul_bf16(const void *planar_dev, const void *x_dev, void *y_dev, int64_t m, int64_t n,
                                   int64_t k, void *stream);
 /* Same GEMM with the f32 accumulators stored as they are (y (m, N) f32, 4-byte aligned): what a caller
