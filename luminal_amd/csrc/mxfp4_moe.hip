@@ -286,7 +286,8 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
     }
     BSet<MT, NT> bs[D];
     auto load_b = [&](int set, int c) __attribute__((always_inline)) {
-        // Dead chunks (past the padded K) re-read the last chunk; compute() zeroes them.
+        // Dead chunks (past the padded K; the refills of the last round) are zeroed by compute(); their requests go to one
+        // line for the whole wave (aimed at the last chunk, a short tile would pull that kilobyte through memory again).
         // (Masking here, next to the loads, would make the wave wait for data it has only just requested.)
         bs[set].valid = c < chunks;
         const int cc = min(c, chunks - 1);
@@ -295,8 +296,9 @@ void mx_moe_gemm_kernel(MoeGemmArgs g) {
             // Short tiles (few routed rows per expert) read every weight once: keep them out of the caches.
             // Tall tiles come several per expert, and the later ones find the weights in L2 / the last-level cache.
             if (MT <= 2) {
-                bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
-                bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+                const uint8_t *wq = c < chunks ? w_tile[f] + static_cast<size_t>(cc) * 1024 : g.w_nib;
+                bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(wq));
+                bs[set].s[f] = s_tile[f][cc * 64];  // (cached: the 64 scale bytes of two consecutive chunks share a line)
             } else {
                 bs[set].q[f] = *reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024);
                 bs[set].s[f] = s_tile[f][cc * 64];

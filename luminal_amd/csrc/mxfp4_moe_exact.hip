@@ -175,13 +175,16 @@ __global__ __launch_bounds__(256 * WR) void mx_moe_gemm_exact_kernel(MoeExactArg
     }
     BSet<MT, NT> bs[D];
     auto load_b = [&](int set, int c) __attribute__((always_inline)) {
-        bs[set].valid = c < chunks;  // dead chunks (past the padded K) re-read the last one and are not multiplied
+        bs[set].valid = c < chunks;  // dead chunks (past the padded K; the refills of the last round) are not multiplied
         const int cc = min(c, chunks - 1);
 #pragma unroll
         for (int f = 0; f < NT; ++f) {
             if (MT <= 2) {  // short tiles read every weight once: keep them out of the caches
-                bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024));
-                bs[set].s[f] = __builtin_nontemporal_load(s_tile[f] + cc * 64);
+                // (a dead chunk's request goes to one line for the whole wave: aimed at the last chunk it would pull
+                // that kilobyte through the memory system again, D + 1 times per wave and fragment)
+                const uint8_t *wq = c < chunks ? w_tile[f] + static_cast<size_t>(cc) * 1024 : g.w_nib;
+                bs[set].q[f] = __builtin_nontemporal_load(reinterpret_cast<const mu32x4 *>(wq));
+                bs[set].s[f] = s_tile[f][cc * 64];  // (cached: the 64 scale bytes of two consecutive chunks share a line)
             } else {
                 bs[set].q[f] = *reinterpret_cast<const mu32x4 *>(w_tile[f] + static_cast<size_t>(cc) * 1024);
                 bs[set].s[f] = s_tile[f][cc * 64];
