@@ -153,7 +153,7 @@ __global__ __launch_bounds__(WM *WN * 64) void q8_gemm_bf16_kernel(const int8_t 
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
             if (i * P / B_CHUNKS != p) continue;
-            b_reg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const gu32x4 *>(b_src[i] + k0));
+            b_reg[set][i] = *reinterpret_cast<const gu32x4 *>(b_src[i] + k0);
             d_reg[set][i] = d_src[i][k0 >> 6];
         }
     };
